@@ -1,0 +1,233 @@
+// C ABI of libfa_mi355x.so: argument checks, mask normalisation, split planning and kernel
+// dispatch.  Host-side counterpart of the reference's mha_fwd / mha_varlen_fwd / mha_fwd_kvcache
+// bodies after tensor unpacking (csrc/flash_attn/flash_api.cpp:248-424, 426-585, 1038-1279) and of
+// run_mha_fwd's dtype x head-dim dispatch (:194-204).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+#include <algorithm>
+#include "fa_prefill.h"
+#include "fa_launch.h"
+
+namespace fa {
+
+static thread_local std::string g_err;
+static int fail(const char* msg) { g_err = msg; return 1; }
+static int fail_hip(int e, const char* where) {
+    g_err = std::string(where) + ": " + hipGetErrorString((hipError_t)e);
+    return 2;
+}
+
+int prefill_block_n(int db) { return db == 64 ? PrefillTile<64>::BN : db == 128 ? PrefillTile<128>::BN : PrefillTile<256>::BN; }
+int prefill_block_m(int db) { return 128 * (db == 64 ? PrefillTile<64>::RB : db == 128 ? PrefillTile<128>::RB : PrefillTile<256>::RB); }
+static int bucket(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
+
+static const int kNumCU = 256;   // MI355X
+
+// The small-q streaming kernel packs seqlen_q x (h / h_k) rows into 16 MFMA columns.
+static bool use_decode_kernel(const fa_fwd_params& p) {
+    return p.cu_seqlens_q == nullptr && (int64_t)p.seqlen_q * (p.h / p.h_k) <= 16;
+}
+
+static int check_common(const fa_fwd_params* p) {
+    if (!p) return fail("params is NULL");
+    if (!p->q || !p->k || !p->v || !p->o || !p->softmax_lse) return fail("q, k, v, o and softmax_lse must be set");
+    if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return fail("FlashAttention only support fp16 and bf16 data type");
+    if (p->b <= 0) return fail("batch size must be positive");
+    if (p->d <= 0 || p->d > 256) return fail("FlashAttention forward only supports head dimension at most 256");
+    if (p->d % 8 != 0) return fail("head dimension must be a multiple of 8 at the C boundary (pad on the host)");
+    if (p->h <= 0 || p->h_k <= 0 || p->h % p->h_k != 0) return fail("Number of heads in key/value must divide number of heads in query");
+    if (p->seqlen_q < 0 || p->seqlen_k < 0) return fail("sequence lengths must be non-negative");
+    if (p->num_splits < 0 || p->num_splits > FA_MAX_SPLITS) return fail("num_splits > 128 not supported");
+    return 0;
+}
+
+// Split planning for 256 CUs.  Returns the chunk count; *split_len receives the chunk length.
+static int plan(const fa_fwd_params& p, bool allow_split, int* split_len_out) {
+    const int sk = p.seqlen_k;
+    const int db = bucket(p.d);
+    const bool dec = use_decode_kernel(p);
+    const int gran = dec ? 128 : prefill_block_n(db);
+    auto rup = [](int64_t x, int64_t m) { return (int)((x + m - 1) / m * m); };
+    int splits = 1;
+    if (allow_split && sk > 0) {
+        if (p.num_splits > 1) {
+            splits = p.num_splits;
+        } else if (p.num_splits == 0) {
+            if (dec) {
+                // ~16k chunk slots over the whole launch, chunks of at least 256 keys: enough
+                // workgroups to balance ragged cache lengths over 256 CUs x 2 resident groups.
+                const int64_t streams = (int64_t)p.b * p.h_k;
+                int64_t len = rup(std::max<int64_t>(256, (int64_t)sk * streams / 16384), 128);
+                splits = (int)((sk + len - 1) / len);
+            } else {
+                const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;
+                if (wgs < kNumCU) {
+                    const int64_t want = (2 * kNumCU + wgs - 1) / wgs;
+                    splits = (int)std::min<int64_t>(want, (sk + 255) / 256);
+                }
+            }
+        }
+        splits = std::max(1, std::min(splits, FA_MAX_SPLITS));
+        // never more chunks than tiles
+        splits = std::min(splits, (sk + gran - 1) / gran);
+        splits = std::max(1, splits);
+    }
+    int len = rup((sk + splits - 1) / std::max(1, splits), gran);
+    if (len <= 0) len = gran;
+    // drop chunks that the rounding made empty
+    splits = std::max(1, (sk + len - 1) / len);
+    if (split_len_out) *split_len_out = len;
+    return splits;
+}
+
+static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
+    kp.p = p;
+    fa_fwd_params& q = kp.p;
+    // mask normalisation (flash_api.cpp:111-114, 296-297)
+    if (q.is_causal) q.window_right = 0;
+    kp.has_left = q.window_left >= 0;
+    kp.has_right = q.window_right >= 0;
+    kp.scale_log2 = q.softmax_scale * (float)M_LOG2E;
+    kp.d_rounded = (q.d + 31) / 32 * 32;
+    kp.num_splits = 1;
+    kp.split_len = 0;
+    kp.num_m_blocks = 0;
+    kp.rotary_q = 0;
+}
+
+static int run_attention(KParams& kp, hipStream_t stream) {
+    const fa_fwd_params& p = kp.p;
+    int e;
+    if (use_decode_kernel(p)) {
+        e = launch_decode(kp, stream);
+        if (e) return fail_hip(e, "decode kernel launch");
+    } else {
+        const bool bf = p.dtype == FA_DTYPE_BF16;
+        switch (bucket(p.d)) {
+            case 64: e = bf ? launch_prefill_bf16_64(kp, stream) : launch_prefill_fp16_64(kp, stream); break;
+            case 128: e = bf ? launch_prefill_bf16_128(kp, stream) : launch_prefill_fp16_128(kp, stream); break;
+            default: e = bf ? launch_prefill_bf16_256(kp, stream) : launch_prefill_fp16_256(kp, stream); break;
+        }
+        if (e) return fail_hip(e, "prefill kernel launch");
+    }
+    if (kp.num_splits > 1) {
+        e = launch_combine(kp, stream);
+        if (e) return fail_hip(e, "combine kernel launch");
+    }
+    return 0;
+}
+
+static int resolve_splits(KParams& kp, const fa_fwd_params& p, bool allow_split) {
+    int len = 0;
+    const int s = plan(p, allow_split, &len);
+    kp.num_splits = s;
+    kp.split_len = len;
+    if (s > 1 && (!p.o_accum || !p.lse_accum)) return fail("o_accum and lse_accum are required when the key range is split (see fa_plan_splits)");
+    return 0;
+}
+
+}  // namespace fa
+
+using namespace fa;
+
+extern "C" {
+
+const char* fa_last_error(void) { return g_err.c_str(); }
+int32_t fa_version(void) { return (0 << 16) | 1; }
+int32_t fa_sizeof_params(void) { return (int32_t)sizeof(fa_fwd_params); }
+
+int fa_num_splits_heuristic_reference(int32_t batch_nheads_mblocks, int32_t num_sms, int32_t num_n_blocks, int32_t max_splits) {
+    if (batch_nheads_mblocks >= 0.8f * num_sms) return 1;
+    max_splits = std::min({max_splits, num_sms, num_n_blocks});
+    auto cdiv = [](int a, int b) { return (a + b - 1) / b; };
+    auto eligible = [&](int s) { return s == 1 || cdiv(num_n_blocks, s) != cdiv(num_n_blocks, s - 1); };
+    std::vector<float> eff(std::max(max_splits, 0) + 1, 0.f);
+    float best = 0.f;
+    for (int s = 1; s <= max_splits; s++) {
+        if (!eligible(s)) continue;
+        const float waves = float(batch_nheads_mblocks * s) / num_sms;
+        eff[s] = waves / std::ceil(waves);
+        best = std::max(best, eff[s]);
+    }
+    for (int s = 1; s <= max_splits; s++)
+        if (eligible(s) && eff[s] >= 0.85f * best) return s;
+    return 1;
+}
+
+int fa_plan_splits(const fa_fwd_params* p, int32_t api, int32_t* num_splits) {
+    g_err.clear();
+    if (int r = check_common(p)) return r;
+    if (!num_splits) return fail("num_splits is NULL");
+    if (api != 0 && api != 2) return fail("api must be 0 (fa_fwd) or 2 (fa_fwd_kvcache)");
+    *num_splits = plan(*p, true, nullptr);
+    return 0;
+}
+
+int fa_fwd(const fa_fwd_params* p, void* hip_stream) {
+    g_err.clear();
+    if (int r = check_common(p)) return r;
+    if (p->cu_seqlens_q || p->cu_seqlens_k) return fail("fa_fwd takes dense batches; use fa_varlen_fwd or fa_fwd_kvcache");
+    if (p->k_new || p->v_new || p->rotary_cos || p->cache_batch_idx) return fail("fa_fwd does not append or rotate; use fa_fwd_kvcache");
+    if (p->seqlen_q == 0) return 0;
+    KParams kp;
+    fill_kparams(kp, *p);
+    kp.p.seqlen_knew = 0;
+    kp.p.rotary_dim = 0;
+    if (int r = resolve_splits(kp, kp.p, true)) return r;
+    return run_attention(kp, (hipStream_t)hip_stream);
+}
+
+int fa_varlen_fwd(const fa_fwd_params* p, void* hip_stream) {
+    g_err.clear();
+    if (int r = check_common(p)) return r;
+    if (!p->cu_seqlens_q || !p->cu_seqlens_k) return fail("cu_seqlens_q and cu_seqlens_k are required");
+    if (!p->is_seqlens_k_cumulative) return fail("cu_seqlens_k must be cumulative for fa_varlen_fwd");
+    if (p->k_new || p->v_new || p->rotary_cos || p->cache_batch_idx) return fail("fa_varlen_fwd does not append or rotate");
+    if (p->seqlen_q == 0) return 0;
+    KParams kp;
+    fill_kparams(kp, *p);
+    kp.p.seqlen_knew = 0;
+    kp.p.rotary_dim = 0;
+    kp.p.num_splits = 1;
+    if (int r = resolve_splits(kp, kp.p, false)) return r;
+    return run_attention(kp, (hipStream_t)hip_stream);
+}
+
+int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
+    g_err.clear();
+    if (int r = check_common(p)) return r;
+    if (p->cu_seqlens_q) return fail("fa_fwd_kvcache takes a dense q batch");
+    if (p->cu_seqlens_k && p->is_seqlens_k_cumulative) return fail("cache_seqlens must be per-batch lengths, not prefix sums");
+    const bool has_new = p->k_new != nullptr;
+    if (has_new) {
+        if (!p->v_new) return fail("If key is supplied, value must also be passed in");
+        if (!p->cu_seqlens_k) return fail("If key is supplied, seqlens_k must also be passed in");
+        if (p->seqlen_knew <= 0) return fail("seqlen_knew must be positive when k_new is given");
+        if (p->seqlen_q > p->seqlen_k) return fail("If key is supplied, it must have seqlen <= the seqlen of the KV cache");
+    } else if (p->v_new) {
+        return fail("If value is supplied, key must also be passed in");
+    }
+    if (p->rotary_cos || p->rotary_sin) {
+        if (!has_new) return fail("If rotary cos/sin are provided, new key / value to be appended to KV cache must also be provided");
+        if (!p->rotary_cos || !p->rotary_sin) return fail("If rotary cos is provided, rotary sin must also be provided");
+        if (p->rotary_dim <= 0 || p->rotary_dim > p->d) return fail("rotary_dim must be <= headdim");
+        if (p->rotary_dim % 16 != 0) return fail("Only rotary dimensions divisible by 16 are currently supported");
+    }
+    if (p->seqlen_q == 0) return 0;
+    KParams kp;
+    fill_kparams(kp, *p);
+    if (!has_new) kp.p.seqlen_knew = 0;
+    if (!p->rotary_cos) kp.p.rotary_dim = 0;
+    kp.rotary_q = kp.p.rotary_dim > 0;
+    if (int r = resolve_splits(kp, kp.p, true)) return r;
+    hipStream_t stream = (hipStream_t)hip_stream;
+    if (has_new) {
+        if (int e = launch_append_kv(kp, stream)) return fail_hip(e, "append_kv kernel launch");
+    }
+    return run_attention(kp, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,116 @@
+// Small memory-bound kernels around the attention kernels:
+//  * combine: log-sum-exp weighted merge of split-KV partials
+//    (reference: combine_attn_seqk_parallel, csrc/flash_attn/src/flash_fwd_kernel.h:1169-1327);
+//  * append_kv: copy of k_new / v_new (new keys rotated) into the cache rows
+//    [cache_seqlens[b], cache_seqlens[b] + seqlen_knew) of cache row cache_batch_idx[b]
+//    (reference: the Append_KV prologue, flash_fwd_kernel.h:763-852, copy_w_min_idx /
+//    copy_rotary_* in csrc/flash_attn/src/utils.h:358-517).
+#include "fa_common.h"
+#include "fa_launch.h"
+
+namespace fa {
+
+// One wave per output row (b, h, i).  Lanes first reduce the per-split log-sum-exp values, then
+// stream the partial rows whose weight is non-zero.
+template <typename T>
+__global__ void __launch_bounds__(256) combine_kernel(const KParams kp) {
+    const fa_fwd_params& p = kp.p;
+    const int lane = threadIdx.x & 63;
+    const int64_t nrows = (int64_t)p.b * p.h * p.seqlen_q;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= nrows) return;
+    const int S = kp.num_splits;
+
+    float l0 = lane < S ? p.lse_accum[(int64_t)lane * nrows + row] : -INFINITY;
+    float l1 = lane + 64 < S ? p.lse_accum[(int64_t)(lane + 64) * nrows + row] : -INFINITY;
+    float mx = fmaxf(l0, l1);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    const float mref = (mx == -INFINITY) ? 0.f : mx;
+    float sum = __expf(l0 - mref) + __expf(l1 - mref);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+    const bool dead = (sum == 0.f) || (sum != sum);
+    const float lse = dead ? INFINITY : __logf(sum) + mref;
+    const float w0 = dead ? 0.f : __expf(l0 - lse);
+    const float w1 = dead ? 0.f : __expf(l1 - lse);
+
+    const int i = (int)(row % p.seqlen_q);
+    const int h = (int)((row / p.seqlen_q) % p.h);
+    const int b = (int)(row / ((int64_t)p.seqlen_q * p.h));
+    if (lane == 0) p.softmax_lse[row] = lse;
+
+    // each lane owns 4 consecutive output dims per pass (64 lanes x 4 = 256 dims max)
+    const int d0 = lane * 4;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < S; s++) {
+        const float w = __shfl(s < 64 ? w0 : w1, s & 63);
+        if (w == 0.f) continue;   // wave-uniform
+        if (d0 < kp.d_rounded) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(p.o_accum + ((int64_t)s * nrows + row) * kp.d_rounded + d0);
+            acc += v * w;
+        }
+    }
+    if (d0 < p.d) {
+        int64_t off = (int64_t)i * p.o_row_stride + (int64_t)h * p.o_head_stride + (int64_t)b * p.o_batch_stride;
+        u32x2 v = {pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
+        st_global8(reinterpret_cast<T*>(p.o) + off + d0, v);
+    }
+}
+
+int launch_combine(const KParams& kp, hipStream_t stream) {
+    const int64_t nrows = (int64_t)kp.p.b * kp.p.h * kp.p.seqlen_q;
+    if (nrows == 0) return 0;
+    dim3 grid((unsigned)((nrows + 3) / 4)), block(256);
+    if (kp.p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(combine_kernel<__bf16>, grid, block, 0, stream, kp);
+    else hipLaunchKernelGGL(combine_kernel<_Float16>, grid, block, 0, stream, kp);
+    return (int)hipGetLastError();
+}
+
+// One thread per 16-byte chunk of one new (token, kv-head) row.
+template <typename T>
+__global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp) {
+    const fa_fwd_params& p = kp.p;
+    const int cpr = p.d / 8;
+    const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * cpr;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int c = (int)(idx % cpr);
+    const int hk = (int)((idx / cpr) % p.h_k);
+    const int t = (int)((idx / ((int64_t)cpr * p.h_k)) % p.seqlen_knew);
+    const int b = (int)(idx / ((int64_t)cpr * p.h_k * p.seqlen_knew));
+    const int len = p.cu_seqlens_k ? p.cu_seqlens_k[b] : p.seqlen_k;
+    const int pos = len + t;
+    if (pos >= p.seqlen_k) return;     // never write past the cache capacity
+    const int bk = p.cache_batch_idx ? p.cache_batch_idx[b] : b;
+    const int d0 = c * 8;
+
+    const T* vsrc = reinterpret_cast<const T*>(p.v_new) + (int64_t)b * p.vnew_batch_stride + (int64_t)t * p.vnew_row_stride + (int64_t)hk * p.vnew_head_stride;
+    T* vdst = reinterpret_cast<T*>(const_cast<void*>(p.v)) + (int64_t)bk * p.v_batch_stride + (int64_t)pos * p.v_row_stride + (int64_t)hk * p.v_head_stride;
+    st_global16(vdst + d0, ld_global16(vsrc + d0));
+
+    const T* ksrc = reinterpret_cast<const T*>(p.k_new) + (int64_t)b * p.knew_batch_stride + (int64_t)t * p.knew_row_stride + (int64_t)hk * p.knew_head_stride;
+    T* kdst = reinterpret_cast<T*>(const_cast<void*>(p.k)) + (int64_t)bk * p.k_batch_stride + (int64_t)pos * p.k_row_stride + (int64_t)hk * p.k_head_stride;
+    u32x4 raw = ld_global16(ksrc + d0);
+    if (p.rotary_dim > 0 && d0 < p.rotary_dim) {
+        const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
+        const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
+        float x[8];
+        unpack8<T>(raw, x);
+        rotary8<T>(x, ksrc, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
+        raw = pack8<T>(x);
+    }
+    st_global16(kdst + d0, raw);
+}
+
+int launch_append_kv(const KParams& kp, hipStream_t stream) {
+    const fa_fwd_params& p = kp.p;
+    const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * (p.d / 8);
+    if (total == 0) return 0;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(append_kv_kernel<__bf16>, grid, block, 0, stream, kp);
+    else hipLaunchKernelGGL(append_kv_kernel<_Float16>, grid, block, 0, stream, kp);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fa

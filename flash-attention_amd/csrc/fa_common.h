@@ -1,0 +1,183 @@
+// Shared device helpers for the gfx950 FlashAttention forward kernels.
+//
+// Everything here is written for CDNA4 wave64: MFMA 32x32x16 / 16x16x32 on 16-bit inputs,
+// transposing LDS reads (ds_read_b64_tr_b16), and the cross-half lane swap (v_permlane32_swap).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "fa_mi355x.h"
+
+namespace fa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define FA_DEV __device__ __forceinline__
+#define FA_LDS_PTR(T) __attribute__((address_space(3))) T*
+
+// Kernel-side view of one problem: the caller's description plus values the host derives once.
+struct KParams {
+    fa_fwd_params p;
+    float scale_log2;      // softmax_scale * log2(e)
+    int32_t num_splits;    // resolved split count (>= 1)
+    int32_t split_len;     // keys per split chunk (multiple of the key tile), when num_splits > 1
+    int32_t d_rounded;     // d rounded up to 32: row pitch of o_accum
+    int32_t num_m_blocks;  // query tiles per (batch, head)
+    int32_t has_left, has_right;  // window bounds active (after causal normalisation)
+    int32_t rotary_q;      // rotate q on load
+};
+
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+    typedef bf16x8 v8; typedef bf16x4 v4; typedef bf16x2 v2;
+    static FA_DEV f32x16 mfma32(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static FA_DEV f32x4 mfma16(v8 a, v8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Elem<_Float16> {
+    typedef f16x8 v8; typedef f16x4 v4; typedef f16x2 v2;
+    static FA_DEV f32x16 mfma32(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static FA_DEV f32x4 mfma16(v8 a, v8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+
+// round-to-nearest-even pack of two floats into one 32-bit register of T
+template <typename T> FA_DEV uint32_t pack2(float a, float b) {
+    typedef typename Elem<T>::v2 v2;
+    f32x2 f = {a, b};
+    v2 h = __builtin_convertvector(f, v2);
+    return __builtin_bit_cast(uint32_t, h);
+}
+template <typename T> FA_DEV float to_float(T x) { return (float)x; }
+
+template <typename T> FA_DEV void unpack8(const u32x4& raw, float* out) {
+    typedef typename Elem<T>::v8 v8;
+    v8 h = __builtin_bit_cast(v8, raw);
+#pragma unroll
+    for (int e = 0; e < 8; e++) out[e] = (float)h[e];
+}
+template <typename T> FA_DEV u32x4 pack8(const float* in) {
+    u32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; e++) r[e] = pack2<T>(in[2 * e], in[2 * e + 1]);
+    return r;
+}
+
+FA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// max / sum over the two 32-lane halves of the wave (lane l <-> lane l^32)
+FA_DEV float xhalf_max(float x) {
+    uint32_t u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+FA_DEV float xhalf_sum(float x) {
+    uint32_t u = __float_as_uint(x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+FA_DEV u32x4 ld_global16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+FA_DEV void st_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+FA_DEV void st_global8(void* p, u32x2 v) { *reinterpret_cast<u32x2*>(p) = v; }
+
+// LDS transposing read: within each block of 16 lanes, lane 4*j+q supplies the address of four
+// consecutive 16-bit elements (row j, columns 4q..4q+3 of a 4 x 16 tile); lane i of the block
+// receives column i of rows 0..3.
+FA_DEV u32x2 lds_read_tr16(const char* p) {
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS_PTR(s16x4))(p));
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// 16-byte-chunk XOR swizzles of a row-major [rows][D] 16-bit tile in LDS.
+// K tiles are read one 16 B chunk per lane by 16 consecutive rows at the same chunk index;
+// V tiles are read by the transposing load as 4 consecutive rows x 4 consecutive chunks.
+template <int D> FA_DEV int swz_k(int chunk, int row) {
+    if constexpr (D >= 128) return chunk ^ (row & 15);
+    else if constexpr (D == 64) return chunk ^ ((row >> 1) & 7);
+    else return chunk ^ ((row >> 2) & 3);   // D == 32
+}
+template <int D> FA_DEV int swz_v(int chunk, int row) {
+    if constexpr (D >= 128) return chunk ^ ((row & 3) << 2);
+    else if constexpr (D == 64) return chunk ^ (((row >> 1) & 1) << 2);
+    else return chunk;                       // D == 32: four rows fill the 256 B bank window
+}
+
+// Rotary embedding of 8 consecutive elements [d0, d0+8) of one row, fp32 math.
+// `x` are the row's own values, `row_ptr` points at the row start (to fetch the partner half for
+// the non-interleaved form), cos/sin point at the table row for this token.
+template <typename T>
+FA_DEV void rotary8(float* x, const T* row_ptr, const T* cos_row, const T* sin_row, int d0,
+                    int rotary_dim, bool interleaved) {
+    if (d0 >= rotary_dim) return;
+    if (interleaved) {
+        float c[4], s[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) { c[e] = (float)cos_row[d0 / 2 + e]; s[e] = (float)sin_row[d0 / 2 + e]; }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float x0 = x[2 * e], x1 = x[2 * e + 1];
+            x[2 * e] = x0 * c[e] - x1 * s[e];
+            x[2 * e + 1] = x0 * s[e] + x1 * c[e];
+        }
+    } else {
+        const int half = rotary_dim / 2;
+        const bool left = d0 < half;
+        const int t0 = left ? d0 : d0 - half;           // table column
+        const int partner = left ? d0 + half : d0 - half;
+        u32x4 praw = ld_global16(row_ptr + partner);
+        float y[8];
+        unpack8<T>(praw, y);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float c = (float)cos_row[t0 + e], s = (float)sin_row[t0 + e];
+            x[e] = left ? (x[e] * c - y[e] * s) : (x[e] * c + y[e] * s);
+        }
+    }
+}
+
+// Resolved per-(batch) sequence bookkeeping.  Mirrors the reference's BlockInfo
+// (csrc/flash_attn/src/block_info.h:11-42) with 64-bit offsets.
+struct SeqInfo {
+    int sq, sk, sk_cache;      // rows of q, visible keys, keys in the cache before the append
+    int64_t q_off, k_off, v_off, o_off;   // element offsets of (row 0, head 0) of this batch entry
+    int q_row0;                // first packed row (varlen) for lse indexing: unused for dense
+};
+FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
+    SeqInfo s;
+    if (p.cu_seqlens_q) {
+        int r0 = p.cu_seqlens_q[b];
+        s.sq = p.cu_seqlens_q[b + 1] - r0;
+        s.q_off = (int64_t)r0 * p.q_row_stride;
+        s.o_off = (int64_t)r0 * p.o_row_stride;
+    } else {
+        s.sq = p.seqlen_q;
+        s.q_off = (int64_t)b * p.q_batch_stride;
+        s.o_off = (int64_t)b * p.o_batch_stride;
+    }
+    if (p.cu_seqlens_k && p.is_seqlens_k_cumulative) {
+        int r0 = p.cu_seqlens_k[b];
+        s.sk_cache = p.cu_seqlens_k[b + 1] - r0;
+        s.sk = s.sk_cache;
+        s.k_off = (int64_t)r0 * p.k_row_stride;
+        s.v_off = (int64_t)r0 * p.v_row_stride;
+    } else {
+        const int bk = p.cache_batch_idx ? p.cache_batch_idx[b] : b;
+        s.sk_cache = p.cu_seqlens_k ? p.cu_seqlens_k[b] : p.seqlen_k;
+        s.sk = s.sk_cache + p.seqlen_knew;
+        s.k_off = (int64_t)bk * p.k_batch_stride;
+        s.v_off = (int64_t)bk * p.v_batch_stride;
+    }
+    s.q_row0 = 0;
+    return s;
+}
+
+}  // namespace fa

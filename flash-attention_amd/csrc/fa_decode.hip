@@ -1,0 +1,321 @@
+// Split-KV decode kernel for gfx950: few query rows against a long K/V stream (HBM-bound).
+// Counterpart of the reference's compute_attn_1rowblock_splitkv used for seqlen_q == 1 after its
+// "seqlen_q <-> ngroups" swap (csrc/flash_attn/flash_api.cpp:1096-1104,
+// csrc/flash_attn/src/flash_fwd_kernel.h:584-1130), designed as a streaming kernel:
+//
+//  * One workgroup = one (batch, kv-head, key-chunk).  All query rows that share the kv head --
+//    seqlen_q positions x (h / h_k) grouped heads, at most 16 -- are packed into the 16 columns of
+//    v_mfma_f32_16x16x32, so every K/V byte is fetched once per group.
+//  * The four waves of the workgroup stream disjoint quarters of the chunk on their own: 128-bit
+//    row-contiguous global loads (a 16-lane group reads one whole K or V row), issued one 32-key
+//    step ahead into registers, staged through a wave-private swizzled LDS tile to reach the MFMA
+//    operand layouts (ds_read_b128 for K, transposing ds_read_b64_tr_b16 for V).  No workgroup
+//    barrier in the loop.
+//  * The four running (max, sum, O) states are merged through LDS at the end and written either as
+//    the final output or as one fp32 partial + log-sum-exp per chunk for the combine kernel.
+#include "fa_common.h"
+#include "fa_launch.h"
+
+namespace fa {
+
+template <int D> FA_DEV int swz_vd(int chunk, int row) {
+    if constexpr (D >= 128) return chunk ^ ((row & 7) << 1);
+    else return chunk ^ (((row >> 1) & 3) << 1);   // D == 64
+}
+
+template <typename T, int D>
+struct DecodeCfg {
+    static constexpr int kThreads = 256, kWaves = 4;
+    static constexpr int STEP = 32;                 // keys per wave step
+    static constexpr int CPR = D / 8;
+    static constexpr int ROWB = D * 2;
+    static constexpr int TILE_BYTES = STEP * ROWB;  // one of K / V for one wave
+    static constexpr int LD = STEP * CPR / 64;      // 16 B loads per lane per tensor per step
+    static constexpr int KC = D / 32;               // k-steps of S^T
+    static constexpr int DB = D / 16;               // 16-row blocks of O^T
+    static constexpr int STAGE_BYTES = kWaves * 2 * TILE_BYTES;
+    static constexpr int MERGE_BYTES = kWaves * 16 * (D + 2) * 4;
+    static constexpr int SMEM = STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES;
+};
+
+template <typename T, int D, bool SPLIT>
+__global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KParams kp) {
+    typedef DecodeCfg<T, D> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_fwd_params& p = kp.p;
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int m = lane & 15, g4 = lane >> 4;     // MFMA column (packed query row), lane group
+    const int split = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int G = p.h / p.h_k;
+    const int rows = p.seqlen_q * G;             // packed rows in use (<= 16)
+
+    const SeqInfo si = seq_info(p, b);
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+
+    int hi = si.sk, lo = 0;
+    if (has_right) hi = min(hi, si.sq + shift + wr);
+    if (has_left) lo = max(0, shift - wl);
+    if (SPLIT) {
+        lo = max(lo, split * kp.split_len);
+        hi = min(hi, (split + 1) * kp.split_len);
+    }
+
+    // packed row m -> query position and head
+    const int qi = m / G, qg = m % G;
+    const int head = hk * G + qg;
+    const bool row_valid = m < rows;
+
+    if (hi <= lo) {   // nothing visible in this chunk
+        if (tid < rows) {
+            const int i = tid / G, hd = hk * G + tid % G;
+            if (SPLIT) {
+                p.lse_accum[(((int64_t)split * p.b + b) * p.h + hd) * p.seqlen_q + i] = -INFINITY;
+            } else {
+                p.softmax_lse[((int64_t)b * p.h + hd) * p.seqlen_q + i] = INFINITY;
+                T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)i * p.o_row_stride + (int64_t)hd * p.o_head_stride;
+                for (int d0 = 0; d0 < p.d; d0 += 8) { u32x4 z = {0, 0, 0, 0}; st_global16(orow + d0, z); }
+            }
+        }
+        return;
+    }
+
+    // ---- Q fragments (B operand): lane (m, g4) holds Q[row m][32c + 8*g4 .. +7]
+    v8 qf[C::KC];
+    {
+        const T* qrow = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)qi * p.q_row_stride + (int64_t)head * p.q_head_stride;
+#pragma unroll
+        for (int c = 0; c < C::KC; c++) {
+            const int d0 = c * 32 + 8 * g4;
+            u32x4 raw = {0, 0, 0, 0};
+            if (row_valid && d0 < p.d) {
+                raw = ld_global16(qrow + d0);
+                if (kp.rotary_q && d0 < p.rotary_dim) {
+                    const int pos = si.sk_cache + ((p.is_causal || has_left || has_right) ? qi : 0);
+                    const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
+                    const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
+                    float x[8];
+                    unpack8<T>(raw, x);
+                    rotary8<T>(x, qrow, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
+                    raw = pack8<T>(x);
+                }
+            }
+            qf[c] = __builtin_bit_cast(v8, raw);
+        }
+    }
+
+    // ---- this wave's key range
+    const int span = hi - lo;
+    const int per_wave = ((span + C::kWaves - 1) / C::kWaves + C::STEP - 1) / C::STEP * C::STEP;
+    const int w_lo = lo + wave * per_wave;
+    const int w_hi = min(hi, w_lo + per_wave);
+
+    const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
+    const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
+    char* kb = smem + wave * 2 * C::TILE_BYTES;
+    char* vb = kb + C::TILE_BYTES;
+
+    u32x4 kr[C::LD], vr[C::LD];
+    auto load_step = [&](int n0) {
+#pragma unroll
+        for (int i = 0; i < C::LD; i++) {
+            const int f = lane + i * 64;
+            const int row = f / C::CPR, c = f % C::CPR;
+            const int n = n0 + row;
+            const bool ok = (n < w_hi) && (c * 8 < p.d);
+            u32x4 z = {0, 0, 0, 0};
+            kr[i] = ok ? ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8) : z;
+            vr[i] = ok ? ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8) : z;
+        }
+    };
+    auto store_step = [&]() {
+#pragma unroll
+        for (int i = 0; i < C::LD; i++) {
+            const int f = lane + i * 64;
+            const int row = f / C::CPR, c = f % C::CPR;
+            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = kr[i];
+            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_vd<D>(c, row) * 16) = vr[i];
+        }
+    };
+
+    f32x4 o_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;   // l_run: this lane's share of the row sum
+    const float sl2 = kp.scale_log2;
+
+    int lim_hi = si.sk - 1;
+    if (has_right) lim_hi = min(lim_hi, qi + shift + wr);
+    const int lim_lo = has_left ? qi + shift - wl : 0;
+    const int tj = (lane & 15) >> 2, tq = lane & 3;
+
+    if (w_lo < w_hi) load_step(w_lo);
+    for (int n0 = w_lo; n0 < w_hi; n0 += C::STEP) {
+        // the previous step's LDS reads are complete (their results were consumed) before these
+        // writes are issued; LDS operations of one wave execute in order.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        store_step();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (n0 + C::STEP < w_hi) load_step(n0 + C::STEP);
+
+        // ---- S^T (2 blocks of 16 keys) = K Q^T
+        f32x4 s_acc[2];
+#pragma unroll
+        for (int kbk = 0; kbk < 2; kbk++) {
+            s_acc[kbk] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            const int krow = kbk * 16 + m;
+#pragma unroll
+            for (int c = 0; c < C::KC; c++) {
+                const int ch = c * 4 + g4;
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(kb + krow * C::ROWB + swz_k<D>(ch, krow) * 16);
+                s_acc[kbk] = Elem<T>::mfma16(__builtin_bit_cast(v8, raw), qf[c], s_acc[kbk]);
+            }
+        }
+        // ---- mask + online softmax; lane (m, g4) holds keys n0 + 16*kbk + 4*g4 + r of row m
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kbk = 0; kbk < 2; kbk++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int n = n0 + kbk * 16 + 4 * g4 + r;
+                if (n > lim_hi || n < lim_lo || n >= w_hi) s_acc[kbk][r] = -INFINITY;
+                mx = fmaxf(mx, s_acc[kbk][r]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = fast_exp2((m_run - m_use) * sl2);
+        const float msc = m_use * sl2;
+        float sum = 0.f;
+        float pv[8];
+#pragma unroll
+        for (int kbk = 0; kbk < 2; kbk++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float e = fast_exp2(s_acc[kbk][r] * sl2 - msc);
+                pv[kbk * 4 + r] = e;
+                sum += e;
+            }
+        l_run = l_run * corr + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int db = 0; db < C::DB; db++) o_acc[db] *= corr;
+        const v8 pf = __builtin_bit_cast(v8, pack8<T>(pv));
+
+        // ---- O^T += V^T P^T ; A operand rows: keys {4*g4 + j, 16 + 4*g4 + j}
+        const int vrow = 4 * g4 + tj;
+#pragma unroll
+        for (int db = 0; db < C::DB; db++) {
+            const int ch = db * 2 + (tq >> 1);
+            const int off = swz_vd<D>(ch, vrow) * 16 + (tq & 1) * 8;
+            const u32x2 lo2 = lds_read_tr16(vb + vrow * C::ROWB + off);
+            const u32x2 hi2 = lds_read_tr16(vb + (vrow + 16) * C::ROWB + off);
+            u32x4 raw = {lo2[0], lo2[1], hi2[0], hi2[1]};
+            o_acc[db] = Elem<T>::mfma16(__builtin_bit_cast(v8, raw), pf, o_acc[db]);
+        }
+    }
+
+    // ---- merge the four waves through LDS.  Layout per wave: 16 rows x (D floats of O, m, l).
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    __syncthreads();   // all waves are done with their staging tiles
+    constexpr int RSTR = D + 2;
+    float* msm = reinterpret_cast<float*>(smem);
+    {
+        float* mine = msm + (wave * 16 + m) * RSTR;
+#pragma unroll
+        for (int db = 0; db < C::DB; db++) {
+            const int d0 = db * 16 + 4 * g4;
+            mine[d0] = o_acc[db][0]; mine[d0 + 1] = o_acc[db][1];
+            mine[d0 + 2] = o_acc[db][2]; mine[d0 + 3] = o_acc[db][3];
+        }
+        if (g4 == 0) { mine[D] = m_run; mine[D + 1] = l_run; }
+    }
+    __syncthreads();
+    {
+        constexpr int EPT = D / 16;              // elements per thread
+        const int row = tid >> 4, dseg = (tid & 15) * EPT;
+        float mw[4], lw[4], mfin = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            mw[w] = msm[(w * 16 + row) * RSTR + D];
+            lw[w] = msm[(w * 16 + row) * RSTR + D + 1];
+            mfin = fmaxf(mfin, mw[w]);
+        }
+        const float m_use = (mfin == -INFINITY) ? 0.f : mfin;
+        float acc[EPT], ltot = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPT; e++) acc[e] = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float sc = fast_exp2((mw[w] - m_use) * sl2);
+            ltot += lw[w] * sc;
+#pragma unroll
+            for (int e = 0; e < EPT; e++) acc[e] += msm[(w * 16 + row) * RSTR + dseg + e] * sc;
+        }
+        const bool dead = (ltot == 0.f) || (ltot != ltot);
+        const float inv = dead ? 1.f : 1.f / ltot;
+        if (row < rows) {
+            const int i = row / G, hd = hk * G + row % G;
+            const float lse_fin = m_use * p.softmax_scale + __logf(ltot);
+            if (SPLIT) {
+                const int64_t ridx = (((int64_t)split * p.b + b) * p.h + hd) * p.seqlen_q + i;
+                if ((tid & 15) == 0) p.lse_accum[ridx] = dead ? -INFINITY : lse_fin;
+                float* orow = p.o_accum + ridx * kp.d_rounded;
+#pragma unroll
+                for (int e = 0; e < EPT; e += 4) {
+                    if (dseg + e < kp.d_rounded) {
+                        f32x4 v = {acc[e] * inv, acc[e + 1] * inv, acc[e + 2] * inv, acc[e + 3] * inv};
+                        *reinterpret_cast<f32x4*>(orow + dseg + e) = v;
+                    }
+                }
+            } else {
+                if ((tid & 15) == 0) p.softmax_lse[((int64_t)b * p.h + hd) * p.seqlen_q + i] = dead ? INFINITY : lse_fin;
+                T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)i * p.o_row_stride + (int64_t)hd * p.o_head_stride;
+#pragma unroll
+                for (int e = 0; e < EPT; e += 4) {
+                    if (dseg + e < p.d) {
+                        u32x2 v = {pack2<T>(acc[e] * inv, acc[e + 1] * inv), pack2<T>(acc[e + 2] * inv, acc[e + 3] * inv)};
+                        st_global8(orow + dseg + e, v);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int D>
+static int launch_decode_t(const KParams& kp, hipStream_t stream) {
+    typedef DecodeCfg<T, D> C;
+    const bool split = kp.num_splits > 1;
+    dim3 grid(split ? kp.num_splits : 1, kp.p.h_k, kp.p.b), block(C::kThreads);
+    hipError_t e;
+    if (split) {
+        auto kern = decode_kernel<T, D, true>;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    } else {
+        auto kern = decode_kernel<T, D, false>;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    }
+    return (int)hipGetLastError();
+}
+
+int launch_decode(const KParams& kp, hipStream_t stream) {
+    const int d = kp.p.d;
+    const bool bf = kp.p.dtype == FA_DTYPE_BF16;
+    if (d <= 64) return bf ? launch_decode_t<__bf16, 64>(kp, stream) : launch_decode_t<_Float16, 64>(kp, stream);
+    if (d <= 128) return bf ? launch_decode_t<__bf16, 128>(kp, stream) : launch_decode_t<_Float16, 128>(kp, stream);
+    return bf ? launch_decode_t<__bf16, 256>(kp, stream) : launch_decode_t<_Float16, 256>(kp, stream);
+}
+
+}  // namespace fa

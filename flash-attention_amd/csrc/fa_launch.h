@@ -1,0 +1,21 @@
+// Host-side launcher declarations shared by the kernel translation units and the C ABI.
+#pragma once
+#include "fa_common.h"
+
+namespace fa {
+#define FA_DECL_PREFILL(name) int name(const KParams& kp, hipStream_t stream);
+FA_DECL_PREFILL(launch_prefill_bf16_64)
+FA_DECL_PREFILL(launch_prefill_bf16_128)
+FA_DECL_PREFILL(launch_prefill_bf16_256)
+FA_DECL_PREFILL(launch_prefill_fp16_64)
+FA_DECL_PREFILL(launch_prefill_fp16_128)
+FA_DECL_PREFILL(launch_prefill_fp16_256)
+#undef FA_DECL_PREFILL
+
+int prefill_block_n(int d_bucket);   // key-tile length of the prefill kernel for a bucket
+int prefill_block_m(int d_bucket);
+
+int launch_decode(const KParams& kp, hipStream_t stream);      // small-q split-KV kernel
+int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials
+int launch_append_kv(const KParams& kp, hipStream_t stream);   // k_new/v_new (+rotary) -> cache
+}  // namespace fa

@@ -1,0 +1,366 @@
+// Tiled online-softmax forward kernel for gfx950 (multi-row query tiles: prefill, training
+// forward, chunked prefill against a KV cache).  Counterpart of the reference's
+// compute_attn_1rowblock / compute_attn_1rowblock_splitkv
+// (csrc/flash_attn/src/flash_fwd_kernel.h:74-580, 584-1130), designed for CDNA4:
+//
+//  * A workgroup is 4 wave64s; each wave owns RB blocks of 32 query rows and keeps its Q
+//    fragments in registers for the whole kernel.
+//  * Scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16: the accumulator
+//    layout then gives every lane 16 keys of ONE query row (row = lane % 32), so row max / row sum
+//    are in-lane reductions plus one v_permlane32_swap, and the probabilities are already in the
+//    B-operand layout of the second product O^T = V^T P^T -- P never leaves registers.
+//  * O^T accumulators likewise hold one query row per lane: the online-softmax rescale is a
+//    per-lane scalar multiply, no broadcast.
+//  * K and V tiles are double-buffered in LDS with 16-byte-chunk XOR swizzles chosen so that the
+//    K fragment reads (ds_read_b128) and the transposing V reads (ds_read_b64_tr_b16) are
+//    bank-conflict free; global loads are 128-bit, issued one tile ahead.
+//  * Key tiles that a wave's rows cannot see (causal / sliding window) are skipped per wave.
+#pragma once
+#include "fa_common.h"
+
+namespace fa {
+
+template <typename T, int D, int RB, int BN>
+struct PrefillCfg {
+    static constexpr int kThreads = 256;
+    static constexpr int kWaves = 4;
+    static constexpr int BM = kWaves * 32 * RB;   // query rows per workgroup
+    static constexpr int NB = BN / 32;            // 32-key blocks per key tile
+    static constexpr int KS = D / 16;             // k-steps of S^T = K Q^T
+    static constexpr int DB = D / 32;             // 32-row blocks of O^T
+    static constexpr int PT = BN / 16;            // k-steps of O^T = V^T P^T
+    static constexpr int CPR = D / 8;             // 16-byte chunks per tile row
+    static constexpr int ROWB = D * 2;            // bytes per tile row
+    static constexpr int TILE_BYTES = BN * ROWB;
+    static constexpr int LOADS = BN * CPR / kThreads;  // 16 B loads per thread, per tensor, per tile
+    static constexpr int SMEM = 4 * TILE_BYTES;   // {K,V} x 2 stages
+    static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
+};
+
+template <typename T, int D, int RB, int BN, int MINW, bool SPLIT>
+__global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
+    typedef PrefillCfg<T, D, RB, BN> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_fwd_params& p = kp.p;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int l32 = lane & 31, hh = lane >> 5;
+
+    // ---- work decode: contiguous ranges of the logical order go to one XCD (block ids are
+    // dealt round-robin over the 8 XCDs), so that workgroups sharing a K/V stream share an L2.
+    const int G = p.h / p.h_k;
+    const int S = SPLIT ? kp.num_splits : 1;
+    const int64_t total = (int64_t)kp.num_m_blocks * p.h * p.b * S;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int split = (int)(w % S); w /= S;
+    const int g = (int)(w % G); w /= G;
+    const int mb = kp.num_m_blocks - 1 - (int)(w % kp.num_m_blocks); w /= kp.num_m_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+    const int head = hk * G + g;
+
+    const SeqInfo si = seq_info(p, b);
+    const int m0 = mb * C::BM;
+    if (m0 >= si.sq) return;
+
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    int n_hi = si.sk;
+    if (has_right) n_hi = min(n_hi, min(m0 + C::BM, si.sq) + shift + wr);
+    int n_lo = 0;
+    if (has_left) n_lo = max(0, m0 + shift - wl);
+    int t_lo = n_lo / BN;
+    int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
+    if (SPLIT) {
+        const int s_lo = split * (kp.split_len / BN);
+        t_lo = max(t_lo, s_lo);
+        t_hi = min(t_hi, s_lo + kp.split_len / BN);
+    }
+
+    const T* __restrict__ qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
+    const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
+    const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
+
+    // ---- Q fragments (B operand of S^T = K Q^T): lane (l32, hh) holds Q[row l32][16*dk + 8*hh ..+7]
+    v8 qf[RB][C::KS];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        const int row = m0 + (wave * RB + rb) * 32 + l32;
+        const bool valid = row < si.sq;
+        const T* qrow = qg + (int64_t)row * p.q_row_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 raw = {0, 0, 0, 0};
+            if (valid && d0 < p.d) {
+                raw = ld_global16(qrow + d0);
+                if (kp.rotary_q && d0 < p.rotary_dim) {
+                    const int pos = si.sk_cache + ((p.is_causal || has_left || has_right) ? row : 0);
+                    const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
+                    const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
+                    float x[8];
+                    unpack8<T>(raw, x);
+                    rotary8<T>(x, qrow, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
+                    raw = pack8<T>(x);
+                }
+            }
+            qf[rb][dk] = __builtin_bit_cast(v8, raw);
+        }
+    }
+
+    f32x16 o_acc[RB][C::DB];
+    float m_run[RB], l_run[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        m_run[rb] = -INFINITY;
+        l_run[rb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < C::DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o_acc[rb][db][r] = 0.f;
+    }
+
+    // ---- tile movers
+    u32x4 kr[C::LOADS], vr[C::LOADS];
+    auto load_tile = [&](int t) {
+        const int n0 = t * BN;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int row = f / C::CPR, c = f % C::CPR;
+            const int n = n0 + row;
+            const bool ok = (n < si.sk) && (c * 8 < p.d);
+            u32x4 z = {0, 0, 0, 0};
+            kr[i] = ok ? ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8) : z;
+            vr[i] = ok ? ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8) : z;
+        }
+    };
+    auto store_tile = [&](int buf) {
+        char* kb = smem + buf * 2 * C::TILE_BYTES;
+        char* vb = kb + C::TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int row = f / C::CPR, c = f % C::CPR;
+            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = kr[i];
+            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_v<D>(c, row) * 16) = vr[i];
+        }
+    };
+
+    // per-lane pieces of the transposing V read: within a 16-lane block lane 4*j+q addresses row j,
+    // columns 4q..4q+3 of a 4-key x 16-dim tile.
+    const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
+
+    const float sl2 = kp.scale_log2;
+
+    if (t_hi > t_lo) {
+        load_tile(t_hi - 1);
+        store_tile(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int t = t_hi - 1; t >= t_lo; --t) {
+        const bool has_next = t > t_lo;
+        if (has_next) load_tile(t - 1);
+
+        const int n0 = t * BN;
+        const char* kb = smem + buf * 2 * C::TILE_BYTES;
+        const char* vb = kb + C::TILE_BYTES;
+
+        bool skip[RB];
+        bool any_work = false;
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            const int r0 = m0 + (wave * RB + rb) * 32;
+            skip[rb] = (has_right && n0 > r0 + 31 + shift + wr) ||
+                       (has_left && n0 + BN - 1 < r0 + shift - wl) || (r0 >= si.sq);
+            any_work |= !skip[rb];
+        }
+
+        if (any_work) {
+            // ---- S^T = K Q^T
+            f32x16 s_acc[RB][C::NB];
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s_acc[rb][nb][r] = 0.f;
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++) {
+                const int krow = nb * 32 + l32;
+#pragma unroll
+                for (int dk = 0; dk < C::KS; dk++) {
+                    const int c = dk * 2 + hh;
+                    const u32x4 raw = *reinterpret_cast<const u32x4*>(kb + krow * C::ROWB + swz_k<D>(c, krow) * 16);
+                    const v8 a = __builtin_bit_cast(v8, raw);
+#pragma unroll
+                    for (int rb = 0; rb < RB; rb++)
+                        if (!skip[rb]) s_acc[rb][nb] = Elem<T>::mfma32(a, qf[rb][dk], s_acc[rb][nb]);
+                }
+            }
+
+            // ---- mask, online softmax, pack P
+            v8 pf[RB][C::PT];
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                if (skip[rb]) continue;
+                const int r0 = m0 + (wave * RB + rb) * 32;
+                const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0 + shift + wr) ||
+                                       (has_left && n0 < r0 + 31 + shift - wl);
+                if (need_mask) {
+                    const int row = r0 + l32;
+                    int lim_hi = si.sk - 1;
+                    if (has_right) lim_hi = min(lim_hi, row + shift + wr);
+                    const int lim_lo = has_left ? row + shift - wl : 0;
+#pragma unroll
+                    for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                            if (n > lim_hi || n < lim_lo) s_acc[rb][nb][r] = -INFINITY;
+                        }
+                }
+                float mx = -INFINITY;
+#pragma unroll
+                for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) mx = fmaxf(mx, s_acc[rb][nb][r]);
+                mx = xhalf_max(mx);
+                const float m_old = m_run[rb];
+                const float m_new = fmaxf(m_old, mx);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                const float corr = fast_exp2((m_old - m_use) * sl2);
+                const float msc = m_use * sl2;
+                float sum = 0.f;
+#pragma unroll
+                for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const float pv = fast_exp2(s_acc[rb][nb][r] * sl2 - msc);
+                        s_acc[rb][nb][r] = pv;
+                        sum += pv;
+                    }
+                l_run[rb] = l_run[rb] * corr + sum;
+                m_run[rb] = m_new;
+                if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
+#pragma unroll
+                    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) o_acc[rb][db][r] *= corr;
+                }
+#pragma unroll
+                for (int t16 = 0; t16 < C::PT; t16++) {
+                    const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
+                    u32x4 pk;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        pk[e] = pack2<T>(s_acc[rb][nb][r8 + 2 * e], s_acc[rb][nb][r8 + 2 * e + 1]);
+                    pf[rb][t16] = __builtin_bit_cast(v8, pk);
+                }
+            }
+
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int t16 = 0; t16 < C::PT; t16++) {
+                const int vrow = t16 * 16 + 4 * hh + tj;   // second read: +8 rows (same row & 3)
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) {
+                    const int c = db * 4 + dhalf * 2 + (tq >> 1);
+                    const int off = swz_v<D>(c, vrow) * 16 + (tq & 1) * 8;
+                    const u32x2 lo = lds_read_tr16(vb + vrow * C::ROWB + off);
+                    const u32x2 hi = lds_read_tr16(vb + (vrow + 8) * C::ROWB + off);
+                    u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+                    const v8 a = __builtin_bit_cast(v8, raw);
+#pragma unroll
+                    for (int rb = 0; rb < RB; rb++)
+                        if (!skip[rb]) o_acc[rb][db] = Elem<T>::mfma32(a, pf[rb][t16], o_acc[rb][db]);
+                }
+            }
+        }
+
+        if (has_next) store_tile(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // ---- epilogue: normalise, write O (and log-sum-exp).  A row that saw no key gives 0 / +inf
+    // (reference: flash_fwd_kernel.h:509-516), a split that saw no key gives 0 / -inf (:623-662).
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        const int row = m0 + (wave * RB + rb) * 32 + l32;
+        const float l_tot = xhalf_sum(l_run[rb]);
+        const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
+        const float inv = dead ? 1.f : 1.f / l_tot;
+        const float lse = dead ? (SPLIT ? -INFINITY : INFINITY) : m_run[rb] * p.softmax_scale + __logf(l_tot);
+        if (row >= si.sq) continue;
+        if (SPLIT) {
+            const int64_t ridx = (((int64_t)split * p.b + b) * p.h + head) * p.seqlen_q + row;
+            if (hh == 0) p.lse_accum[ridx] = lse;
+            float* orow = p.o_accum + ridx * kp.d_rounded;
+#pragma unroll
+            for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int d0 = db * 32 + 8 * q4 + 4 * hh;
+                    if (d0 < kp.d_rounded) {
+                        f32x4 v = {o_acc[rb][db][4 * q4] * inv, o_acc[rb][db][4 * q4 + 1] * inv,
+                                   o_acc[rb][db][4 * q4 + 2] * inv, o_acc[rb][db][4 * q4 + 3] * inv};
+                        *reinterpret_cast<f32x4*>(orow + d0) = v;
+                    }
+                }
+        } else {
+            if (hh == 0) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
+            T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)row * p.o_row_stride + (int64_t)head * p.o_head_stride;
+#pragma unroll
+            for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int d0 = db * 32 + 8 * q4 + 4 * hh;
+                    if (d0 < p.d) {
+                        u32x2 v = {pack2<T>(o_acc[rb][db][4 * q4] * inv, o_acc[rb][db][4 * q4 + 1] * inv),
+                                   pack2<T>(o_acc[rb][db][4 * q4 + 2] * inv, o_acc[rb][db][4 * q4 + 3] * inv)};
+                        st_global8(orow + d0, v);
+                    }
+                }
+        }
+    }
+}
+
+template <typename T, int D, int RB, int BN, int MINW>
+int launch_prefill(KParams kp, hipStream_t stream) {
+    typedef PrefillCfg<T, D, RB, BN> C;
+    kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
+    const bool split = kp.num_splits > 1;
+    const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b * (split ? kp.num_splits : 1);
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
+    hipError_t e;
+    if (split) {
+        auto kern = prefill_kernel<T, D, RB, BN, MINW, true>;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    } else {
+        auto kern = prefill_kernel<T, D, RB, BN, MINW, false>;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    }
+    return (int)hipGetLastError();
+}
+
+// key-tile length used by launch_prefill for a head-dim bucket (the split planner needs it)
+template <int D> struct PrefillTile;
+template <> struct PrefillTile<64> { static constexpr int RB = 1, BN = 64, MINW = 2; };
+template <> struct PrefillTile<128> { static constexpr int RB = 1, BN = 64, MINW = 2; };
+template <> struct PrefillTile<256> { static constexpr int RB = 1, BN = 32, MINW = 1; };
+
+}  // namespace fa

@@ -1,0 +1,412 @@
+"""ctypes binding of libfa_mi355x.so, shaped like the reference's pybind11 module.
+
+The three functions `fwd`, `varlen_fwd`, `fwd_kvcache` take the same positional arguments and
+return the same tensor lists as `flash_attn_2_cuda.fwd / varlen_fwd / fwd_kvcache`
+(csrc/flash_attn/flash_api.cpp:248-259, 426-442, 1038-1055, return lists at :423, :584, :1278),
+so `flash_attn_interface.py` calls them exactly as the reference does.  What the reference does in
+C++ with ATen before its kernels run -- argument checks with the same messages, head-dim padding
+to a multiple of 8, output / log-sum-exp / split-accumulator allocation on q's device with the
+torch caching allocator, current-stream launch -- happens here; the shared library itself takes
+plain pointers and sizes and allocates nothing.
+
+There is no fallback: if the library is missing or cannot be loaded, importing this module fails.
+"""
+import ctypes
+import math
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libfa_mi355x.so")
+
+FA_DTYPE_FP16 = 0
+FA_DTYPE_BF16 = 1
+
+
+class FaFwdParams(ctypes.Structure):
+    """Mirror of `fa_fwd_params` in include/fa_mi355x.h (field order matters)."""
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in (
+            "q", "k", "v", "o", "softmax_lse", "o_accum", "lse_accum", "k_new", "v_new",
+            "rotary_cos", "rotary_sin", "cu_seqlens_q", "cu_seqlens_k", "cache_batch_idx")]
+        + [(n, ctypes.c_int64) for n in (
+            "q_batch_stride", "q_row_stride", "q_head_stride",
+            "k_batch_stride", "k_row_stride", "k_head_stride",
+            "v_batch_stride", "v_row_stride", "v_head_stride",
+            "o_batch_stride", "o_row_stride", "o_head_stride",
+            "knew_batch_stride", "knew_row_stride", "knew_head_stride",
+            "vnew_batch_stride", "vnew_row_stride", "vnew_head_stride")]
+        + [(n, ctypes.c_int32) for n in (
+            "b", "h", "h_k", "seqlen_q", "seqlen_k", "seqlen_knew", "d", "rotary_dim",
+            "window_left", "window_right", "is_causal", "is_seqlens_k_cumulative",
+            "is_rotary_interleaved", "num_splits", "dtype")]
+        + [("softmax_scale", ctypes.c_float)]
+    )
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            "flash_attn: %s not found. Build it with `python flash-attention_amd/build.py` "
+            "(hipcc, gfx950). There is no fallback implementation." % _LIB_PATH)
+    lib = ctypes.CDLL(_LIB_PATH)
+    P = ctypes.POINTER(FaFwdParams)
+    for name in ("fa_fwd", "fa_varlen_fwd", "fa_fwd_kvcache"):
+        f = getattr(lib, name)
+        f.argtypes = [P, ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    lib.fa_plan_splits.argtypes = [P, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)]
+    lib.fa_plan_splits.restype = ctypes.c_int
+    lib.fa_num_splits_heuristic_reference.argtypes = [ctypes.c_int32] * 4
+    lib.fa_num_splits_heuristic_reference.restype = ctypes.c_int
+    lib.fa_last_error.argtypes = []
+    lib.fa_last_error.restype = ctypes.c_char_p
+    lib.fa_version.argtypes = []
+    lib.fa_version.restype = ctypes.c_int32
+    lib.fa_sizeof_params.argtypes = []
+    lib.fa_sizeof_params.restype = ctypes.c_int32
+    if lib.fa_sizeof_params() != ctypes.sizeof(FaFwdParams):
+        raise ImportError("flash_attn: fa_fwd_params layout mismatch between %s (%d bytes) and its "
+                          "Python mirror (%d bytes); rebuild the library" %
+                          (_LIB_PATH, lib.fa_sizeof_params(), ctypes.sizeof(FaFwdParams)))
+    return lib
+
+
+lib = _load()
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _call(fn, params, stream):
+    rc = fn(ctypes.byref(params), ctypes.c_void_p(stream))
+    if rc != 0:
+        raise RuntimeError(lib.fa_last_error().decode() or "libfa_mi355x: error %d" % rc)
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _dtype_code(dtype):
+    _check(dtype in (torch.float16, torch.bfloat16), "FlashAttention only support fp16 and bf16 data type")
+    return FA_DTYPE_BF16 if dtype == torch.bfloat16 else FA_DTYPE_FP16
+
+
+def _check_device(*ts):
+    for t in ts:
+        _check(t.is_cuda, "Input tensor must be on CUDA device")
+
+
+def _pad8(t):
+    d = t.shape[-1]
+    return t if d % 8 == 0 else torch.nn.functional.pad(t, (0, 8 - d % 8))
+
+
+def _round_up(x, m):
+    return (x + m - 1) // m * m
+
+
+def _stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _plan_and_alloc(params, api, batch, heads, seqlen_q, d, device):
+    """Resolve the split count and allocate the fp32 partial buffers like the reference does
+    (flash_api.cpp:373-389, 1241-1257).  The returned tensors must stay alive until launch."""
+    n = ctypes.c_int32(0)
+    rc = lib.fa_plan_splits(ctypes.byref(params), api, ctypes.byref(n))
+    if rc != 0:
+        raise RuntimeError(lib.fa_last_error().decode())
+    params.num_splits = n.value
+    keep = None
+    if n.value > 1:
+        lse_accum = torch.empty((n.value, batch, heads, seqlen_q), dtype=torch.float32, device=device)
+        o_accum = torch.empty((n.value, batch, heads, seqlen_q, _round_up(d, 32)), dtype=torch.float32, device=device)
+        params.lse_accum = lse_accum.data_ptr()
+        params.o_accum = o_accum.data_ptr()
+        keep = (lse_accum, o_accum)
+    return keep
+
+
+def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, window_size_right,
+        return_softmax, gen_):
+    """Dense batch forward; mirrors mha_fwd (flash_api.cpp:248-424)."""
+    if p_dropout != 0.0:
+        raise NotImplementedError("dropout is not implemented in the MI355X forward path")
+    q_dtype = q.dtype
+    dt = _dtype_code(q_dtype)
+    _check(k.dtype == q_dtype, "query and key must have the same dtype")
+    _check(v.dtype == q_dtype, "query and value must have the same dtype")
+    _check_device(q, k, v)
+    for t in (q, k, v):
+        _check(t.stride(-1) == 1, "Input tensor must have contiguous last dimension")
+    _check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be 4-dimensional")
+    batch_size, seqlen_q, num_heads, head_size_og = q.shape
+    seqlen_k, num_heads_k = k.shape[1], k.shape[2]
+    _check(batch_size > 0, "batch size must be postive")
+    _check(head_size_og <= 256, "FlashAttention forward only supports head dimension at most 256")
+    _check(num_heads % num_heads_k == 0, "Number of heads in key/value must divide number of heads in query")
+    _check(tuple(k.shape) == (batch_size, seqlen_k, num_heads_k, head_size_og), "k must have shape (batch_size, seqlen_k, num_heads_k, head_size)")
+    _check(tuple(v.shape) == (batch_size, seqlen_k, num_heads_k, head_size_og), "v must have shape (batch_size, seqlen_k, num_heads_k, head_size)")
+    _check(not return_softmax, "return_softmax is only supported when p_dropout > 0.0")
+    if seqlen_q == 1:
+        is_causal = False
+    if is_causal:
+        window_size_right = 0
+
+    q_padded, k_padded, v_padded = _pad8(q), _pad8(k), _pad8(v)
+    if out_ is not None:
+        out = out_
+        _check(out.dtype == q_dtype, "Output must have the same dtype as inputs")
+        _check_device(out)
+        _check(out.stride(-1) == 1, "Output tensor must have contiguous last dimension")
+        _check(tuple(out.shape) == (batch_size, seqlen_q, num_heads, head_size_og), "out has the wrong shape")
+        if head_size_og % 8 != 0:
+            out = torch.empty_like(q_padded)
+    else:
+        out = torch.empty_like(q_padded)
+    head_size = q_padded.shape[-1]
+
+    with torch.cuda.device(q.device):
+        softmax_lse = torch.empty((batch_size, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
+        p = FaFwdParams()
+        p.q, p.k, p.v, p.o = q_padded.data_ptr(), k_padded.data_ptr(), v_padded.data_ptr(), out.data_ptr()
+        p.softmax_lse = softmax_lse.data_ptr()
+        p.q_batch_stride, p.q_row_stride, p.q_head_stride = q_padded.stride(0), q_padded.stride(1), q_padded.stride(2)
+        p.k_batch_stride, p.k_row_stride, p.k_head_stride = k_padded.stride(0), k_padded.stride(1), k_padded.stride(2)
+        p.v_batch_stride, p.v_row_stride, p.v_head_stride = v_padded.stride(0), v_padded.stride(1), v_padded.stride(2)
+        p.o_batch_stride, p.o_row_stride, p.o_head_stride = out.stride(0), out.stride(1), out.stride(2)
+        p.b, p.h, p.h_k = batch_size, num_heads, num_heads_k
+        p.seqlen_q, p.seqlen_k, p.d = seqlen_q, seqlen_k, head_size
+        p.window_left, p.window_right, p.is_causal = window_size_left, window_size_right, int(is_causal)
+        p.is_seqlens_k_cumulative = 1
+        p.num_splits = 0
+        p.dtype = dt
+        p.softmax_scale = softmax_scale
+        if seqlen_q > 0 and seqlen_k > 0:
+            keep = _plan_and_alloc(p, 0, batch_size, num_heads, seqlen_q, head_size, q.device)
+            _call(lib.fa_fwd, p, _stream(q.device))
+            del keep
+        else:
+            out.zero_()
+            softmax_lse.fill_(float("inf"))
+
+    out_padded = out
+    if head_size_og % 8 != 0:
+        out = out[..., :head_size_og]
+        if out_ is not None:
+            out_.copy_(out)
+    rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
+    return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, None, rng_state]
+
+
+def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout,
+               softmax_scale, zero_tensors, is_causal, window_size_left, window_size_right,
+               return_softmax, gen_):
+    """Packed variable-length forward; mirrors mha_varlen_fwd (flash_api.cpp:426-585)."""
+    if p_dropout != 0.0:
+        raise NotImplementedError("dropout is not implemented in the MI355X forward path")
+    q_dtype = q.dtype
+    dt = _dtype_code(q_dtype)
+    _check(k.dtype == q_dtype, "query and key must have the same dtype")
+    _check(v.dtype == q_dtype, "query and value must have the same dtype")
+    _check(cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
+    _check(cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
+    _check_device(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    for t in (q, k, v):
+        _check(t.stride(-1) == 1, "Input tensor must have contiguous last dimension")
+    _check(cu_seqlens_q.is_contiguous(), "cu_seqlens_q must be contiguous")
+    _check(cu_seqlens_k.is_contiguous(), "cu_seqlens_k must be contiguous")
+    _check(q.dim() == 3 and k.dim() == 3 and v.dim() == 3, "q, k, v must be 3-dimensional")
+    total_q, num_heads, head_size_og = q.shape
+    total_k, num_heads_k = k.shape[0], k.shape[1]
+    batch_size = cu_seqlens_q.numel() - 1
+    _check(batch_size > 0, "batch size must be positive")
+    _check(head_size_og <= 256, "FlashAttention forward only supports head dimension at most 256")
+    _check(num_heads % num_heads_k == 0, "Number of heads in key/value must divide number of heads in query")
+    _check(tuple(k.shape) == (total_k, num_heads_k, head_size_og), "k must have shape (total_k, num_heads_k, head_size)")
+    _check(tuple(v.shape) == (total_k, num_heads_k, head_size_og), "v must have shape (total_k, num_heads_k, head_size)")
+    _check(tuple(cu_seqlens_q.shape) == (batch_size + 1,), "cu_seqlens_q must have shape (batch_size + 1)")
+    _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
+    _check(not return_softmax, "return_softmax is only supported when p_dropout > 0.0")
+    if is_causal:
+        window_size_right = 0
+
+    q_padded, k_padded, v_padded = _pad8(q), _pad8(k), _pad8(v)
+    if out_ is not None:
+        out = out_
+        _check(out.dtype == q_dtype, "Output must have the same dtype as inputs")
+        _check_device(out)
+        _check(out.stride(-1) == 1, "Output tensor must have contiguous last dimension")
+        _check(tuple(out.shape) == (total_q, num_heads, head_size_og), "out has the wrong shape")
+        if head_size_og % 8 != 0:
+            out = torch.empty_like(q_padded)
+    else:
+        out = torch.empty_like(q_padded)
+    head_size = q_padded.shape[-1]
+
+    with torch.cuda.device(q.device):
+        softmax_lse = torch.empty((batch_size, num_heads, max_seqlen_q), dtype=torch.float32, device=q.device)
+        if zero_tensors:
+            out.zero_()
+            softmax_lse.fill_(float("-inf"))
+        p = FaFwdParams()
+        p.q, p.k, p.v, p.o = q_padded.data_ptr(), k_padded.data_ptr(), v_padded.data_ptr(), out.data_ptr()
+        p.softmax_lse = softmax_lse.data_ptr()
+        p.cu_seqlens_q, p.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
+        p.q_row_stride, p.q_head_stride = q_padded.stride(0), q_padded.stride(1)
+        p.k_row_stride, p.k_head_stride = k_padded.stride(0), k_padded.stride(1)
+        p.v_row_stride, p.v_head_stride = v_padded.stride(0), v_padded.stride(1)
+        p.o_row_stride, p.o_head_stride = out.stride(0), out.stride(1)
+        p.b, p.h, p.h_k = batch_size, num_heads, num_heads_k
+        p.seqlen_q, p.seqlen_k, p.d = max_seqlen_q, max_seqlen_k, head_size
+        p.window_left, p.window_right, p.is_causal = window_size_left, window_size_right, int(is_causal)
+        p.is_seqlens_k_cumulative = 1
+        p.num_splits = 1
+        p.dtype = dt
+        p.softmax_scale = softmax_scale
+        if total_q > 0 and max_seqlen_q > 0:
+            _call(lib.fa_varlen_fwd, p, _stream(q.device))
+
+    out_padded = out
+    if head_size_og % 8 != 0:
+        out = out[..., :head_size_og]
+        if out_ is not None:
+            out_.copy_(out)
+    rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
+    return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, None, rng_state]
+
+
+def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_,
+                out_, softmax_scale, is_causal, window_size_left, window_size_right,
+                is_rotary_interleaved, num_splits):
+    """KV-cache forward with optional append + rotary; mirrors mha_fwd_kvcache
+    (flash_api.cpp:1038-1279).  Returns [out, softmax_lse]."""
+    q_dtype = q.dtype
+    dt = _dtype_code(q_dtype)
+    _check(kcache.dtype == q_dtype, "query and key must have the same dtype")
+    _check(vcache.dtype == q_dtype, "query and value must have the same dtype")
+    _check_device(q, kcache, vcache)
+    for t in (q, kcache, vcache):
+        _check(t.stride(-1) == 1, "Input tensor must have contiguous last dimension")
+    _check(q.dim() == 4 and kcache.dim() == 4 and vcache.dim() == 4, "q, k_cache, v_cache must be 4-dimensional")
+    batch_size, seqlen_q, num_heads, head_size_og = q.shape
+    batch_size_c, seqlen_k, num_heads_k = kcache.shape[0], kcache.shape[1], kcache.shape[2]
+    _check(batch_size > 0, "batch size must be postive")
+    _check(head_size_og <= 256, "FlashAttention forward only supports head dimension at most 256")
+    _check(num_heads % num_heads_k == 0, "Number of heads in key/value must divide number of heads in query")
+    _check(tuple(kcache.shape) == (batch_size_c, seqlen_k, num_heads_k, head_size_og), "k_cache has the wrong shape")
+    _check(tuple(vcache.shape) == (batch_size_c, seqlen_k, num_heads_k, head_size_og), "v_cache has the wrong shape")
+    if cache_batch_idx_ is None:
+        _check(batch_size_c >= batch_size, "k_cache must hold at least batch_size rows")
+    if seqlen_q == 1:
+        is_causal = False
+    if is_causal:
+        window_size_right = 0
+
+    padded = head_size_og % 8 != 0
+    q_padded, kcache_padded, vcache_padded = _pad8(q), _pad8(kcache), _pad8(vcache)
+    if out_ is not None:
+        out = out_
+        _check(out.dtype == q_dtype, "Output must have the same dtype as inputs")
+        _check_device(out)
+        _check(out.stride(-1) == 1, "Output tensor must have contiguous last dimension")
+        _check(tuple(out.shape) == (batch_size, seqlen_q, num_heads, head_size_og), "out has the wrong shape")
+        if padded:
+            out = torch.empty_like(q_padded)
+    else:
+        out = torch.empty_like(q_padded)
+    head_size = q_padded.shape[-1]
+
+    with torch.cuda.device(q.device):
+        softmax_lse = torch.empty((batch_size, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
+        p = FaFwdParams()
+        p.q, p.k, p.v, p.o = q_padded.data_ptr(), kcache_padded.data_ptr(), vcache_padded.data_ptr(), out.data_ptr()
+        p.softmax_lse = softmax_lse.data_ptr()
+        p.q_batch_stride, p.q_row_stride, p.q_head_stride = q_padded.stride(0), q_padded.stride(1), q_padded.stride(2)
+        p.k_batch_stride, p.k_row_stride, p.k_head_stride = kcache_padded.stride(0), kcache_padded.stride(1), kcache_padded.stride(2)
+        p.v_batch_stride, p.v_row_stride, p.v_head_stride = vcache_padded.stride(0), vcache_padded.stride(1), vcache_padded.stride(2)
+        p.o_batch_stride, p.o_row_stride, p.o_head_stride = out.stride(0), out.stride(1), out.stride(2)
+        p.b, p.h, p.h_k = batch_size, num_heads, num_heads_k
+        p.seqlen_q, p.seqlen_k, p.d = seqlen_q, seqlen_k, head_size
+        p.window_left, p.window_right, p.is_causal = window_size_left, window_size_right, int(is_causal)
+        p.dtype = dt
+        p.softmax_scale = softmax_scale
+
+        keep = []
+        if k_ is not None:
+            _check(v_ is not None, "If key is supplied, value must also be passed in")
+            _check(seqlens_k_ is not None, "If key is supplied, seqlens_k must also be passed in")
+            _check(seqlen_q <= seqlen_k, "If key is supplied, it must have seqlen <= the seqlen of the KV cache")
+            _check(k_.dtype == q_dtype, "Key must have the same dtype as query")
+            _check(v_.dtype == q_dtype, "Value must have the same dtype as query")
+            _check_device(k_, v_)
+            _check(k_.stride(-1) == 1, "Key tensor must have contiguous last dimension")
+            _check(v_.stride(-1) == 1, "Value tensor must have contiguous last dimension")
+            seqlen_knew = k_.shape[1]
+            _check(tuple(k_.shape) == (batch_size, seqlen_knew, num_heads_k, head_size_og), "k has the wrong shape")
+            _check(tuple(v_.shape) == (batch_size, seqlen_knew, num_heads_k, head_size_og), "v has the wrong shape")
+            k_padded, v_padded = _pad8(k_), _pad8(v_)
+            keep += [k_padded, v_padded]
+            p.seqlen_knew = seqlen_knew
+            p.k_new, p.v_new = k_padded.data_ptr(), v_padded.data_ptr()
+            p.knew_batch_stride, p.knew_row_stride, p.knew_head_stride = k_padded.stride(0), k_padded.stride(1), k_padded.stride(2)
+            p.vnew_batch_stride, p.vnew_row_stride, p.vnew_head_stride = v_padded.stride(0), v_padded.stride(1), v_padded.stride(2)
+        if seqlens_k_ is not None:
+            _check(seqlens_k_.dtype == torch.int32, "seqlens_k must have dtype int32")
+            _check_device(seqlens_k_)
+            _check(seqlens_k_.is_contiguous(), "seqlens_k must be contiguous")
+            _check(tuple(seqlens_k_.shape) == (batch_size,), "seqlens_k must have shape (batch_size)")
+            p.cu_seqlens_k = seqlens_k_.data_ptr()
+        p.is_seqlens_k_cumulative = int(seqlens_k_ is None)
+        if rotary_cos_ is not None:
+            _check(k_ is not None, "If rotary cos/sin are provided, new key / value to be appended to KV cache must also be provided")
+            _check_device(rotary_cos_)
+            rotary_dim = rotary_cos_.shape[1] * 2
+            _check(rotary_dim <= head_size, "rotary_dim must be <= headdim")
+            _check(rotary_dim % 16 == 0, "Only rotary dimensions divisible by 16 are currently supported")
+            seqlen_ro = rotary_cos_.shape[0]
+            _check(seqlen_ro >= seqlen_k, "cos/sin seqlen must be at least the seqlen of KV cache")
+            _check(tuple(rotary_cos_.shape) == (seqlen_ro, rotary_dim // 2), "rotary_cos has the wrong shape")
+            _check(rotary_cos_.is_contiguous(), "rotary_cos must be contiguous")
+            _check(rotary_cos_.dtype == q_dtype, "rotary_cos must have the same dtype as query")
+            _check(rotary_sin_ is not None, "If rotary cos is provided, rotary sin must also be provided")
+            _check_device(rotary_sin_)
+            _check(tuple(rotary_sin_.shape) == (seqlen_ro, rotary_dim // 2), "rotary_sin has the wrong shape")
+            _check(rotary_sin_.is_contiguous(), "rotary_sin must be contiguous")
+            _check(rotary_sin_.dtype == q_dtype, "rotary_cos must have the same dtype as query")
+            p.rotary_cos, p.rotary_sin = rotary_cos_.data_ptr(), rotary_sin_.data_ptr()
+            p.rotary_dim = rotary_dim
+            p.is_rotary_interleaved = int(is_rotary_interleaved)
+        if cache_batch_idx_ is not None:
+            _check_device(cache_batch_idx_)
+            _check(cache_batch_idx_.is_contiguous(), "cache_batch_idx must be contiguous")
+            _check(cache_batch_idx_.dtype == torch.int32, "cache_batch_idx must have dtype int32")
+            p.cache_batch_idx = cache_batch_idx_.data_ptr()
+        _check(num_splits <= 128, "num_splits > 128 not supported")
+        p.num_splits = max(int(num_splits), 0)
+        if seqlen_q > 0 and seqlen_k > 0:
+            keep.append(_plan_and_alloc(p, 2, batch_size, num_heads, seqlen_q, head_size, q.device))
+            _call(lib.fa_fwd_kvcache, p, _stream(q.device))
+        else:
+            out.zero_()
+            softmax_lse.fill_(float("inf"))
+        del keep
+
+    if padded:
+        out = out[..., :head_size_og]
+        if out_ is not None:
+            out_.copy_(out)
+        if k_ is not None:
+            # the appended rows live in the padded copies; write them back (flash_api.cpp:1263-1272)
+            kcache.copy_(kcache_padded[..., :head_size_og])
+            vcache.copy_(vcache_padded[..., :head_size_og])
+    return [out, softmax_lse]
+
+
+def num_splits_heuristic_reference(batch_nheads_mblocks, num_sms, num_n_blocks, max_splits):
+    return lib.fa_num_splits_heuristic_reference(batch_nheads_mblocks, num_sms, num_n_blocks, max_splits)

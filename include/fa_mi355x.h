@@ -1,0 +1,136 @@
+/*
+ * C ABI of libfa_mi355x.so: FlashAttention-2 forward for AMD MI355X (gfx950).
+ *
+ * This is the native boundary that the `flash_attn` Python API binds.  It replaces the three
+ * forward entry points of the reference's pybind11 module `flash_attn_2_cuda`
+ * (csrc/flash_attn/flash_api.cpp:1281-1288).  Plain pointers and sizes only: no torch types, no
+ * allocation, no retained state.  Every buffer is owned by the caller; kernels are enqueued on the
+ * given HIP stream and the call returns without synchronising.
+ *
+ * Return value of every int function: 0 on success, non-zero on error; fa_last_error() then
+ * holds a message (thread-local).  The library never aborts the process.
+ */
+#ifndef FA_MI355X_H
+#define FA_MI355X_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_DTYPE_FP16 0
+#define FA_DTYPE_BF16 1
+
+#define FA_MAX_SPLITS 128
+
+/*
+ * Problem description.  POD mirror of the reference's Flash_fwd_params
+ * (csrc/flash_attn/src/flash.h:24-130), with 64-bit element strides so that tensors of 2^31
+ * elements and more are addressable.
+ *
+ * Layouts (all strides in ELEMENTS, last dimension contiguous):
+ *   q      (b, seqlen_q, h,   d)   or packed (total_q, h, d)   when cu_seqlens_q != NULL
+ *   k, v   (b_k, seqlen_k, h_k, d) or packed (total_k, h_k, d) when cu_seqlens_k is cumulative
+ *   o      like q
+ *   softmax_lse  (b, h, seqlen_q) fp32, natural log; +inf for a row that sees no key
+ *   o_accum      (num_splits, b, h, seqlen_q, d_rounded) fp32, d_rounded = d rounded up to 32
+ *   lse_accum    (num_splits, b, h, seqlen_q) fp32
+ * Masking is bottom-right aligned: query i sees key j iff
+ *   i + sk - sq - window_left <= j <= i + sk - sq + window_right and j < sk,
+ * a negative window bound meaning unbounded; is_causal forces window_right = 0.
+ */
+typedef struct fa_fwd_params {
+    const void *q, *k, *v;
+    void *o;
+    float *softmax_lse;
+    float *o_accum;   /* needed when the resolved split count is > 1 (see fa_plan_splits) */
+    float *lse_accum;
+
+    /* new keys/values appended to the cache before attention (fa_fwd_kvcache only), or NULL:
+     * (b, seqlen_knew, h_k, d) */
+    const void *k_new, *v_new;
+    /* rotary tables (seqlen_ro, rotary_dim/2) in the q dtype, contiguous, or NULL */
+    const void *rotary_cos, *rotary_sin;
+
+    const int32_t *cu_seqlens_q;    /* (b+1) prefix sums, or NULL for a dense batch */
+    const int32_t *cu_seqlens_k;    /* (b+1) prefix sums if is_seqlens_k_cumulative, else (b)
+                                       per-batch key lengths (cache_seqlens), or NULL */
+    const int32_t *cache_batch_idx; /* (b) row of k/v used (and updated) for batch i, or NULL */
+
+    int64_t q_batch_stride, q_row_stride, q_head_stride;
+    int64_t k_batch_stride, k_row_stride, k_head_stride;
+    int64_t v_batch_stride, v_row_stride, v_head_stride;
+    int64_t o_batch_stride, o_row_stride, o_head_stride;
+    int64_t knew_batch_stride, knew_row_stride, knew_head_stride;
+    int64_t vnew_batch_stride, vnew_row_stride, vnew_head_stride;
+
+    int32_t b;            /* batch size of q */
+    int32_t h, h_k;       /* query heads, key/value heads (h % h_k == 0) */
+    int32_t seqlen_q;     /* rows per batch entry; max_seqlen_q for packed input */
+    int32_t seqlen_k;     /* keys per batch entry (cache capacity); max_seqlen_k for packed input */
+    int32_t seqlen_knew;  /* rows of k_new / v_new, 0 if none */
+    int32_t d;            /* head dimension, multiple of 8, <= 256 */
+    int32_t rotary_dim;   /* 0 = no rotary; multiple of 16, <= d */
+
+    int32_t window_left, window_right;
+    int32_t is_causal;
+    int32_t is_seqlens_k_cumulative;
+    int32_t is_rotary_interleaved;
+    int32_t num_splits;   /* request: 0 = library decides, 1 = never split, n = at most n chunks */
+    int32_t dtype;        /* FA_DTYPE_* */
+    float softmax_scale;
+} fa_fwd_params;
+
+/*
+ * Dense batch forward.  Replaces mha_fwd (csrc/flash_attn/flash_api.cpp:248-424): same masking
+ * rules (seqlen_q == 1 disables causal, :296), same outputs (o and softmax_lse).  Splits the key
+ * range when p->num_splits resolves to > 1 (then o_accum / lse_accum must be set).
+ */
+int fa_fwd(const fa_fwd_params *p, void *hip_stream);
+
+/*
+ * Packed variable-length forward.  Replaces mha_varlen_fwd (flash_api.cpp:426-585): cu_seqlens_q
+ * and cu_seqlens_k are int32 prefix sums; softmax_lse is (b, h, max_seqlen_q) and rows beyond a
+ * sequence's length are left unwritten (:527).  Never splits.
+ */
+int fa_varlen_fwd(const fa_fwd_params *p, void *hip_stream);
+
+/*
+ * KV-cache forward.  Replaces mha_fwd_kvcache (flash_api.cpp:1038-1279): optional append of
+ * k_new/v_new at rows cache_seqlens[b] .. of cache row cache_batch_idx[b] (new keys rotated when
+ * rotary tables are given, :763-852 of flash_fwd_kernel.h), q rotated on load (:854-891), then
+ * attention over cache_seqlens[b] + seqlen_knew keys.  Mutates k and v in place.
+ */
+int fa_fwd_kvcache(const fa_fwd_params *p, void *hip_stream);
+
+/*
+ * Resolves the split count the library will use for this problem, so that the caller can size
+ * o_accum / lse_accum before the call (the reference does this inside mha_fwd / mha_fwd_kvcache,
+ * flash_api.cpp:373-389, 1241-1257, with num_splits_heuristic :212-246; this library uses its
+ * own rule for 256 CUs).  `api` is 0 for fa_fwd, 2 for fa_fwd_kvcache.  Writes the resolved count
+ * (1..FA_MAX_SPLITS) to *num_splits.  The same value must then be passed in p->num_splits.
+ */
+int fa_plan_splits(const fa_fwd_params *p, int32_t api, int32_t *num_splits);
+
+/*
+ * The reference's own split-count rule, kept as a pure utility for callers that rely on it
+ * (num_splits_heuristic, flash_api.cpp:212-246).
+ */
+int fa_num_splits_heuristic_reference(int32_t batch_nheads_mblocks, int32_t num_sms,
+                                      int32_t num_n_blocks, int32_t max_splits);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *fa_last_error(void);
+
+/* Library version, (major << 16) | minor. */
+int32_t fa_version(void);
+
+/* sizeof(fa_fwd_params) as the library was compiled: lets a foreign-language binding verify its
+ * mirror of the struct.  No counterpart in the reference (pybind11 passes tensors). */
+int32_t fa_sizeof_params(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA_MI355X_H */
