@@ -1,0 +1,167 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X FlashAttention forward path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu]
+
+One "step" is one forward pass over one synthetic batch already resident in HBM:
+  * prefill  -- flash_attn_func, bf16, batch 4, seqlen 8192, 32 heads, head dim 128, causal
+                (the configuration the headline metric is quoted on); value = TFLOP/s with the
+                reference's FLOP convention 4*b*s^2*h*d/2 (benchmarks/benchmark_flash_attention.py:27-30);
+  * decode   -- flash_attn_with_kvcache, bf16, batch 64, 1 new token appended with rotary, caches
+                (64, 32768, 8, 128), 64 query heads, cache_seqlens uniform in [1024, 32767];
+                reported as achieved HBM GB/s over the algorithmic bytes.
+Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
+attention_ref) timed on the host cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "flash-attention_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def _traffic(key):
+    """Measured HBM bytes per launch from the committed rocprofv3 --pmc summaries, if recorded."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall_ms / steps
+
+
+def bench_prefill(steps, warmup):
+    import torch
+    import flash_attn
+    b, s, h, d = 4, 8192, 32, 128
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+    fn = lambda: flash_attn.flash_attn_func(q, k, v, causal=True)
+    ms, wall_ms = time_steps(fn, steps, warmup)
+    flops = 4.0 * b * s * s * h * d / 2
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {
+        "ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"),
+                     "kernel": "prefill_kernel<bf16,128>", "flops_per_launch": flops},
+    }
+
+
+def bench_decode(steps, warmup):
+    import torch
+    import flash_attn
+    from oracle import attention_oracle as orc
+    b, cap, hk, h, d = 64, 32768, 8, 64, 128
+    torch.manual_seed(0)
+    k_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
+    v_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
+    q = torch.randn(b, 1, h, d, device="cuda", dtype=torch.bfloat16)
+    kn = torch.randn(b, 1, hk, d, device="cuda", dtype=torch.bfloat16)
+    vn = torch.randn(b, 1, hk, d, device="cuda", dtype=torch.bfloat16)
+    cache_seqlens = torch.randint(1024, cap, (b,), dtype=torch.int32).cuda()   # [1024, 32767]
+    cos, sin = orc.rotary_table(cap, d, dtype=torch.bfloat16)
+    cos, sin = cos.cuda(), sin.cuda()
+    fn = lambda: flash_attn.flash_attn_with_kvcache(q, k_cache, v_cache, kn, vn, cos, sin, cache_seqlens,
+                                                    causal=True, rotary_interleaved=True)
+    ms, wall_ms = time_steps(fn, steps, warmup)
+    keys = int((cache_seqlens.long() + 1).sum().item())
+    algo_bytes = keys * hk * d * 2 * 2 + 2 * b * h * d * 2 + 2 * b * hk * d * 2 * 2
+    gbs = algo_bytes / (ms * 1e-3) / 1e9
+    return {
+        "ms": ms, "wall_ms": wall_ms, "gb_per_s": gbs, "tokens_per_s": b / (ms * 1e-3),
+        "workload": "flash_attn_with_kvcache bf16 b64 cache(64,32768,8,128) hq64 append1+rotary128 causal",
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": gbs / PEAK_HBM_GBS, "traffic": _traffic("decode_bf16_d128_b64_32k"),
+                     "kernel": "append_kv + decode_kernel<bf16,128,split> + combine", "bytes_per_launch": algo_bytes},
+    }
+
+
+def cpu_baseline():
+    """Oracle on the host cores: 1 batch entry x 2 heads of the prefill workload (1/64 of the
+    (batch, head) pairs, which are independent), scaled to the whole batch."""
+    import torch
+    from oracle import attention_oracle as orc
+    b, s, h, d = 4, 8192, 32, 128
+    hs = 2
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(1, s, hs, d).to(torch.bfloat16) for _ in range(3))
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        orc.attention_forward(q, k, v, causal=True, head_block=1)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 8:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    flops_sample = 4.0 * 1 * s * s * hs * d / 2
+    return {"value": flops_sample / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "host_cpus": os.cpu_count(), "kind": "port",
+            "sample": "attention oracle (fp32 upcast) on 1 batch x %d heads of the prefill workload "
+                      "(%d repeats, %.2f s each); whole batch would take %.0f s" % (hs, reps, dt, dt * b * h / hs)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU only (the hot path uses no collectives); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    import flash_attn  # noqa: F401  fails loudly if the HIP library is missing
+
+    pre = bench_prefill(a.steps, a.warmup)
+    out = {
+        "metric": "fwd TFLOP/s (bf16, hdim128, causal, 8k)",
+        "value": pre["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": pre["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "flash_attn_func fwd bf16 batch=4 seqlen=8192 nheads=32 headdim=128 causal",
+                   "global_batch": 4, "seq_len": 8192},
+        "tokens_per_s": pre["tokens_per_s"],
+        "roofline": pre["roofline"],
+    }
+    if not a.no_decode:
+        dec = bench_decode(a.steps, a.warmup)
+        out["decode"] = dec
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
