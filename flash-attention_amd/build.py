@@ -41,15 +41,24 @@ def units():
     return u
 
 
+EXTRA = []
+
+
 def compile_one(args):
     src, obj, defs = args
-    cmd = [HIPCC] + FLAGS + defs + ["-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ_DIR, obj)]
+    cmd = [HIPCC] + FLAGS + EXTRA + defs + ["-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ_DIR, obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     return r.returncode, obj, err
 
 
-def build(jobs=None, verbose=True):
+def build(jobs=None, verbose=True, out=None, defines=(), obj_dir=None):
+    global OBJ_DIR, LIB
+    EXTRA[:] = ["-D" + d for d in defines]
+    if obj_dir:
+        OBJ_DIR = obj_dir
+    if out:
+        LIB = out
     os.makedirs(OBJ_DIR, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     us = units()
@@ -73,5 +82,8 @@ def build(jobs=None, verbose=True):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", type=int, default=None)
+    ap.add_argument("--out", default=None, help="write the library here instead of the package dir")
+    ap.add_argument("--obj-dir", default=None)
+    ap.add_argument("-D", dest="defines", action="append", default=[], help="extra preprocessor define")
     a = ap.parse_args()
-    build(a.j)
+    build(a.j, out=a.out, defines=a.defines, obj_dir=a.obj_dir)

@@ -25,6 +25,9 @@ int prefill_block_m(int db) { return 128 * (db == 64 ? PrefillTile<64>::RB : db 
 static int bucket(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
 static const int kNumCU = 256;   // MI355X
+#ifndef FA_DEC_SLOTS
+#define FA_DEC_SLOTS 8192
+#endif
 
 // The small-q streaming kernel packs seqlen_q x (h / h_k) rows into 16 MFMA columns.
 static bool use_decode_kernel(const fa_fwd_params& p) {
@@ -57,10 +60,11 @@ static int plan(const fa_fwd_params& p, bool allow_split, int* split_len_out) {
             splits = p.num_splits;
         } else if (p.num_splits == 0) {
             if (dec) {
-                // ~16k chunk slots over the whole launch, chunks of at least 256 keys: enough
-                // workgroups to balance ragged cache lengths over 256 CUs x 2 resident groups.
+                // ~8k chunk slots over the whole launch (16 per resident workgroup), chunks of at
+                // least 256 keys: measured best trade between per-workgroup start-up cost and
+                // the tail left by ragged cache lengths on 256 CUs x 2 resident groups.
                 const int64_t streams = (int64_t)p.b * p.h_k;
-                int64_t len = rup(std::max<int64_t>(256, (int64_t)sk * streams / 16384), 128);
+                int64_t len = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS), 128);
                 splits = (int)((sk + len - 1) / len);
             } else {
                 const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;

@@ -47,7 +47,9 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int m = lane & 15, g4 = lane >> 4;     // MFMA column (packed query row), lane group
-    const int split = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    // kv heads vary fastest over the grid: the h_k workgroups that share the rows of one
+    // (batch, chunk) of a (b, s, h_k, d) cache run together and consume whole cache rows.
+    const int hk = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
     const int G = p.h / p.h_k;
     const int rows = p.seqlen_q * G;             // packed rows in use (<= 16)
 
@@ -119,25 +121,27 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
     char* vb = kb + C::TILE_BYTES;
 
     u32x4 kr[C::LD], vr[C::LD];
+    // unconditional loads (clamped into range), zeroed on the way into LDS
+    const int d_last_chunk = p.d / 8 - 1;
     auto load_step = [&](int n0) {
 #pragma unroll
         for (int i = 0; i < C::LD; i++) {
             const int f = lane + i * 64;
-            const int row = f / C::CPR, c = f % C::CPR;
-            const int n = n0 + row;
-            const bool ok = (n < w_hi) && (c * 8 < p.d);
-            u32x4 z = {0, 0, 0, 0};
-            kr[i] = ok ? ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8) : z;
-            vr[i] = ok ? ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8) : z;
+            const int row = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
+            const int n = min(n0 + row, w_hi - 1);
+            kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
+            vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
         }
     };
-    auto store_step = [&]() {
+    auto store_step = [&](int n0) {
 #pragma unroll
         for (int i = 0; i < C::LD; i++) {
             const int f = lane + i * 64;
             const int row = f / C::CPR, c = f % C::CPR;
-            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = kr[i];
-            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_vd<D>(c, row) * 16) = vr[i];
+            const bool ok = (n0 + row < w_hi) && (c <= d_last_chunk);
+            const u32x4 z = {0, 0, 0, 0};
+            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = ok ? kr[i] : z;
+            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_vd<D>(c, row) * 16) = ok ? vr[i] : z;
         }
     };
 
@@ -157,7 +161,7 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
         // the previous step's LDS reads are complete (their results were consumed) before these
         // writes are issued; LDS operations of one wave execute in order.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        store_step();
+        store_step(n0);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -294,7 +298,7 @@ template <typename T, int D>
 static int launch_decode_t(const KParams& kp, hipStream_t stream) {
     typedef DecodeCfg<T, D> C;
     const bool split = kp.num_splits > 1;
-    dim3 grid(split ? kp.num_splits : 1, kp.p.h_k, kp.p.b), block(C::kThreads);
+    dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b), block(C::kThreads);
     hipError_t e;
     if (split) {
         auto kern = decode_kernel<T, D, true>;

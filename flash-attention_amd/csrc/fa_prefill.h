@@ -127,28 +127,32 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
 
     // ---- tile movers
     u32x4 kr[C::LOADS], vr[C::LOADS];
+    // Loads are unconditional (row / column clamped into range) so that they stay in flight across
+    // the tile's compute; out-of-range rows and columns are zeroed when the tile is written to LDS.
+    const int d_last_chunk = p.d / 8 - 1;
     auto load_tile = [&](int t) {
         const int n0 = t * BN;
 #pragma unroll
         for (int i = 0; i < C::LOADS; i++) {
             const int f = tid + i * C::kThreads;
-            const int row = f / C::CPR, c = f % C::CPR;
-            const int n = n0 + row;
-            const bool ok = (n < si.sk) && (c * 8 < p.d);
-            u32x4 z = {0, 0, 0, 0};
-            kr[i] = ok ? ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8) : z;
-            vr[i] = ok ? ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8) : z;
+            const int row = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
+            const int n = min(n0 + row, si.sk - 1);
+            kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
+            vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
         }
     };
-    auto store_tile = [&](int buf) {
+    auto store_tile = [&](int buf, int t) {
         char* kb = smem + buf * 2 * C::TILE_BYTES;
         char* vb = kb + C::TILE_BYTES;
+        const int n0 = t * BN;
 #pragma unroll
         for (int i = 0; i < C::LOADS; i++) {
             const int f = tid + i * C::kThreads;
             const int row = f / C::CPR, c = f % C::CPR;
-            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = kr[i];
-            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_v<D>(c, row) * 16) = vr[i];
+            const bool ok = (n0 + row < si.sk) && (c <= d_last_chunk);
+            const u32x4 z = {0, 0, 0, 0};
+            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = ok ? kr[i] : z;
+            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_v<D>(c, row) * 16) = ok ? vr[i] : z;
         }
     };
 
@@ -160,7 +164,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
 
     if (t_hi > t_lo) {
         load_tile(t_hi - 1);
-        store_tile(0);
+        store_tile(0, t_hi - 1);
     }
     __syncthreads();
     int buf = 0;
@@ -284,7 +288,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
             }
         }
 
-        if (has_next) store_tile(buf ^ 1);
+        if (has_next) store_tile(buf ^ 1, t - 1);
         __syncthreads();
         buf ^= 1;
     }

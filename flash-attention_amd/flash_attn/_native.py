@@ -18,7 +18,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libfa_mi355x.so")
+# FLASH_ATTN_MI355X_LIB selects another build of the same library (kernel tuning experiments).
+_LIB_PATH = os.environ.get("FLASH_ATTN_MI355X_LIB") or os.path.join(_HERE, "libfa_mi355x.so")
 
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
