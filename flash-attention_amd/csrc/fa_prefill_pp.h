@@ -1,0 +1,386 @@
+// "Ping-pong" variant of the tiled forward kernel for long query sequences on gfx950.
+//
+// Same mathematics and register layouts as prefill_kernel (fa_prefill.h): S^T = K Q^T and
+// O^T = V^T P^T on v_mfma_f32_32x32x16 with one query row per lane.  What changes is how the
+// execution pipes of a SIMD are kept busy.  A CDNA4 SIMD issues matrix (MFMA) and vector (VALU)
+// instructions from different waves at the same time, and for head dim 128 the exp2/max/sum work
+// of a key tile costs about as many cycles as its two matrix products.  So:
+//
+//  * a workgroup is 8 waves = two groups of 4; waves w and w+4 sit on the same SIMD;
+//  * every wave alternates a VALU phase Y(i) (mask + online softmax of tile i) and an MFMA phase
+//    X(i) (O += P_i V_i, then S = K_{i+1} Q), separated by workgroup barriers;
+//  * group 1 runs one phase behind group 0 (it takes one extra barrier up front, group 0 one extra
+//    at the end), so at any time one wave of each SIMD is in its MFMA phase and the other in its
+//    VALU phase.
+//
+// K and V tiles are shared by all 8 waves (256 query rows per workgroup) and move from global
+// memory straight into LDS with global_load_lds_dwordx4 (no staging registers, no ds_write):
+// each wave instruction deposits 64 x 16 B contiguously in LDS, so the bank-conflict-avoiding XOR
+// swizzle is applied on the global side (lane -> which 16 B chunk of which row it fetches).  A ring
+// of 4 tile slots per tensor is filled 3 tiles ahead; the barrier pattern guarantees that a slot is
+// refilled only after both groups have passed the phase that read it, and each wave waits for its
+// own outstanding fills (vmcnt) before the barrier that publishes them.
+//
+// The running max is updated lazily: a row's reference max moves only when the new max exceeds it
+// by more than 2^8 in the exp2 domain, which makes the O rescale rare after the first tiles while
+// keeping every probability <= 256 (exact in the final normalisation, safe in fp16/bf16).
+#pragma once
+#include "fa_common.h"
+
+namespace fa {
+
+#ifndef FA_PP_LA
+#define FA_PP_LA 4
+#endif
+
+template <typename T, int D, int BN>
+struct PPCfg {
+    static constexpr int kThreads = 512;
+    static constexpr int kWaves = 8;
+    static constexpr int BM = kWaves * 32;
+    static constexpr int NB = BN / 32;
+    static constexpr int KS = D / 16;
+    static constexpr int DB = D / 32;
+    static constexpr int PT = BN / 16;
+    static constexpr int CPR = D / 8;                       // 16 B chunks per tile row
+    static constexpr int ROWB = D * 2;
+    static constexpr int TILE = BN * ROWB;                  // bytes of one K or V tile
+    static constexpr int NS = 4;                            // ring slots per tensor
+    static constexpr int PF = NS - 1;                       // tiles of look-ahead
+    static constexpr int LOADS = BN * CPR / kThreads;       // 16 B fills per thread per tile
+    static constexpr int ROWS_PER_PASS = kThreads / CPR;
+    static constexpr int SMEM = 2 * NS * TILE;              // K ring, then V ring
+    static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
+};
+
+// 16 B from global memory to LDS address m0_base + lane * 16, bypassing registers.
+FA_DEV void async_fill16(const void* gptr, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :: "s"(lds_base_uniform), "v"(gptr) : "memory", "m0");
+}
+// wait until at most N of this wave's vector-memory operations are outstanding (N < 16)
+template <int N> FA_DEV void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));
+}
+
+template <typename T, int D, int BN>
+__global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
+    typedef PPCfg<T, D, BN> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_fwd_params& p = kp.p;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int group = wave >> 2;
+
+    const int G = p.h / p.h_k;
+    const int64_t total = (int64_t)kp.num_m_blocks * p.h * p.b;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int g = (int)(w % G); w /= G;
+    const int mb = kp.num_m_blocks - 1 - (int)(w % kp.num_m_blocks); w /= kp.num_m_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+    const int head = hk * G + g;
+
+    const SeqInfo si = seq_info(p, b);
+    const int m0 = mb * C::BM;
+    if (m0 >= si.sq) return;
+
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    int n_hi = si.sk;
+    if (has_right) n_hi = min(n_hi, min(m0 + C::BM, si.sq) + shift + wr);
+    int n_lo = 0;
+    if (has_left) n_lo = max(0, m0 + shift - wl);
+    const int t_lo = n_lo / BN;
+    const int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
+    const int nt = max(0, t_hi - t_lo);           // tiles visited, the same for all 8 waves
+
+    const T* __restrict__ qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
+    const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
+    const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
+
+    const int r0 = m0 + wave * 32;                // first query row of this wave
+    const int row = r0 + l32;
+
+    v8 qf[C::KS];
+    {
+        const bool valid = row < si.sq;
+        const T* qrow = qg + (int64_t)row * p.q_row_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 raw = {0, 0, 0, 0};
+            if (valid && d0 < p.d) raw = ld_global16(qrow + d0);
+            qf[dk] = __builtin_bit_cast(v8, raw);
+        }
+    }
+
+    f32x16 o_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const float sl2 = kp.scale_log2;
+
+    // tiles are visited from the last key tile down to the first; tile i of the visit is key tile
+    // t_hi - 1 - i and lives in ring slot i % NS
+    auto tile_of = [&](int i) { return t_hi - 1 - i; };
+
+    // ---- asynchronous tile fills.  Pass j of wave w fills LDS positions [(w + 8j) * 64, +64) of the
+    // tile (16 B each); position p is tile row p / CPR, stored chunk p % CPR, and holds global chunk
+    // (p % CPR) ^ swizzle(row).
+    const int frow = (wave * 64 + lane) / C::CPR;              // tile row of pass 0
+    const int fch = lane % C::CPR;
+    const int kch = min(swz_k<D>(fch, frow), p.d / 8 - 1);     // clamped: columns >= d are never used
+    const int vch = min(swz_v<D>(fch, frow), p.d / 8 - 1);
+    const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
+    const uint32_t fill_base = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(wave * 1024));
+    const int64_t kstep = (int64_t)BN * p.k_row_stride, vstep = (int64_t)BN * p.v_row_stride;
+    const int64_t kpass = (int64_t)C::ROWS_PER_PASS * p.k_row_stride, vpass = (int64_t)C::ROWS_PER_PASS * p.v_row_stride;
+    // running pointers: tile (visit index) next to be requested
+    const T* kptr = kg + (int64_t)((t_hi - 1) * BN + frow) * p.k_row_stride + kch * 8;
+    const T* vptr = vg + (int64_t)((t_hi - 1) * BN + frow) * p.v_row_stride + vch * 8;
+    const bool has_tail = t_hi * BN > si.sk;       // only visit 0 can reach past seqlen_k: clamp its rows
+    auto fill_k = [&](int i) {
+        const uint32_t dst = fill_base + (uint32_t)((i & (C::NS - 1)) * C::TILE);
+        if (i == 0 && has_tail) {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) {
+                const int n = min((t_hi - 1) * BN + frow + j * C::ROWS_PER_PASS, si.sk - 1);
+                async_fill16(kg + (int64_t)n * p.k_row_stride + kch * 8, dst + j * 8192);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) async_fill16(kptr + j * kpass, dst + j * 8192);
+        }
+        kptr -= kstep;
+    };
+    auto fill_v = [&](int i) {
+        const uint32_t dst = fill_base + (uint32_t)((C::NS + (i & (C::NS - 1))) * C::TILE);
+        if (i == 0 && has_tail) {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) {
+                const int n = min((t_hi - 1) * BN + frow + j * C::ROWS_PER_PASS, si.sk - 1);
+                async_fill16(vg + (int64_t)n * p.v_row_stride + vch * 8, dst + j * 8192);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) async_fill16(vptr + j * vpass, dst + j * 8192);
+        }
+        vptr -= vstep;
+    };
+
+    // Per-wave tile classes, as ranges of the absolute key-tile index t: the wave has visible keys
+    // in tiles [ta_lo, ta_hi]; tiles in [tf_lo, tf_hi] are fully visible to all 32 rows (no masking).
+    int ta_lo = t_lo, ta_hi = t_hi - 1, tf_lo = 0, tf_hi = si.sk / BN - 1;
+    if (has_right) {
+        const int c = r0 + shift + wr;            // last visible key of the wave's first row
+        ta_hi = min(ta_hi, (c + 31 >= 0) ? (c + 31) / BN : -1);
+        tf_hi = min(tf_hi, (c + 1 >= BN) ? (c + 1) / BN - 1 : -1);
+    }
+    if (has_left) {
+        const int c = r0 + shift - wl;            // first visible key of the wave's first row
+        ta_lo = max(ta_lo, (c > 0) ? c / BN : 0);
+        tf_lo = (c + 31 > 0) ? (c + 31 + BN - 1) / BN : 0;
+    }
+    if (r0 >= si.sq) ta_hi = ta_lo - 1;
+    auto active = [&](int i) -> bool { const int t = tile_of(i); return t >= ta_lo && t <= ta_hi; };
+
+    // ---- S^T = K Q^T.  Fragment reads run LA matrix instructions ahead of their use and are
+    // interleaved one-for-one with the MFMAs.
+    int kofs[C::KS];
+#pragma unroll
+    for (int dk = 0; dk < C::KS; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dk * 2 + hh, l32) * 16;
+    f32x16 s_acc[C::NB];
+    auto qk = [&](int i) {
+        const char* kb = smem + (i & (C::NS - 1)) * C::TILE;
+        constexpr int NF = C::NB * C::KS;          // fragments in (nb, dk) order
+        constexpr int LA = FA_PP_LA;
+        auto frag_ptr = [&](int f) { return kb + (f / C::KS) * 32 * C::ROWB + kofs[f % C::KS]; };
+        u32x4 fr[LA];
+#pragma unroll
+        for (int e = 0; e < LA; e++) fr[e] = *reinterpret_cast<const u32x4*>(frag_ptr(e));
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s_acc[nb][r] = 0.f;
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            s_acc[f / C::KS] = Elem<T>::mfma32(__builtin_bit_cast(v8, fr[f % LA]), qf[f % C::KS], s_acc[f / C::KS]);
+            if (f + LA < NF) fr[f % LA] = *reinterpret_cast<const u32x4*>(frag_ptr(f + LA));
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, LA, 0);      // look-ahead reads
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+            if (f + LA < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 DS read
+        }
+    };
+
+    // ---- O^T += V^T P^T, same interleave with two transposing reads per MFMA
+    const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
+    int vofs[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+        vofs[db] = (4 * hh + tj) * C::ROWB + swz_v<D>(db * 4 + dhalf * 2 + (tq >> 1), 4 * hh + tj) * 16 + (tq & 1) * 8;
+    v8 pf[C::PT];
+    auto pv = [&](int i) {
+        const char* vb = smem + (C::NS + (i & (C::NS - 1))) * C::TILE;
+        constexpr int NF = C::PT * C::DB;          // fragments in (t16, db) order
+        constexpr int LA = FA_PP_LA;
+        auto fetch = [&](int f) {
+            const int t16 = f / C::DB, db = f % C::DB;
+            const u32x2 lo = lds_read_tr16(vb + t16 * 16 * C::ROWB + vofs[db]);
+            const u32x2 hi = lds_read_tr16(vb + (t16 * 16 + 8) * C::ROWB + vofs[db]);
+            return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+        };
+        u32x4 fr[LA];
+#pragma unroll
+        for (int e = 0; e < LA; e++) fr[e] = fetch(e);
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            o_acc[f % C::DB] = Elem<T>::mfma32(__builtin_bit_cast(v8, fr[f % LA]), pf[f / C::DB], o_acc[f % C::DB]);
+            if (f + LA < NF) fr[f % LA] = fetch(f + LA);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * LA, 0);  // look-ahead reads
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+            if (f + LA < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 DS reads
+        }
+    };
+
+    auto softmax = [&](int i) {
+        const int tt = tile_of(i);
+        if (tt < tf_lo || tt > tf_hi) {
+            const int n0 = tt * BN;
+            int lim_hi = si.sk - 1;
+            if (has_right) lim_hi = min(lim_hi, row + shift + wr);
+            const int lim_lo = has_left ? row + shift - wl : 0;
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                    if (n > lim_hi || n < lim_lo) s_acc[nb][r] = -INFINITY;
+                }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s_acc[nb][r]);
+        mx = xhalf_max(mx);
+        // lazy reference max: move it only when the tile max exceeds it by more than 2^8 (exp2 domain)
+        const bool move = (mx - m_run) * sl2 > 8.f;       // false for NaN (-inf - -inf)
+        if (__builtin_amdgcn_ballot_w64(move) != 0) {
+            const float m_new = move ? mx : m_run;
+            const float corr = move ? fast_exp2((m_run - m_new) * sl2) : 1.f;   // m_run = -inf -> 0
+            l_run *= corr;
+#pragma unroll
+            for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
+            m_run = m_new;
+        }
+        const float msc = (m_run == -INFINITY) ? 0.f : m_run * sl2;
+        float suma = 0.f, sumb = 0.f;
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float e0 = fast_exp2(s_acc[nb][r] * sl2 - msc);
+                const float e1 = fast_exp2(s_acc[nb][r + 1] * sl2 - msc);
+                s_acc[nb][r] = e0;
+                s_acc[nb][r + 1] = e1;
+                suma += e0;
+                sumb += e1;
+            }
+        l_run += suma + sumb;
+#pragma unroll
+        for (int t16 = 0; t16 < C::PT; t16++) {
+            const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
+            u32x4 pk;
+#pragma unroll
+            for (int e = 0; e < 4; e++) pk[e] = pack2<T>(s_acc[nb][r8 + 2 * e], s_acc[nb][r8 + 2 * e + 1]);
+            pf[t16] = __builtin_bit_cast(v8, pk);
+        }
+    };
+
+    if (nt > 0) {
+        // ---- prologue: request K(0), V(0), K(1), V(1), K(2); S = K(0) Q
+        fill_k(0);
+        fill_v(0);
+        if (nt > 1) { fill_k(1); fill_v(1); }
+        if (nt > 2) fill_k(2);
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (active(0)) qk(0);
+        if (group == 1) __syncthreads();   // group 1 runs one phase behind group 0
+
+        for (int i = 0; i < nt; i++) {
+            // ---- Y(i): VALU phase (and requests for the tiles needed 3 iterations ahead)
+            if (i + C::PF < nt) fill_k(i + C::PF);
+            if (i + C::PF - 1 < nt) fill_v(i + C::PF - 1);
+            const bool act = active(i);
+            if (act) softmax(i);
+            __syncthreads();
+            // ---- X(i): MFMA phase
+            __builtin_amdgcn_s_setprio(1);
+            if (act) pv(i);
+            if (i + 1 < nt && active(i + 1)) qk(i + 1);
+            __builtin_amdgcn_s_setprio(0);
+            // this wave's fills of K(i+2), V(i+1) must have landed before the barrier publishes them;
+            // the 2 * LOADS requests of Y(i) may stay in flight
+            if (i + C::PF < nt) wait_vmcnt<2 * C::LOADS>(); else wait_vmcnt<0>();
+            __syncthreads();
+        }
+        if (group == 0) __syncthreads();
+    }
+
+    // ---- epilogue
+    const float l_tot = xhalf_sum(l_run);
+    const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
+    const float inv = dead ? 1.f : 1.f / l_tot;
+    const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
+    if (row < si.sq) {
+        if (hh == 0) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
+        T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)row * p.o_row_stride + (int64_t)head * p.o_head_stride;
+#pragma unroll
+        for (int db = 0; db < C::DB; db++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int d0 = db * 32 + 8 * q4 + 4 * hh;
+                if (d0 < p.d) {
+                    u32x2 v = {pack2<T>(o_acc[db][4 * q4] * inv, o_acc[db][4 * q4 + 1] * inv),
+                               pack2<T>(o_acc[db][4 * q4 + 2] * inv, o_acc[db][4 * q4 + 3] * inv)};
+                    st_global8(orow + d0, v);
+                }
+            }
+    }
+}
+
+template <typename T, int D, int BN>
+int launch_prefill_pp(KParams kp, hipStream_t stream) {
+    typedef PPCfg<T, D, BN> C;
+    kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
+    const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
+    auto kern = prefill_pp_kernel<T, D, BN>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fa
