@@ -108,7 +108,7 @@ def cpu_baseline():
     import torch
     from oracle import attention_oracle as orc
     b, s, h, d = 4, 8192, 32, 128
-    hs = 2
+    hs = 4
     torch.manual_seed(0)
     q, k, v = (torch.randn(1, s, hs, d).to(torch.bfloat16) for _ in range(3))
     t0 = time.perf_counter()
@@ -116,7 +116,7 @@ def cpu_baseline():
     while True:
         orc.attention_forward(q, k, v, causal=True, head_block=1)
         reps += 1
-        if time.perf_counter() - t0 > 10.0 or reps >= 8:
+        if time.perf_counter() - t0 > 12.0 or reps >= 64:
             break
     dt = (time.perf_counter() - t0) / reps
     flops_sample = 4.0 * 1 * s * s * hs * d / 2
@@ -133,6 +133,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
+                         "FETCH_SIZE / WRITE_SIZE can be scaled against a kernel of known traffic")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path uses no collectives); "
@@ -144,6 +147,13 @@ def main():
         sys.exit(1)
     import flash_attn  # noqa: F401  fails loudly if the HIP library is missing
 
+    if a.calibrate_copy:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     pre = bench_prefill(a.steps, a.warmup)
     out = {
         "metric": "fwd TFLOP/s (bf16, hdim128, causal, 8k)",

@@ -1,0 +1,156 @@
+"""The five benchmark configurations at their full sizes on the GPU.
+
+The whole problem runs through the public API; the CPU oracle then checks a seeded SAMPLE of
+(batch, head) pairs / sequences / cache rows (the units are independent, and the full score tensors
+would be tens of GB), under the reference's tolerance rule (tests/test_flash_attn.py:648-650) with
+log-sum-exp within 1e-3 relative.  Size-independent properties (bit-repeatability, split-count
+invariance, appended cache rows) are checked on the whole output."""
+import math
+import sys
+
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _fa():
+    import flash_attn
+    return flash_attn
+
+
+def _check_heads(out, lse, q, k, v, pairs, group, mult=2.0, **kw):
+    """Compare (batch, q-head) pairs against the oracle; k/v heads follow the GQA mapping."""
+    for (b, h) in pairs:
+        qs = q[b:b + 1, :, h:h + 1].cpu()
+        ks = k[b:b + 1, :, h // group:h // group + 1].cpu()
+        vs = v[b:b + 1, :, h // group:h // group + 1].cpu()
+        o_ref, l_ref, o_pt = orc.attention_reference_pair(qs, ks, vs, **kw)
+        ok, err, bound = orc.tolerance_ok(out[b:b + 1, :, h:h + 1].cpu(), o_ref, o_pt, mult, 1e-5)
+        _say("   (b=%d,h=%d) out err %.3e bound %.3e" % (b, h, err, bound))
+        assert ok, (b, h, err, bound)
+        if lse is not None:
+            okl, rel = orc.lse_ok(lse[b:b + 1, h:h + 1].cpu(), l_ref)
+            assert okl, (b, h, rel)
+
+
+def test_config2_bf16_causal_8k():
+    """bf16, batch 4, seqlen 8192, 32 heads, head dim 128, causal, scale 1/sqrt(128); out + lse."""
+    _say("config2")
+    torch.manual_seed(0)
+    b, s, h, d = 4, 8192, 32, 128
+    q, k, v = (torch.randn(b, s, h, d, device=DEV, dtype=torch.bfloat16) for _ in range(3))
+    fa = _fa()
+    out, lse, _ = fa.flash_attn_func(q, k, v, softmax_scale=1 / math.sqrt(128), causal=True, return_attn_probs=True)
+    assert not torch.isnan(out).any() and torch.isfinite(lse).all()
+    _check_heads(out, lse, q, k, v, [(0, 0), (3, 31), (1, 17)], 1, causal=True, softmax_scale=1 / math.sqrt(128))
+    out2, lse2, _ = fa.flash_attn_func(q, k, v, softmax_scale=1 / math.sqrt(128), causal=True, return_attn_probs=True)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+    # first row of every (batch, head) sees exactly one key: out = v[0], lse = scale * q0.k0
+    assert torch.equal(out[:, 0], v[:, 0])
+    s00 = (q[:, 0].float() * k[:, 0].float()).sum(-1) / math.sqrt(128)
+    assert torch.allclose(lse[:, :, 0], s00, rtol=1e-3, atol=1e-3)
+
+
+def test_config2_dense_matches_qkvpacked():
+    _say("config2 dense / qkvpacked")
+    torch.manual_seed(1)
+    b, s, h, d = 2, 4096, 16, 128
+    qkv = torch.randn(b, s, 3, h, d, device=DEV, dtype=torch.bfloat16)
+    fa = _fa()
+    o1 = fa.flash_attn_qkvpacked_func(qkv)
+    o2 = fa.flash_attn_func(qkv[:, :, 0].contiguous(), qkv[:, :, 1].contiguous(), qkv[:, :, 2].contiguous())
+    assert torch.equal(o1, o2)
+    _check_heads(o1, None, qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], [(1, 5)], 1)
+
+
+def test_config3_gqa_sliding_window_16k():
+    """bf16, batch 2, seqlen 16384, 32 q heads / 8 kv heads, head dim 128, causal, window (4096, 0)."""
+    _say("config3")
+    torch.manual_seed(0)
+    b, s, h, hk, d = 2, 16384, 32, 8, 128
+    q = torch.randn(b, s, h, d, device=DEV, dtype=torch.bfloat16)
+    k = torch.randn(b, s, hk, d, device=DEV, dtype=torch.bfloat16)
+    v = torch.randn(b, s, hk, d, device=DEV, dtype=torch.bfloat16)
+    out, lse, _ = _fa().flash_attn_func(q, k, v, causal=True, window_size=(4096, 0), return_attn_probs=True)
+    assert not torch.isnan(out).any()
+    _check_heads(out, lse, q, k, v, [(0, 3), (1, 30)], h // hk, causal=True, window_size=(4096, 0))
+
+
+@pytest.mark.parametrize("d", [128, 256])
+def test_config4_varlen_64_sequences(d):
+    """bf16, 64 packed sequences with lengths uniform in [128, 4096], 16 heads, causal."""
+    _say("config4", d)
+    torch.manual_seed(0)
+    h = 16
+    lens = torch.randint(128, 4097, (64,))
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).int()
+    total, mx = int(cu[-1]), int(lens.max())
+    q, k, v = (torch.randn(total, h, d, device=DEV, dtype=torch.bfloat16) for _ in range(3))
+    cu_d = cu.to(DEV)
+    out, lse, _ = _fa().flash_attn_varlen_func(q, k, v, cu_d, cu_d, mx, mx, causal=True, return_attn_probs=True)
+    assert out.shape == q.shape and lse.shape == (64, h, mx)
+    assert not torch.isnan(out).any()
+    order = torch.argsort(lens)
+    for i in (int(order[0]), int(order[31]), int(order[-1]), 7):     # shortest, median, longest, one more
+        a, e = int(cu[i]), int(cu[i + 1])
+        for hh in (0, 11):
+            qs, ks, vs = (t[a:e, hh:hh + 1][None].cpu() for t in (q, k, v))
+            o_ref, l_ref, o_pt = orc.attention_reference_pair(qs, ks, vs, causal=True)
+            ok, err, bound = orc.tolerance_ok(out[a:e, hh:hh + 1][None].cpu(), o_ref, o_pt, 2.0, 1e-5)
+            _say("   seq %d (len %d) head %d: err %.3e bound %.3e" % (i, e - a, hh, err, bound))
+            assert ok
+            assert orc.lse_ok(lse[i, hh:hh + 1, : e - a][None].cpu(), l_ref)[0]
+
+
+def test_config5_decode_kvcache_rotary():
+    """bf16 decode: batch 64, caches (64, 32768, 8, 128), 64 q heads (GQA 8:1), one new token
+    appended with rotary (dim 128, base 10000, interleaved), cache_seqlens uniform in [1024, 32767]."""
+    _say("config5")
+    torch.manual_seed(0)
+    b, cap, hk, h, d = 64, 32768, 8, 64, 128
+    kc = torch.randn(b, cap, hk, d, device=DEV, dtype=torch.bfloat16)
+    vc = torch.randn(b, cap, hk, d, device=DEV, dtype=torch.bfloat16)
+    q = torch.randn(b, 1, h, d, device=DEV, dtype=torch.bfloat16)
+    kn = torch.randn(b, 1, hk, d, device=DEV, dtype=torch.bfloat16)
+    vn = torch.randn(b, 1, hk, d, device=DEV, dtype=torch.bfloat16)
+    lens = torch.randint(1024, cap, (b,), dtype=torch.int32)
+    lens[0], lens[1] = 1024, cap - 1
+    cos, sin = orc.rotary_table(cap, d, dtype=torch.bfloat16)
+    sample = [0, 1, 17, 63]
+    before_k = {i: kc[i, : int(lens[i]) + 2].cpu() for i in sample}
+    before_v = {i: vc[i, : int(lens[i]) + 2].cpu() for i in sample}
+    lens_d = lens.to(DEV)
+    fa = _fa()
+    out = fa.flash_attn_with_kvcache(q, kc, vc, kn, vn, cos.to(DEV), sin.to(DEV), lens_d, causal=True,
+                                     rotary_interleaved=True)
+    assert not torch.isnan(out).any()
+    for i in sample:
+        L = int(lens[i])
+        o_ref, _, k_ref, v_ref = orc.kvcache_forward(q[i:i + 1].cpu(), before_k[i][None], before_v[i][None],
+                                                     kn[i:i + 1].cpu(), vn[i:i + 1].cpu(), cos, sin,
+                                                     torch.tensor([L], dtype=torch.int32), causal=True)
+        o_pt, _, _, _ = orc.kvcache_forward(q[i:i + 1].cpu(), before_k[i][None], before_v[i][None],
+                                            kn[i:i + 1].cpu(), vn[i:i + 1].cpu(), cos, sin,
+                                            torch.tensor([L], dtype=torch.int32), causal=True, upcast=False,
+                                            reorder_ops=True)
+        ok, err, bound = orc.tolerance_ok(out[i:i + 1].cpu(), o_ref, o_pt, 3.0, 1e-5)
+        _say("   batch %d (len %d): err %.3e bound %.3e" % (i, L, err, bound))
+        assert ok
+        assert torch.equal(vc[i, : L + 2].cpu(), v_ref[0])                       # V rows bit-exact
+        assert torch.allclose(kc[i, : L + 2].cpu().float(), k_ref[0].float(), rtol=1e-3, atol=1e-3)
+    # the appended V row of EVERY batch entry is the new value, bit for bit
+    rows = vc[torch.arange(b, device=DEV), lens_d.long()]
+    assert torch.equal(rows, vn[:, 0])
+    # split-count invariance on the whole output (cache already holds the appended token: no k/v now)
+    lens1 = lens_d + 1
+    outs = [fa.flash_attn_with_kvcache(q, kc, vc, cache_seqlens=lens1, num_splits=n).float() for n in (0, 1, 5)]
+    assert (outs[0] - outs[1]).abs().max().item() < 2e-2 and (outs[0] - outs[2]).abs().max().item() < 2e-2
