@@ -129,9 +129,14 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     float m_run = -INFINITY, l_run = 0.f;
     const float sl2 = kp.scale_log2;
 
-    // tiles are visited from the last key tile down to the first; tile i of the visit is key tile
-    // t_hi - 1 - i and lives in ring slot i % NS
+    // visit i of the key loop handles key tile tile_of(i) and uses ring slot i % NS
+#ifdef FA_PP_ASCENDING
+    constexpr int kDir = 1;
+    auto tile_of = [&](int i) { return t_lo + i; };
+#else
+    constexpr int kDir = -1;
     auto tile_of = [&](int i) { return t_hi - 1 - i; };
+#endif
 
     // ---- asynchronous tile fills.  Pass j of wave w fills LDS positions [(w + 8j) * 64, +64) of the
     // tile (16 B each); position p is tile row p / CPR, stored chunk p % CPR, and holds global chunk
@@ -145,12 +150,14 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const int64_t kstep = (int64_t)BN * p.k_row_stride, vstep = (int64_t)BN * p.v_row_stride;
     const int64_t kpass = (int64_t)C::ROWS_PER_PASS * p.k_row_stride, vpass = (int64_t)C::ROWS_PER_PASS * p.v_row_stride;
     // running pointers: tile (visit index) next to be requested
-    const T* kptr = kg + (int64_t)((t_hi - 1) * BN + frow) * p.k_row_stride + kch * 8;
-    const T* vptr = vg + (int64_t)((t_hi - 1) * BN + frow) * p.v_row_stride + vch * 8;
-    const bool has_tail = t_hi * BN > si.sk;       // only visit 0 can reach past seqlen_k: clamp its rows
+    const int t_first = kDir > 0 ? t_lo : t_hi - 1;
+    const T* kptr = kg + (int64_t)(t_first * BN + frow) * p.k_row_stride + kch * 8;
+    const T* vptr = vg + (int64_t)(t_first * BN + frow) * p.v_row_stride + vch * 8;
+    // only key tile t_hi - 1 can reach past seqlen_k: its rows are clamped
+    const int i_tail = (t_hi * BN > si.sk) ? (kDir > 0 ? nt - 1 : 0) : -1;
     auto fill_k = [&](int i) {
         const uint32_t dst = fill_base + (uint32_t)((i & (C::NS - 1)) * C::TILE);
-        if (i == 0 && has_tail) {
+        if (i == i_tail) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) {
                 const int n = min((t_hi - 1) * BN + frow + j * C::ROWS_PER_PASS, si.sk - 1);
@@ -160,11 +167,11 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) async_fill16(kptr + j * kpass, dst + j * 8192);
         }
-        kptr -= kstep;
+        kptr += kDir * kstep;
     };
     auto fill_v = [&](int i) {
         const uint32_t dst = fill_base + (uint32_t)((C::NS + (i & (C::NS - 1))) * C::TILE);
-        if (i == 0 && has_tail) {
+        if (i == i_tail) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) {
                 const int n = min((t_hi - 1) * BN + frow + j * C::ROWS_PER_PASS, si.sk - 1);
@@ -174,7 +181,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) async_fill16(vptr + j * vpass, dst + j * 8192);
         }
-        vptr -= vstep;
+        vptr += kDir * vstep;
     };
 
     // Per-wave tile classes, as ranges of the absolute key-tile index t: the wave has visible keys
