@@ -47,18 +47,28 @@ static int check_common(const fa_fwd_params* p) {
     return 0;
 }
 
-// Split planning for 256 CUs.  Returns the chunk count; *split_len receives the chunk length.
-static int plan(const fa_fwd_params& p, bool allow_split, int* split_len_out) {
+// Split planning for 256 CUs.
+struct SplitPlan {
+    int splits = 1;        // partial slots (what the caller allocates)
+    int len = 0;           // keys per chunk
+    int persistent = 0;    // ticket-scheduled decode kernel
+    int sa = 0, sb = 0, sub = 0;
+};
+
+static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
+    SplitPlan r;
     const int sk = p.seqlen_k;
     const int db = bucket(p.d);
     const bool dec = use_decode_kernel(p);
     const int gran = dec ? 128 : prefill_block_n(db);
     auto rup = [](int64_t x, int64_t m) { return (int)((x + m - 1) / m * m); };
     int splits = 1;
+    bool automatic = false;
     if (allow_split && sk > 0) {
         if (p.num_splits > 1) {
             splits = p.num_splits;
         } else if (p.num_splits == 0) {
+            automatic = true;
             if (dec) {
                 // ~8k chunk slots over the whole launch (16 per resident workgroup), chunks of at
                 // least 256 keys: measured best trade between per-workgroup start-up cost and
@@ -75,16 +85,24 @@ static int plan(const fa_fwd_params& p, bool allow_split, int* split_len_out) {
             }
         }
         splits = std::max(1, std::min(splits, FA_MAX_SPLITS));
-        // never more chunks than tiles
-        splits = std::min(splits, (sk + gran - 1) / gran);
+        splits = std::min(splits, (sk + gran - 1) / gran);   // never more chunks than tiles
         splits = std::max(1, splits);
     }
     int len = rup((sk + splits - 1) / std::max(1, splits), gran);
     if (len <= 0) len = gran;
-    // drop chunks that the rounding made empty
-    splits = std::max(1, (sk + len - 1) / len);
-    if (split_len_out) *split_len_out = len;
-    return splits;
+    splits = std::max(1, (sk + len - 1) / len);               // drop chunks the rounding emptied
+    r.splits = splits;
+    r.len = len;
+    // Persistent two-pass schedule: complete chunks first, then each sequence's ragged remainder in
+    // eighths of a chunk, drawn from a ticket counter.  Needs the caller's scratch word.
+    if (dec && automatic && splits > 1 && p.work_counter && len >= 1024 && splits + 8 <= FA_MAX_SPLITS) {
+        r.persistent = 1;
+        r.sa = splits;
+        r.sb = 8;
+        r.sub = len / 8;
+        r.splits = r.sa + r.sb;
+    }
+    return r;
 }
 
 static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
@@ -100,12 +118,18 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.split_len = 0;
     kp.num_m_blocks = 0;
     kp.rotary_q = 0;
+    kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = 0;
+    kp.work_counter = q.work_counter;
 }
 
 static int run_attention(KParams& kp, hipStream_t stream) {
     const fa_fwd_params& p = kp.p;
     int e;
     if (use_decode_kernel(p)) {
+        if (kp.dec_persistent) {
+            e = launch_zero_counter(kp.work_counter, stream);
+            if (e) return fail_hip(e, "ticket reset launch");
+        }
         e = launch_decode(kp, stream);
         if (e) return fail_hip(e, "decode kernel launch");
     } else {
@@ -125,10 +149,12 @@ static int run_attention(KParams& kp, hipStream_t stream) {
 }
 
 static int resolve_splits(KParams& kp, const fa_fwd_params& p, bool allow_split) {
-    int len = 0;
-    const int s = plan(p, allow_split, &len);
+    const SplitPlan r = plan(p, allow_split);
+    const int s = r.splits;
     kp.num_splits = s;
-    kp.split_len = len;
+    kp.split_len = r.len;
+    kp.dec_persistent = r.persistent;
+    kp.dec_sa = r.sa; kp.dec_sb = r.sb; kp.dec_sub = r.sub;
     if (s > 1 && (!p.o_accum || !p.lse_accum)) return fail("o_accum and lse_accum are required when the key range is split (see fa_plan_splits)");
     return 0;
 }
@@ -166,7 +192,7 @@ int fa_plan_splits(const fa_fwd_params* p, int32_t api, int32_t* num_splits) {
     if (int r = check_common(p)) return r;
     if (!num_splits) return fail("num_splits is NULL");
     if (api != 0 && api != 2) return fail("api must be 0 (fa_fwd) or 2 (fa_fwd_kvcache)");
-    *num_splits = plan(*p, true, nullptr);
+    *num_splits = plan(*p, true).splits;
     return 0;
 }
 

@@ -35,6 +35,10 @@ struct KParams {
     int32_t num_m_blocks;  // query tiles per (batch, head)
     int32_t has_left, has_right;  // window bounds active (after causal normalisation)
     int32_t rotary_q;      // rotate q on load
+    // persistent decode schedule (see fa_decode.hip): dec_sa slots of split_len keys, then dec_sb
+    // slots of dec_sub keys for each sequence's ragged remainder; tickets from *work_counter
+    int32_t dec_persistent, dec_sa, dec_sb, dec_sub;
+    int32_t* work_counter;
 };
 
 template <typename T> struct Elem;

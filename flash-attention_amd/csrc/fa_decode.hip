@@ -38,18 +38,24 @@ struct DecodeCfg {
     static constexpr int SMEM = STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES;
 };
 
+// Key range of one work item.  kChunk: chunk `idx` of kp.split_len keys.  kMacro / kSub are the two
+// passes of the persistent schedule: first every COMPLETE chunk of kp.split_len keys, then the
+// ragged remainder of each sequence in pieces of kp.dec_sub keys, so that the last items handed out
+// are small and the workgroups finish together.
+enum ItemMode { kChunk = 0, kMacro = 1, kSub = 2 };
+
+// One (batch, kv head, key range) item: attention of the packed query rows over the range, written
+// as the final output (SPLIT = false) or as partial `slot` (SPLIT = true).
 template <typename T, int D, bool SPLIT>
-__global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KParams kp) {
+FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b, const int slot,
+                        const int mode, const int idx) {
     typedef DecodeCfg<T, D> C;
     typedef typename Elem<T>::v8 v8;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_fwd_params& p = kp.p;
+    const int split = slot;
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int m = lane & 15, g4 = lane >> 4;     // MFMA column (packed query row), lane group
-    // kv heads vary fastest over the grid: the h_k workgroups that share the rows of one
-    // (batch, chunk) of a (b, s, h_k, d) cache run together and consume whole cache rows.
-    const int hk = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
     const int G = p.h / p.h_k;
     const int rows = p.seqlen_q * G;             // packed rows in use (<= 16)
 
@@ -62,8 +68,18 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
     if (has_right) hi = min(hi, si.sq + shift + wr);
     if (has_left) lo = max(0, shift - wl);
     if (SPLIT) {
-        lo = max(lo, split * kp.split_len);
-        hi = min(hi, (split + 1) * kp.split_len);
+        int c_lo, c_hi;
+        if (mode == kSub) {
+            const int base = hi / kp.split_len * kp.split_len;     // start of the incomplete chunk
+            c_lo = base + idx * kp.dec_sub;
+            c_hi = (base == hi) ? c_lo : c_lo + kp.dec_sub;
+        } else {
+            c_lo = idx * kp.split_len;
+            c_hi = c_lo + kp.split_len;
+            if (mode == kMacro && c_hi > hi) c_hi = c_lo;          // incomplete: left to the kSub pass
+        }
+        lo = max(lo, c_lo);
+        hi = min(hi, c_hi);
     }
 
     // packed row m -> query position and head
@@ -83,30 +99,6 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
             }
         }
         return;
-    }
-
-    // ---- Q fragments (B operand): lane (m, g4) holds Q[row m][32c + 8*g4 .. +7]
-    v8 qf[C::KC];
-    {
-        const T* qrow = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)qi * p.q_row_stride + (int64_t)head * p.q_head_stride;
-#pragma unroll
-        for (int c = 0; c < C::KC; c++) {
-            const int d0 = c * 32 + 8 * g4;
-            u32x4 raw = {0, 0, 0, 0};
-            if (row_valid && d0 < p.d) {
-                raw = ld_global16(qrow + d0);
-                if (kp.rotary_q && d0 < p.rotary_dim) {
-                    const int pos = si.sk_cache + ((p.is_causal || has_left || has_right) ? qi : 0);
-                    const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
-                    const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
-                    float x[8];
-                    unpack8<T>(raw, x);
-                    rotary8<T>(x, qrow, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
-                    raw = pack8<T>(x);
-                }
-            }
-            qf[c] = __builtin_bit_cast(v8, raw);
-        }
     }
 
     // ---- this wave's key range
@@ -156,7 +148,34 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
     const int lim_lo = has_left ? qi + shift - wl : 0;
     const int tj = (lane & 15) >> 2, tq = lane & 3;
 
+    // the first K/V step is requested before anything else so that its latency overlaps the q
+    // (and rotary table) fetches below
     if (w_lo < w_hi) load_step(w_lo);
+
+    // ---- Q fragments (B operand): lane (m, g4) holds Q[row m][32c + 8*g4 .. +7]
+    v8 qf[C::KC];
+    {
+        const T* qrow = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)qi * p.q_row_stride + (int64_t)head * p.q_head_stride;
+#pragma unroll
+        for (int c = 0; c < C::KC; c++) {
+            const int d0 = c * 32 + 8 * g4;
+            u32x4 raw = {0, 0, 0, 0};
+            if (row_valid && d0 < p.d) {
+                raw = ld_global16(qrow + d0);
+                if (kp.rotary_q && d0 < p.rotary_dim) {
+                    const int pos = si.sk_cache + ((p.is_causal || has_left || has_right) ? qi : 0);
+                    const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
+                    const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
+                    float x[8];
+                    unpack8<T>(raw, x);
+                    rotary8<T>(x, qrow, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
+                    raw = pack8<T>(x);
+                }
+            }
+            qf[c] = __builtin_bit_cast(v8, raw);
+        }
+    }
+
     for (int n0 = w_lo; n0 < w_hi; n0 += C::STEP) {
         // the previous step's LDS reads are complete (their results were consumed) before these
         // writes are issued; LDS operations of one wave execute in order.
@@ -294,12 +313,58 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
     }
 }
 
+template <typename T, int D, bool SPLIT>
+__global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KParams kp) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    // kv heads vary fastest over the grid: the h_k workgroups that share the rows of one
+    // (batch, chunk) of a (b, s, h_k, d) cache run together and consume whole cache rows.
+    decode_item<T, D, SPLIT>(kp, smem, blockIdx.x, blockIdx.z, blockIdx.y, kChunk, blockIdx.y);
+}
+
+// Persistent form: a fixed number of resident workgroups draw items from a ticket counter, in the
+// same cache-row-friendly order (kv head fastest), first the kMacro pass then the kSub pass.
+template <typename T, int D>
+__global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kernel(const KParams kp) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int s_ticket;
+    const fa_fwd_params& p = kp.p;
+    const int n_macro = p.b * kp.dec_sa * p.h_k;
+    const int total = n_macro + p.b * kp.dec_sb * p.h_k;
+    for (;;) {
+        __syncthreads();          // previous item is done with LDS and with s_ticket
+        if (threadIdx.x == 0) s_ticket = atomicAdd(kp.work_counter, 1);
+        __syncthreads();
+        int t = s_ticket;
+        if (t >= total) break;
+        if (t < n_macro) {
+            const int hk = t % p.h_k, s = (t / p.h_k) % kp.dec_sa, b = t / (p.h_k * kp.dec_sa);
+            decode_item<T, D, true>(kp, smem, hk, b, s, kMacro, s);
+        } else {
+            t -= n_macro;
+            const int hk = t % p.h_k, j = (t / p.h_k) % kp.dec_sb, b = t / (p.h_k * kp.dec_sb);
+            decode_item<T, D, true>(kp, smem, hk, b, kp.dec_sa + j, kSub, j);
+        }
+    }
+}
+
+__global__ void zero_counter_kernel(int32_t* c) { if (threadIdx.x == 0) *c = 0; }
+
 template <typename T, int D>
 static int launch_decode_t(const KParams& kp, hipStream_t stream) {
     typedef DecodeCfg<T, D> C;
     const bool split = kp.num_splits > 1;
-    dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b), block(C::kThreads);
     hipError_t e;
+    if (kp.dec_persistent) {
+        const int total = kp.p.b * (kp.dec_sa + kp.dec_sb) * kp.p.h_k;
+        const int resident = 256 * (D > 128 ? 1 : 2);          // workgroups the 256 CUs hold at once
+        dim3 grid(total < resident ? total : resident), block(C::kThreads);
+        auto kern = decode_persistent_kernel<T, D>;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+        return (int)hipGetLastError();
+    }
+    dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b), block(C::kThreads);
     if (split) {
         auto kern = decode_kernel<T, D, true>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
@@ -311,6 +376,11 @@ static int launch_decode_t(const KParams& kp, hipStream_t stream) {
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     }
+    return (int)hipGetLastError();
+}
+
+int launch_zero_counter(int32_t* c, hipStream_t stream) {
+    hipLaunchKernelGGL(zero_counter_kernel, dim3(1), dim3(64), 0, stream, c);
     return (int)hipGetLastError();
 }
 

@@ -16,6 +16,7 @@ int prefill_block_n(int d_bucket);   // key-tile length of the prefill kernel fo
 int prefill_block_m(int d_bucket);
 
 int launch_decode(const KParams& kp, hipStream_t stream);      // small-q split-KV kernel
+int launch_zero_counter(int32_t* c, hipStream_t stream);     // ticket counter of the persistent decode
 int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials
 int launch_append_kv(const KParams& kp, hipStream_t stream);   // k_new/v_new (+rotary) -> cache
 }  // namespace fa

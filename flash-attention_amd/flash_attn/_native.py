@@ -30,7 +30,7 @@ class FaFwdParams(ctypes.Structure):
     _fields_ = (
         [(n, ctypes.c_void_p) for n in (
             "q", "k", "v", "o", "softmax_lse", "o_accum", "lse_accum", "k_new", "v_new",
-            "rotary_cos", "rotary_sin", "cu_seqlens_q", "cu_seqlens_k", "cache_batch_idx")]
+            "rotary_cos", "rotary_sin", "cu_seqlens_q", "cu_seqlens_k", "cache_batch_idx", "work_counter")]
         + [(n, ctypes.c_int64) for n in (
             "q_batch_stride", "q_row_stride", "q_head_stride",
             "k_batch_stride", "k_row_stride", "k_head_stride",
@@ -119,17 +119,18 @@ def _plan_and_alloc(params, api, batch, heads, seqlen_q, d, device):
     """Resolve the split count and allocate the fp32 partial buffers like the reference does
     (flash_api.cpp:373-389, 1241-1257).  The returned tensors must stay alive until launch."""
     n = ctypes.c_int32(0)
+    counter = torch.empty((1,), dtype=torch.int32, device=device)   # ticket scratch of the persistent decode
+    params.work_counter = counter.data_ptr()
     rc = lib.fa_plan_splits(ctypes.byref(params), api, ctypes.byref(n))
     if rc != 0:
         raise RuntimeError(lib.fa_last_error().decode())
-    params.num_splits = n.value
-    keep = None
+    keep = (counter,)
     if n.value > 1:
         lse_accum = torch.empty((n.value, batch, heads, seqlen_q), dtype=torch.float32, device=device)
         o_accum = torch.empty((n.value, batch, heads, seqlen_q, _round_up(d, 32)), dtype=torch.float32, device=device)
         params.lse_accum = lse_accum.data_ptr()
         params.o_accum = o_accum.data_ptr()
-        keep = (lse_accum, o_accum)
+        keep = (counter, lse_accum, o_accum)
     return keep
 
 

@@ -57,6 +57,10 @@ typedef struct fa_fwd_params {
     const int32_t *cu_seqlens_k;    /* (b+1) prefix sums if is_seqlens_k_cumulative, else (b)
                                        per-batch key lengths (cache_seqlens), or NULL */
     const int32_t *cache_batch_idx; /* (b) row of k/v used (and updated) for batch i, or NULL */
+    int32_t *work_counter;          /* optional: one int32 of device scratch (any value; the library
+                                       resets it on the stream before use).  When set, split-KV
+                                       decode launches run as a persistent, ticket-scheduled kernel.
+                                       Must not be shared by calls that overlap on the GPU. */
 
     int64_t q_batch_stride, q_row_stride, q_head_stride;
     int64_t k_batch_stride, k_row_stride, k_head_stride;
@@ -108,8 +112,10 @@ int fa_fwd_kvcache(const fa_fwd_params *p, void *hip_stream);
  * Resolves the split count the library will use for this problem, so that the caller can size
  * o_accum / lse_accum before the call (the reference does this inside mha_fwd / mha_fwd_kvcache,
  * flash_api.cpp:373-389, 1241-1257, with num_splits_heuristic :212-246; this library uses its
- * own rule for 256 CUs).  `api` is 0 for fa_fwd, 2 for fa_fwd_kvcache.  Writes the resolved count
- * (1..FA_MAX_SPLITS) to *num_splits.  The same value must then be passed in p->num_splits.
+ * own rule for 256 CUs).  `api` is 0 for fa_fwd, 2 for fa_fwd_kvcache.  Writes the number of
+ * partial slots (1..FA_MAX_SPLITS) to *num_splits: o_accum / lse_accum must hold that many.  The
+ * subsequent call takes the SAME params (same num_splits request, same work_counter): it repeats
+ * the same deterministic plan.
  */
 int fa_plan_splits(const fa_fwd_params *p, int32_t api, int32_t *num_splits);
 
