@@ -26,7 +26,13 @@ static int bucket(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
 static const int kNumCU = 256;   // MI355X
 #ifndef FA_DEC_SLOTS
-#define FA_DEC_SLOTS 8192
+#define FA_DEC_SLOTS 8192       // chunk slots per launch, one workgroup per chunk
+#endif
+#ifndef FA_DEC_SLOTS_P
+#define FA_DEC_SLOTS_P 4096     // same for the persistent, ticket-scheduled kernel
+#endif
+#ifndef FA_DEC_SB
+#define FA_DEC_SB 8
 #endif
 
 // The small-q streaming kernel packs seqlen_q x (h / h_k) rows into 16 MFMA columns.
@@ -73,8 +79,14 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
                 // ~8k chunk slots over the whole launch (16 per resident workgroup), chunks of at
                 // least 256 keys: measured best trade between per-workgroup start-up cost and
                 // the tail left by ragged cache lengths on 256 CUs x 2 resident groups.
+                // With the caller's scratch word the kernel is persistent and takes longer chunks
+                // (4096 keys at batch 64 x 8 kv heads x 32k), their ragged remainders in eighths.
                 const int64_t streams = (int64_t)p.b * p.h_k;
                 int64_t len = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS), 128);
+                if (p.work_counter) {
+                    const int64_t lp = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS_P), 128);
+                    if (lp >= 1024) len = lp;
+                }
                 splits = (int)((sk + len - 1) / len);
             } else {
                 const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;
@@ -95,11 +107,11 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
     r.len = len;
     // Persistent two-pass schedule: complete chunks first, then each sequence's ragged remainder in
     // eighths of a chunk, drawn from a ticket counter.  Needs the caller's scratch word.
-    if (dec && automatic && splits > 1 && p.work_counter && len >= 1024 && splits + 8 <= FA_MAX_SPLITS) {
+    if (dec && automatic && splits > 1 && p.work_counter && len >= 1024 && splits + FA_DEC_SB <= FA_MAX_SPLITS) {
         r.persistent = 1;
         r.sa = splits;
-        r.sb = 8;
-        r.sub = len / 8;
+        r.sb = FA_DEC_SB;
+        r.sub = len / FA_DEC_SB;
         r.splits = r.sa + r.sb;
     }
     return r;
