@@ -20,8 +20,9 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
 #define FA_PP_MIN_SQ 1024
 #endif
     // long query sequences: the 8-wave ping-pong kernel (256 rows per workgroup)
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= FA_PP_MIN_SQ)
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= FA_PP_MIN_SQ) {
         return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
+    }
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }

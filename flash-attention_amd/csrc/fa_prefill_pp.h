@@ -207,10 +207,15 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     for (int dk = 0; dk < C::KS; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dk * 2 + hh, l32) * 16;
     f32x16 s_acc[C::NB];
     auto qk = [&](int i) {
-        const char* kb = smem + (i & (C::NS - 1)) * C::TILE;
+        // one address register per k-step, advanced to the tile's ring slot once; every other
+        // displacement is an instruction immediate
+        const int slot = (i & (C::NS - 1)) * C::TILE;
+        const char* kb[C::KS];
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) kb[dk] = smem + (slot + kofs[dk]);
         constexpr int NF = C::NB * C::KS;          // fragments in (nb, dk) order
         constexpr int LA = FA_PP_LA;
-        auto frag_ptr = [&](int f) { return kb + (f / C::KS) * 32 * C::ROWB + kofs[f % C::KS]; };
+        auto frag_ptr = [&](int f) { return kb[f % C::KS] + (f / C::KS) * 32 * C::ROWB; };
         u32x4 fr[LA];
 #pragma unroll
         for (int e = 0; e < LA; e++) fr[e] = *reinterpret_cast<const u32x4*>(frag_ptr(e));
@@ -239,13 +244,16 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         vofs[db] = (4 * hh + tj) * C::ROWB + swz_v<D>(db * 4 + dhalf * 2 + (tq >> 1), 4 * hh + tj) * 16 + (tq & 1) * 8;
     v8 pf[C::PT];
     auto pv = [&](int i) {
-        const char* vb = smem + (C::NS + (i & (C::NS - 1))) * C::TILE;
+        const int slot = (C::NS + (i & (C::NS - 1))) * C::TILE;
+        const char* vb[C::DB];
+#pragma unroll
+        for (int db = 0; db < C::DB; db++) vb[db] = smem + (slot + vofs[db]);
         constexpr int NF = C::PT * C::DB;          // fragments in (t16, db) order
         constexpr int LA = FA_PP_LA;
         auto fetch = [&](int f) {
             const int t16 = f / C::DB, db = f % C::DB;
-            const u32x2 lo = lds_read_tr16(vb + t16 * 16 * C::ROWB + vofs[db]);
-            const u32x2 hi = lds_read_tr16(vb + (t16 * 16 + 8) * C::ROWB + vofs[db]);
+            const u32x2 lo = lds_read_tr16(vb[db] + t16 * 16 * C::ROWB);
+            const u32x2 hi = lds_read_tr16(vb[db] + (t16 * 16 + 8) * C::ROWB);
             return (u32x4){lo[0], lo[1], hi[0], hi[1]};
         };
         u32x4 fr[LA];
