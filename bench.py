@@ -69,7 +69,7 @@ def bench_prefill(steps, warmup):
         "ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"),
-                     "kernel": "prefill_kernel<bf16,128>", "flops_per_launch": flops},
+                     "kernel": "fa::prefill_pp_kernel<bf16,128,64>", "flops_per_launch": flops},
     }
 
 
@@ -98,7 +98,7 @@ def bench_decode(steps, warmup):
         "workload": "flash_attn_with_kvcache bf16 b64 cache(64,32768,8,128) hq64 append1+rotary128 causal",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": gbs / PEAK_HBM_GBS, "traffic": _traffic("decode_bf16_d128_b64_32k"),
-                     "kernel": "append_kv + decode_kernel<bf16,128,split> + combine", "bytes_per_launch": algo_bytes},
+                     "kernel": "fa::decode_persistent_kernel<bf16,128> (step = ticket reset + append_kv + decode + combine)", "bytes_per_launch": algo_bytes},
     }
 
 
