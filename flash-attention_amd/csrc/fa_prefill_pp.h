@@ -75,16 +75,18 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const int l32 = lane & 31, hh = lane >> 5;
     const int group = wave >> 2;
 
-    const int G = p.h / p.h_k;
-    const int64_t total = (int64_t)kp.num_m_blocks * p.h * p.b;
-    const int per_xcd = gridDim.x >> 3;
-    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
+    const uint32_t G = (uint32_t)(p.h / p.h_k);
+    const uint32_t nmb = (uint32_t)kp.num_m_blocks;
+    const uint32_t total = nmb * (uint32_t)p.h * (uint32_t)p.b;
+    const uint32_t per_xcd = gridDim.x >> 3;
+    uint32_t w = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
     if (w >= total) return;
     const int g = (int)(w % G); w /= G;
-    const int mb = kp.num_m_blocks - 1 - (int)(w % kp.num_m_blocks); w /= kp.num_m_blocks;
-    const int hk = (int)(w % p.h_k);
-    const int b = (int)(w / p.h_k);
-    const int head = hk * G + g;
+    const int mb = (int)(nmb - 1 - w % nmb); w /= nmb;
+    const int hk = (int)(w % (uint32_t)p.h_k);
+    const int b = (int)(w / (uint32_t)p.h_k);
+    const int head = hk * (int)G + g;
 
     const SeqInfo si = seq_info(p, b);
     const int m0 = mb * C::BM;
@@ -365,20 +367,32 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
     const float inv = dead ? 1.f : 1.f / l_tot;
     const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
-    if (row < si.sq) {
-        if (hh == 0) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
-        T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)row * p.o_row_stride + (int64_t)head * p.o_head_stride;
+    if (hh == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
+    // The output tile of the wave (32 rows x D) goes through LDS so that every store instruction
+    // writes whole rows (16 B per lane, 64 / (D/8) rows per instruction) instead of 8-byte pieces
+    // of 32 rows.  All tile reads of the ring are behind the last barrier and each wave uses its
+    // own region, so no barrier is needed.
+    {
+        constexpr int PITCH = C::ROWB + 16;
+        char* stage = smem + wave * (32 * PITCH);
 #pragma unroll
         for (int db = 0; db < C::DB; db++)
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const int d0 = db * 32 + 8 * q4 + 4 * hh;
-                if (d0 < p.d) {
-                    u32x2 v = {pack2<T>(o_acc[db][4 * q4] * inv, o_acc[db][4 * q4 + 1] * inv),
-                               pack2<T>(o_acc[db][4 * q4 + 2] * inv, o_acc[db][4 * q4 + 3] * inv)};
-                    st_global8(orow + d0, v);
-                }
+                const u32x2 v = {pack2<T>(o_acc[db][4 * q4] * inv, o_acc[db][4 * q4 + 1] * inv),
+                                 pack2<T>(o_acc[db][4 * q4 + 2] * inv, o_acc[db][4 * q4 + 3] * inv)};
+                *reinterpret_cast<u32x2*>(stage + l32 * PITCH + d0 * 2) = v;
             }
+        constexpr int RPP = 64 / C::CPR;                // rows per store instruction
+        const int srow = lane / C::CPR, sch = lane % C::CPR;
+        T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + sch * 8;
+#pragma unroll
+        for (int j = 0; j < 32 / RPP; j++) {
+            const int rr = j * RPP + srow;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
+            if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
+        }
     }
 }
 
