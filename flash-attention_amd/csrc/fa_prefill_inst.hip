@@ -17,7 +17,7 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     typedef PrefillTile<FA_D> Tile;
 #if FA_D <= 128
 #ifndef FA_PP_MIN_SQ
-#define FA_PP_MIN_SQ 1024
+#define FA_PP_MIN_SQ (FA_D >= 128 ? 512 : 1024)     // measured cross-over against the 4-wave kernel
 #endif
     // long query sequences: the 8-wave ping-pong kernel (256 rows per workgroup)
     if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= FA_PP_MIN_SQ) {

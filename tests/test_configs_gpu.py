@@ -154,3 +154,56 @@ def test_config5_decode_kvcache_rotary():
     lens1 = lens_d + 1
     outs = [fa.flash_attn_with_kvcache(q, kc, vc, cache_seqlens=lens1, num_splits=n).float() for n in (0, 1, 5)]
     assert (outs[0] - outs[1]).abs().max().item() < 2e-2 and (outs[0] - outs[2]).abs().max().item() < 2e-2
+
+
+def test_decode_ticket_schedule_matches_one_workgroup_per_chunk(monkeypatch):
+    """The decode call takes the persistent, ticket-scheduled kernel when the caller passes a scratch
+    word and the one-workgroup-per-chunk kernel when it does not (work_counter == NULL at the C
+    boundary); both must give the same attention output (up to fp32 re-association of the combine)
+    and agree with the oracle."""
+    _say("decode: ticket schedule vs plain")
+    from flash_attn import _native as nat
+    torch.manual_seed(3)
+    b, cap, hk, h, d = 16, 32768, 8, 64, 128
+    kc = torch.randn(b, cap, hk, d, device=DEV, dtype=torch.bfloat16)
+    vc = torch.randn(b, cap, hk, d, device=DEV, dtype=torch.bfloat16)
+    q = torch.randn(b, 1, h, d, device=DEV, dtype=torch.bfloat16)
+    lens = torch.randint(1, cap + 1, (b,), dtype=torch.int32)
+    lens[0], lens[1], lens[2] = 1, cap, 4097
+    lens_d = lens.to(DEV)
+    fa = _fa()
+    out_ticket = fa.flash_attn_with_kvcache(q, kc, vc, cache_seqlens=lens_d, causal=True)
+
+    seen = []
+
+    # the plan must be made with the same (absent) scratch word as the launch: patch before planning
+    def plan_without(params, api, batch, heads, seqlen_q, dd, device):
+        import ctypes
+        n = ctypes.c_int32(0)
+        params.work_counter = None
+        rc = nat.lib.fa_plan_splits(ctypes.byref(params), api, ctypes.byref(n))
+        assert rc == 0
+        seen.append(n.value)
+        keep = ()
+        if n.value > 1:
+            lse_accum = torch.empty((n.value, batch, heads, seqlen_q), dtype=torch.float32, device=device)
+            o_accum = torch.empty((n.value, batch, heads, seqlen_q, (dd + 31) // 32 * 32), dtype=torch.float32, device=device)
+            params.lse_accum = lse_accum.data_ptr()
+            params.o_accum = o_accum.data_ptr()
+            keep = (lse_accum, o_accum)
+        return keep
+    monkeypatch.setattr(nat, "_plan_and_alloc", plan_without)
+    out_plain = fa.flash_attn_with_kvcache(q, kc, vc, cache_seqlens=lens_d, causal=True)
+    monkeypatch.undo()
+    assert seen and seen[0] > 1                      # the plain path did split
+    assert not torch.isnan(out_ticket).any() and not torch.isnan(out_plain).any()
+    diff = (out_ticket.float() - out_plain.float()).abs().max().item()
+    _say("   max |ticket - plain| = %.3e" % diff)
+    assert diff < 2e-2
+    for i in (0, 1, 2, 9):
+        L = int(lens[i])
+        o_ref, _, o_pt = orc.attention_reference_pair(q[i:i + 1].cpu(), kc[i:i + 1, :L].cpu(), vc[i:i + 1, :L].cpu(), causal=True)
+        for name, o in (("ticket", out_ticket), ("plain", out_plain)):
+            ok, err, bound = orc.tolerance_ok(o[i:i + 1].cpu(), o_ref, o_pt, 3.0, 1e-5)
+            _say("   batch %d (len %d) %s: err %.3e bound %.3e" % (i, L, name, err, bound))
+            assert ok
