@@ -1,0 +1,531 @@
+// Software-pipelined forward kernel for gfx950: 4 waves x 32 query rows, two workgroups per CU.
+//
+// Same mathematics, register layouts and LDS tile format as prefill_pp_kernel (fa_prefill_pp.h):
+// S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16 with one query row per lane, K/V tiles of 64
+// keys moved global -> LDS by global_load_lds_dwordx4.  What differs is the schedule.  Every wave
+// runs the three independent pieces of work of one loop step in ONE instruction stream:
+//
+//     step i:   O += P(i-1) V(i-1)      (16 MFMA for head dim 128)
+//               S(i+1) = K(i+1) Q       (16 MFMA)
+//               P(i) = softmax(S(i))    (vector/transcendental work)
+//
+// written as one chunk per matrix instruction (the MFMA, the LDS fragment read a few chunks ahead,
+// a slice of the softmax) with scheduling barriers between chunks, so the matrix pipe of a SIMD is
+// fed by whichever of its two resident waves is ready.  Those two waves belong to DIFFERENT
+// workgroups (128 query rows and a 64 KB two-slot K/V ring each), so they never wait for each other,
+// and the start-up and output phases of one workgroup overlap the steady state of the other.  The
+// price is that each K/V tile is fetched from L2 once per 128 rows instead of once per 256: the
+// ping-pong kernel stays ahead for long non-causal sequences at head dim 128, this one wins for
+// shorter sequences and for head dim 64.  S and P are double-buffered in registers (the loop is
+// unrolled by two so that the buffers alternate without copies).
+//
+// Steps whose tile needs masking, and the first and last steps, run the same three pieces one
+// after the other ("plain" step).  The running max is lazy as in the ping-pong kernel; the rescale
+// of O that a moved max needs is applied after the step's matrix instructions.
+#pragma once
+#include "fa_common.h"
+#include "fa_prefill_pp.h"
+
+namespace fa {
+
+#ifndef FA_IL_LA
+#define FA_IL_LA 4
+#endif
+
+template <typename T, int D, int BN>
+struct ILCfg {
+    static constexpr int kThreads = 256;
+    static constexpr int kWaves = 4;
+    static constexpr int BM = kWaves * 32;
+    static constexpr int NB = BN / 32;
+    static constexpr int KS = D / 16;
+    static constexpr int DB = D / 32;
+    static constexpr int PT = BN / 16;
+    static constexpr int CPR = D / 8;                       // 16 B chunks per tile row
+    static constexpr int ROWB = D * 2;
+    static constexpr int TILE = BN * ROWB;                  // bytes of one K or V tile
+    static constexpr int NS = 2;                            // ring slots per tensor
+    static constexpr int LOADS = BN * CPR / kThreads;       // 16 B fills per thread per tile
+    static constexpr int ROWS_PER_PASS = kThreads / CPR;
+    static constexpr int PASSB = kThreads * 16;             // LDS bytes filled by one pass of the workgroup
+    static constexpr int SMEM = 2 * NS * TILE;              // K ring, then V ring
+    static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
+};
+
+template <typename T, int D, int BN>
+__global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
+    typedef ILCfg<T, D, BN> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_fwd_params& p = kp.p;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int l32 = lane & 31, hh = lane >> 5;
+
+    const int G = p.h / p.h_k;
+    const int64_t total = (int64_t)kp.num_m_blocks * p.h * p.b;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int g = (int)(w % G); w /= G;
+    const int mb = kp.num_m_blocks - 1 - (int)(w % kp.num_m_blocks); w /= kp.num_m_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+    const int head = hk * G + g;
+
+    const SeqInfo si = seq_info(p, b);
+    const int m0 = mb * C::BM;
+    if (m0 >= si.sq) return;
+
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    int n_hi = si.sk;
+    if (has_right) n_hi = min(n_hi, min(m0 + C::BM, si.sq) + shift + wr);
+    int n_lo = 0;
+    if (has_left) n_lo = max(0, m0 + shift - wl);
+    const int t_lo = n_lo / BN;
+    const int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
+    const int nt = max(0, t_hi - t_lo);           // tiles visited, the same for all 8 waves
+
+    const T* __restrict__ qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
+    const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
+    const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
+
+    const int r0 = m0 + wave * 32;                // first query row of this wave
+    const int row = r0 + l32;
+
+    v8 qf[C::KS];
+    {
+        const bool valid = row < si.sq;
+        const T* qrow = qg + (int64_t)row * p.q_row_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 raw = {0, 0, 0, 0};
+            if (valid && d0 < p.d) raw = ld_global16(qrow + d0);
+            qf[dk] = __builtin_bit_cast(v8, raw);
+        }
+    }
+
+    f32x16 o_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const float sl2 = kp.scale_log2;
+
+    // visit i of the key loop handles key tile t_hi - 1 - i and uses ring slot i % NS
+    auto tile_of = [&](int i) { return t_hi - 1 - i; };
+
+    // ---- asynchronous tile fills (layout as in prefill_pp_kernel)
+    const int frow = (wave * 64 + lane) / C::CPR;
+    const int fch = lane % C::CPR;
+    const int kch = min(swz_k<D>(fch, frow), p.d / 8 - 1);
+    const int vch = min(swz_v<D>(fch, frow), p.d / 8 - 1);
+    const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
+    const uint32_t fill_base = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(wave * 1024));
+    // Scalar base of the tile (uniform over the workgroup) + a 32-bit per-lane byte offset: the
+    // fill instruction takes its address as SGPR pair + VGPR offset, and moving on to the next tile
+    // is scalar arithmetic.
+    const int64_t kstep = (int64_t)BN * p.k_row_stride, vstep = (int64_t)BN * p.v_row_stride;
+    const int64_t kpass = (int64_t)C::ROWS_PER_PASS * p.k_row_stride, vpass = (int64_t)C::ROWS_PER_PASS * p.v_row_stride;
+    const T* ktile = kg + (int64_t)(t_hi - 1) * BN * p.k_row_stride;     // uniform
+    const T* vtile = vg + (int64_t)(t_hi - 1) * BN * p.v_row_stride;
+    const uint32_t koff = (uint32_t)(((int64_t)frow * p.k_row_stride + kch * 8) * 2);
+    const uint32_t voff = (uint32_t)(((int64_t)frow * p.v_row_stride + vch * 8) * 2);
+    const bool tail_clamp = t_hi * BN > si.sk;    // only visit 0 can reach past seqlen_k
+    auto fill_s = [&](const T* sbase_any, uint32_t off, uint32_t dst) {
+        // the base is uniform by construction; say so, or it may be kept in vector registers
+        const uint64_t a = (uint64_t)sbase_any;
+        const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                               ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(dst), "v"(off), "s"(sbase) : "memory", "m0");
+    };
+    auto fill_k = [&](int i) {
+        const uint32_t dst = fill_base + (uint32_t)((i & (C::NS - 1)) * C::TILE);
+        if (i == 0 && tail_clamp) {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) {
+                const int n = min(frow + j * C::ROWS_PER_PASS, si.sk - 1 - (t_hi - 1) * BN);
+                fill_s(ktile, (uint32_t)(((int64_t)n * p.k_row_stride + kch * 8) * 2), dst + j * C::PASSB);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) fill_s(ktile + j * kpass, koff, dst + j * C::PASSB);
+        }
+        ktile -= kstep;
+    };
+    auto fill_v = [&](int i) {
+        const uint32_t dst = fill_base + (uint32_t)((C::NS + (i & (C::NS - 1))) * C::TILE);
+        if (i == 0 && tail_clamp) {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) {
+                const int n = min(frow + j * C::ROWS_PER_PASS, si.sk - 1 - (t_hi - 1) * BN);
+                fill_s(vtile, (uint32_t)(((int64_t)n * p.v_row_stride + vch * 8) * 2), dst + j * C::PASSB);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) fill_s(vtile + j * vpass, voff, dst + j * C::PASSB);
+        }
+        vtile -= vstep;
+    };
+
+    // Tiles in [tf_lo, tf_hi] (absolute key-tile index) are fully visible to all 32 rows of the wave.
+    int tf_lo = 0, tf_hi = si.sk / BN - 1;
+    if (has_right) {
+        const int c = r0 + shift + wr;            // last visible key of the wave's first row
+        tf_hi = min(tf_hi, (c + 1 >= BN) ? (c + 1) / BN - 1 : -1);
+    }
+    if (has_left) {
+        const int c = r0 + shift - wl;            // first visible key of the wave's first row
+        tf_lo = (c + 31 > 0) ? (c + 31 + BN - 1) / BN : 0;
+    }
+
+    // ---- LDS fragment addressing
+    int kofs[C::KS];
+#pragma unroll
+    for (int dk = 0; dk < C::KS; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dk * 2 + hh, l32) * 16;
+    const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
+    int vofs[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+        vofs[db] = (4 * hh + tj) * C::ROWB + swz_v<D>(db * 4 + dhalf * 2 + (tq >> 1), 4 * hh + tj) * 16 + (tq & 1) * 8;
+
+    constexpr int LA = FA_IL_LA;
+    constexpr int NFV = C::PT * C::DB;             // V fragments in (t16, db) order
+    constexpr int NFK = C::NB * C::KS;             // K fragments in (nb, dk) order
+    static_assert(LA <= NFV && LA <= NFK, "look-ahead depth");
+
+    // The matrix stream of one step: O += P(iv) V(iv) when PV, then s_out = K(ik) Q when QK.
+    // Fragment reads run LA matrix instructions ahead.
+    auto mma = [&](auto with_pv, auto with_qk, int iv, int ik, const v8 (&pf)[C::PT],
+                   f32x16 (&s_out)[C::NB]) __attribute__((always_inline)) {
+        constexpr bool PV = decltype(with_pv)::value, QK = decltype(with_qk)::value;
+        constexpr int F0 = PV ? 0 : NFV, F1 = QK ? NFV + NFK : NFV;
+        const int vslot = (C::NS + (iv & (C::NS - 1))) * C::TILE;
+        const int kslot = (ik & (C::NS - 1)) * C::TILE;
+        const char* vb[C::DB];
+        const char* kb[C::KS];
+        if (PV) {
+#pragma unroll
+            for (int db = 0; db < C::DB; db++) vb[db] = smem + (vslot + vofs[db]);
+        }
+        if (QK) {
+#pragma unroll
+            for (int dk = 0; dk < C::KS; dk++) kb[dk] = smem + (kslot + kofs[dk]);
+        }
+        auto fetch = [&](int f) {
+            if (f < NFV) {
+                const int t16 = f / C::DB, db = f % C::DB;
+                const u32x2 lo = lds_read_tr16(vb[db] + t16 * 16 * C::ROWB);
+                const u32x2 hi = lds_read_tr16(vb[db] + (t16 * 16 + 8) * C::ROWB);
+                return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+            }
+            const int gk = f - NFV;
+            return *reinterpret_cast<const u32x4*>(kb[gk % C::KS] + (gk / C::KS) * 32 * C::ROWB);
+        };
+        u32x4 fr[LA];
+#pragma unroll
+        for (int e = 0; e < LA; e++) fr[e] = fetch(F0 + e);
+#pragma unroll
+        for (int f = F0; f < F1; f++) {
+            const v8 a = __builtin_bit_cast(v8, fr[(f - F0) % LA]);
+            if (f < NFV) {
+                o_acc[f % C::DB] = Elem<T>::mfma32(a, pf[f / C::DB], o_acc[f % C::DB]);
+            } else {
+                const int gk = f - NFV, nb = gk / C::KS, dk = gk % C::KS;
+                if (dk == 0) {
+                    f32x16 z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0.f;
+                    s_out[nb] = Elem<T>::mfma32(a, qf[dk], z);
+                } else {
+                    s_out[nb] = Elem<T>::mfma32(a, qf[dk], s_out[nb]);
+                }
+            }
+            if (f + LA < F1) fr[(f - F0) % LA] = fetch(f + LA);
+        }
+        // look-ahead reads first
+        __builtin_amdgcn_sched_group_barrier(0x100, PV ? 2 * LA : LA, 0);
+#pragma unroll
+        for (int f = F0; f < F1; f++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                            // 1 MFMA
+            if (f + LA < NFV) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);          // V fragment
+            else if (f + LA < F1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // K fragment
+        }
+    };
+
+    // ---- softmax pieces.  decide(): tile max, lazy reference-max update; returns the factor the
+    // old O and row sum must be scaled by (1 when the reference max did not move).
+    auto mask_tile = [&](int i, f32x16 (&s)[C::NB]) __attribute__((always_inline)) {
+        const int tt = tile_of(i);
+        if (tt < tf_lo || tt > tf_hi) {
+            const int n0 = tt * BN;
+            int lim_hi = si.sk - 1;
+            if (has_right) lim_hi = min(lim_hi, row + shift + wr);
+            const int lim_lo = has_left ? row + shift - wl : 0;
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                    if (n > lim_hi || n < lim_lo) s[nb][r] = -INFINITY;
+                }
+        }
+    };
+    auto probs = [&](const f32x16 (&s)[C::NB], v8 (&pf)[C::PT], float& corr_out, bool& move_out, float sl2) __attribute__((always_inline)) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[nb][r]);
+        mx = xhalf_max(mx);
+        // lazy reference max: move it only when the tile max exceeds it by more than 2^8 (exp2 domain)
+        const bool move = (mx - m_run) * sl2 > 8.f;       // false for NaN (-inf - -inf)
+        const float m_new = move ? mx : m_run;
+        const float corr = move ? fast_exp2((m_run - m_new) * sl2) : 1.f;   // m_run = -inf -> 0
+        m_run = m_new;
+        const float msc = (m_new == -INFINITY) ? 0.f : m_new * sl2;
+        float suma = 0.f, sumb = 0.f;
+#pragma unroll
+        for (int t16 = 0; t16 < C::PT; t16++) {
+            const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
+            u32x4 pk;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float e0 = fast_exp2(s[nb][r8 + 2 * e] * sl2 - msc);
+                const float e1 = fast_exp2(s[nb][r8 + 2 * e + 1] * sl2 - msc);
+                suma += e0;
+                sumb += e1;
+                pk[e] = pack2<T>(e0, e1);
+            }
+            pf[t16] = __builtin_bit_cast(v8, pk);
+        }
+        l_run = l_run * corr + (suma + sumb);
+        corr_out = corr;
+        move_out = move;
+    };
+    auto rescale = [&](float corr, bool move) __attribute__((always_inline)) {
+        if (__builtin_amdgcn_ballot_w64(move) != 0) {
+#pragma unroll
+            for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
+        }
+    };
+
+    f32x16 sA[C::NB], sB[C::NB];
+    v8 pA[C::PT], pB[C::PT];
+#pragma unroll
+    for (int t = 0; t < C::PT; t++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) { pA[t][e] = (T)0.f; pB[t][e] = (T)0.f; }
+
+    // Two-slot rings.  Step i reads V(i-1) and K(i+1).  When it opens, every wave of the workgroup
+    // has passed the barrier that closed step i-1, so the slots of V(i-2) and K(i) are free: the
+    // step requests V(i) and K(i+2) into them, and closes by waiting for those requests before
+    // the barrier that publishes them.  The second workgroup resident on the CU (its own rings)
+    // keeps the SIMDs busy while this one waits.
+    auto open_step = [&](int i) __attribute__((always_inline)) {
+        if (i < nt) fill_v(i);
+        if (i + 2 < nt) fill_k(i + 2);
+    };
+    auto advance_ring = [&](int i) __attribute__((always_inline)) {
+        wait_vmcnt<0>();
+        __syncthreads();
+    };
+    // Steady-state step: s_cur holds S(i), p_prev holds P(i-1); leaves S(i+1) in s_nxt and P(i) in
+    // p_cur.  The step is written as NF chunks, one per matrix instruction: the MFMA, the fragment
+    // read LA chunks ahead, and a slice of the softmax of S(i) (running max in the first chunks,
+    // then the decision about the reference max, then the exponentials two at a time).  Scheduling
+    // barriers between the chunks keep the compiler from regrouping them.
+    auto fast_step = [&](int i, const f32x16 (&s_cur)[C::NB], f32x16 (&s_nxt)[C::NB], const v8 (&p_prev)[C::PT],
+                         v8 (&p_cur)[C::PT]) __attribute__((always_inline)) {
+        constexpr int NF = NFV + NFK;
+        constexpr int NE = C::NB * 16;             // S elements per lane
+        constexpr int NP = NE / 2;                 // pairs
+        constexpr int CM = 3;                      // chunks that take the running max
+        constexpr int CD = CM;                     // chunk of the decision
+        constexpr int CE = CD + 1;                 // first chunk with exponentials
+        static_assert(NF > CE + 1, "tile too small for the chunked step");
+        open_step(i);
+        // an opaque copy of the scale keeps the vector work in this block (behind the barrier)
+        float sc = sl2;
+        asm volatile("" : "+v"(sc));
+        const int vslot = (C::NS + ((i - 1) & (C::NS - 1))) * C::TILE;
+        const int kslot = ((i + 1) & (C::NS - 1)) * C::TILE;
+        const char* vb[C::DB];
+        const char* kb[C::KS];
+#pragma unroll
+        for (int db = 0; db < C::DB; db++) vb[db] = smem + (vslot + vofs[db]);
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) kb[dk] = smem + (kslot + kofs[dk]);
+        auto fetch = [&](int f) {
+            if (f < NFV) {
+                const int t16 = f / C::DB, db = f % C::DB;
+                const u32x2 lo = lds_read_tr16(vb[db] + t16 * 16 * C::ROWB);
+                const u32x2 hi = lds_read_tr16(vb[db] + (t16 * 16 + 8) * C::ROWB);
+                return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+            }
+            const int gk = f - NFV;
+            return *reinterpret_cast<const u32x4*>(kb[gk % C::KS] + (gk / C::KS) * 32 * C::ROWB);
+        };
+        u32x4 fr[LA];
+#pragma unroll
+        for (int e = 0; e < LA; e++) fr[e] = fetch(e);
+        __builtin_amdgcn_sched_barrier(0);
+
+        float mx = -INFINITY, msc = 0.f, corr = 1.f, suma = 0.f, sumb = 0.f;
+        bool move = false;
+        uint32_t pk[NP];
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            // ---- matrix instruction f and the read for f + LA
+            const v8 a = __builtin_bit_cast(v8, fr[f % LA]);
+            if (f < NFV) {
+                o_acc[f % C::DB] = Elem<T>::mfma32(a, p_prev[f / C::DB], o_acc[f % C::DB]);
+            } else {
+                const int gk = f - NFV, nb = gk / C::KS, dk = gk % C::KS;
+                if (dk == 0) {
+                    f32x16 z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0.f;
+                    s_nxt[nb] = Elem<T>::mfma32(a, qf[dk], z);
+                } else {
+                    s_nxt[nb] = Elem<T>::mfma32(a, qf[dk], s_nxt[nb]);
+                }
+            }
+            if (f + LA < NF) fr[f % LA] = fetch(f + LA);
+            // ---- vector slice f
+            if (f < CM) {
+#pragma unroll
+                for (int e = f * NE / CM; e < (f + 1) * NE / CM; e++) mx = fmaxf(mx, s_cur[e / 16][e % 16]);
+            }
+            if (f == CD) {
+                mx = xhalf_max(mx);
+                move = (mx - m_run) * sc > 8.f;               // false for NaN (-inf - -inf)
+                const float m_new = move ? mx : m_run;
+                corr = move ? fast_exp2((m_run - m_new) * sc) : 1.f;
+                m_run = m_new;
+                msc = (m_new == -INFINITY) ? 0.f : m_new * sc;
+            }
+            if (f >= CE) {
+#pragma unroll
+                for (int pr = 0; pr < NP; pr++) {
+                    if (CE + (pr * (NF - CE)) / NP == f) {
+                        const float e0 = fast_exp2(s_cur[(2 * pr) / 16][(2 * pr) % 16] * sc - msc);
+                        const float e1 = fast_exp2(s_cur[(2 * pr + 1) / 16][(2 * pr + 1) % 16] * sc - msc);
+                        suma += e0;
+                        sumb += e1;
+                        pk[pr] = pack2<T>(e0, e1);
+                    }
+                }
+            }
+            if (f == NF - 1) l_run = l_run * corr + (suma + sumb);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // pin the step's results here, or the compiler sinks the vector work past the branch below,
+        // out of the block that holds the matrix instructions
+#pragma unroll
+        for (int t = 0; t < C::PT; t++) {
+            u32x4 u = {pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]};
+            asm volatile("" : "+v"(u));
+            p_cur[t] = __builtin_bit_cast(v8, u);
+        }
+        asm volatile("" : "+v"(l_run));
+        rescale(corr, move);
+        advance_ring(i);
+    };
+    // Plain step (first, last and masked tiles): the same pieces one after the other; S stays in sA
+    // and P in pA.
+    auto plain_step = [&](int i) __attribute__((always_inline)) {
+        open_step(i);
+        if (i > 0) mma(std::true_type(), std::false_type(), i - 1, 0, pA, sB);
+        if (i + 1 < nt) mma(std::false_type(), std::true_type(), 0, i + 1, pA, sB);
+        mask_tile(i, sA);
+        float corr; bool move;
+        probs(sA, pA, corr, move, sl2);
+        rescale(corr, move);
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++) sA[nb] = sB[nb];
+        advance_ring(i);
+    };
+
+    if (nt > 0) {
+        // ---- prologue: K(0), K(1); S(0) = K(0) Q
+        fill_k(0);
+        if (nt > 1) fill_k(1);
+        wait_vmcnt<0>();
+        __syncthreads();
+        mma(std::false_type(), std::true_type(), 0, 0, pA, sA);
+        __syncthreads();      // K(0)'s ring slot is refilled when step 0 opens
+
+        // steps [i_fb, i_fe) visit tiles that need no masking for this wave, an even number of them
+        int i_fb = max(1, t_hi - 1 - tf_hi);
+        int i_fe = min(nt - 1, t_hi - tf_lo);
+        i_fb = __builtin_amdgcn_readfirstlane(min(i_fb, nt));
+        i_fe = __builtin_amdgcn_readfirstlane(i_fe <= i_fb ? i_fb : i_fb + ((i_fe - i_fb) & ~1));
+        int i = 0;
+        for (; i < i_fb; i++) plain_step(i);
+        for (; i < i_fe; i += 2) {
+            fast_step(i, sA, sB, pA, pB);
+            fast_step(i + 1, sB, sA, pB, pA);
+        }
+        for (; i < nt; i++) plain_step(i);
+        mma(std::true_type(), std::false_type(), nt - 1, 0, pA, sB);
+    }
+
+    // ---- epilogue
+    const float l_tot = xhalf_sum(l_run);
+    const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
+    const float inv = dead ? 1.f : 1.f / l_tot;
+    const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
+    if (hh == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
+    // output tile of the wave through LDS (whole rows per store instruction); all ring reads are
+    // behind the last barrier and each wave uses its own region
+    {
+        constexpr int PITCH = C::ROWB + 16;
+        static_assert(C::kWaves * 32 * PITCH <= C::SMEM, "staging region");
+        char* stage = smem + wave * (32 * PITCH);
+#pragma unroll
+        for (int db = 0; db < C::DB; db++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int d0 = db * 32 + 8 * q4 + 4 * hh;
+                const u32x2 v = {pack2<T>(o_acc[db][4 * q4] * inv, o_acc[db][4 * q4 + 1] * inv),
+                                 pack2<T>(o_acc[db][4 * q4 + 2] * inv, o_acc[db][4 * q4 + 3] * inv)};
+                *reinterpret_cast<u32x2*>(stage + l32 * PITCH + d0 * 2) = v;
+            }
+        constexpr int RPP = 64 / C::CPR;
+        const int srow = lane / C::CPR, sch = lane % C::CPR;
+        T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + sch * 8;
+#pragma unroll
+        for (int j = 0; j < 32 / RPP; j++) {
+            const int rr = j * RPP + srow;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
+            if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
+        }
+    }
+}
+
+template <typename T, int D, int BN>
+int launch_prefill_il(KParams kp, hipStream_t stream) {
+    typedef ILCfg<T, D, BN> C;
+    kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
+    const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
+    auto kern = prefill_il_kernel<T, D, BN>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fa

@@ -1,6 +1,7 @@
 // One translation unit per (dtype, head-dim bucket): compiled with -DFA_T_BF16=0/1 -DFA_D=64/128/256.
 #include "fa_prefill.h"
 #include "fa_prefill_pp.h"
+#include "fa_prefill_il.h"
 #include "fa_launch.h"
 
 namespace fa {
@@ -16,12 +17,17 @@ typedef _Float16 InstT;
 int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     typedef PrefillTile<FA_D> Tile;
 #if FA_D <= 128
-#ifndef FA_PP_MIN_SQ
-#define FA_PP_MIN_SQ (FA_D >= 128 ? 512 : 1024)     // measured cross-over against the 4-wave kernel
-#endif
-    // long query sequences: the 8-wave ping-pong kernel (256 rows per workgroup)
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= FA_PP_MIN_SQ) {
-        return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
+    // Long query sequences (measured cross-overs on MI355X):
+    //  * head dim 128, keys beyond 4096 (causal / windowed) or 2048 (full): the 8-wave ping-pong
+    //    kernel, 256 rows per workgroup, each K/V tile fetched once per 256 rows;
+    //  * otherwise from 512 query rows on: the software-pipelined kernel, two independent
+    //    128-row workgroups per CU, whose start-up and output phases overlap.
+    // Shorter sequences, split key ranges and q rotary take the general 4-wave kernel.
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) {
+        const bool masked = kp.has_right || kp.has_left;
+        const bool long_keys = kp.p.seqlen_k > (masked ? 4096 : 2048);
+        if (FA_D >= 128 && long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
+        return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
