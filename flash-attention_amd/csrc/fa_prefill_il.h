@@ -137,14 +137,7 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
     const uint32_t koff = (uint32_t)(((int64_t)frow * p.k_row_stride + kch * 8) * 2);
     const uint32_t voff = (uint32_t)(((int64_t)frow * p.v_row_stride + vch * 8) * 2);
     const bool tail_clamp = t_hi * BN > si.sk;    // only visit 0 can reach past seqlen_k
-    auto fill_s = [&](const T* sbase_any, uint32_t off, uint32_t dst) {
-        // the base is uniform by construction; say so, or it may be kept in vector registers
-        const uint64_t a = (uint64_t)sbase_any;
-        const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
-                               ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(dst), "v"(off), "s"(sbase) : "memory", "m0");
-    };
+    auto fill_s = [&](const T* base, uint32_t off, uint32_t dst) { async_fill16(base, off, dst); };
     auto fill_k = [&](int i) {
         const uint32_t dst = fill_base + (uint32_t)((i & (C::NS - 1)) * C::TILE);
         if (i == 0 && tail_clamp) {

@@ -53,10 +53,15 @@ struct PPCfg {
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
-// 16 B from global memory to LDS address m0_base + lane * 16, bypassing registers.
-FA_DEV void async_fill16(const void* gptr, uint32_t lds_base_uniform) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :: "s"(lds_base_uniform), "v"(gptr) : "memory", "m0");
+// 16 B per lane from global memory (uniform base + per-lane byte offset) to LDS address
+// m0_base + lane * 16, bypassing registers.  The base is uniform by construction; reading it through
+// readfirstlane tells the compiler so (the instruction takes it in scalar registers).
+FA_DEV void async_fill16(const void* base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
+    const uint64_t a = (uint64_t)base_uniform;
+    const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                           ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base_uniform), "v"(lane_offset), "s"(sbase) : "memory", "m0");
 }
 // wait until at most N of this wave's vector-memory operations are outstanding (N < 16)
 template <int N> FA_DEV void wait_vmcnt() {
@@ -149,12 +154,15 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const int vch = min(swz_v<D>(fch, frow), p.d / 8 - 1);
     const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
     const uint32_t fill_base = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(wave * 1024));
+    // The address of a fill is a scalar base (start of the tile, uniform over the workgroup) plus a
+    // 32-bit per-lane byte offset, so stepping to the next tile is scalar arithmetic.
     const int64_t kstep = (int64_t)BN * p.k_row_stride, vstep = (int64_t)BN * p.v_row_stride;
     const int64_t kpass = (int64_t)C::ROWS_PER_PASS * p.k_row_stride, vpass = (int64_t)C::ROWS_PER_PASS * p.v_row_stride;
-    // running pointers: tile (visit index) next to be requested
     const int t_first = kDir > 0 ? t_lo : t_hi - 1;
-    const T* kptr = kg + (int64_t)(t_first * BN + frow) * p.k_row_stride + kch * 8;
-    const T* vptr = vg + (int64_t)(t_first * BN + frow) * p.v_row_stride + vch * 8;
+    const T* ktile = kg + (int64_t)t_first * BN * p.k_row_stride;       // tile next to be requested
+    const T* vtile = vg + (int64_t)t_first * BN * p.v_row_stride;
+    const uint32_t koff = (uint32_t)(((int64_t)frow * p.k_row_stride + kch * 8) * 2);
+    const uint32_t voff = (uint32_t)(((int64_t)frow * p.v_row_stride + vch * 8) * 2);
     // only key tile t_hi - 1 can reach past seqlen_k: its rows are clamped
     const int i_tail = (t_hi * BN > si.sk) ? (kDir > 0 ? nt - 1 : 0) : -1;
     auto fill_k = [&](int i) {
@@ -162,28 +170,28 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         if (i == i_tail) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) {
-                const int n = min((t_hi - 1) * BN + frow + j * C::ROWS_PER_PASS, si.sk - 1);
-                async_fill16(kg + (int64_t)n * p.k_row_stride + kch * 8, dst + j * 8192);
+                const int n = min(frow + j * C::ROWS_PER_PASS, si.sk - 1 - (t_hi - 1) * BN);
+                async_fill16(ktile, (uint32_t)(((int64_t)n * p.k_row_stride + kch * 8) * 2), dst + j * 8192);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < C::LOADS; j++) async_fill16(kptr + j * kpass, dst + j * 8192);
+            for (int j = 0; j < C::LOADS; j++) async_fill16(ktile + j * kpass, koff, dst + j * 8192);
         }
-        kptr += kDir * kstep;
+        ktile += kDir * kstep;
     };
     auto fill_v = [&](int i) {
         const uint32_t dst = fill_base + (uint32_t)((C::NS + (i & (C::NS - 1))) * C::TILE);
         if (i == i_tail) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) {
-                const int n = min((t_hi - 1) * BN + frow + j * C::ROWS_PER_PASS, si.sk - 1);
-                async_fill16(vg + (int64_t)n * p.v_row_stride + vch * 8, dst + j * 8192);
+                const int n = min(frow + j * C::ROWS_PER_PASS, si.sk - 1 - (t_hi - 1) * BN);
+                async_fill16(vtile, (uint32_t)(((int64_t)n * p.v_row_stride + vch * 8) * 2), dst + j * 8192);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < C::LOADS; j++) async_fill16(vptr + j * vpass, dst + j * 8192);
+            for (int j = 0; j < C::LOADS; j++) async_fill16(vtile + j * vpass, voff, dst + j * 8192);
         }
-        vptr += kDir * vstep;
+        vtile += kDir * vstep;
     };
 
     // Per-wave tile classes, as ranges of the absolute key-tile index t: the wave has visible keys
