@@ -32,14 +32,18 @@ namespace fa {
 #define FA_IL_LA 4
 #endif
 
-template <typename T, int D, int BN>
+// One query-row group of 32 rows per wave, the whole head dimension in that wave (d <= 128).
+template <typename T, int D_, int BN_>
 struct ILCfg {
+    static constexpr int D = D_, BN = BN_;
+    static constexpr bool kPair = false;
     static constexpr int kThreads = 256;
     static constexpr int kWaves = 4;
     static constexpr int BM = kWaves * 32;
+    static constexpr int DH = D;                            // head-dim slice of one wave
     static constexpr int NB = BN / 32;
-    static constexpr int KS = D / 16;
-    static constexpr int DB = D / 32;
+    static constexpr int KS = DH / 16;
+    static constexpr int DB = DH / 32;
     static constexpr int PT = BN / 16;
     static constexpr int CPR = D / 8;                       // 16 B chunks per tile row
     static constexpr int ROWB = D * 2;
@@ -48,13 +52,44 @@ struct ILCfg {
     static constexpr int LOADS = BN * CPR / kThreads;       // 16 B fills per thread per tile
     static constexpr int ROWS_PER_PASS = kThreads / CPR;
     static constexpr int PASSB = kThreads * 16;             // LDS bytes filled by one pass of the workgroup
+    static constexpr int XCH = 0;
     static constexpr int SMEM = 2 * NS * TILE;              // K ring, then V ring
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
-template <typename T, int D, int BN>
-__global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
-    typedef ILCfg<T, D, BN> C;
+// Head dim 256: O (128 accumulator registers for 32 rows) plus Q fragments (64) do not leave room
+// for two waves per SIMD, so two waves share each group of 32 query rows and split the head
+// dimension between them.  Each computes the partial scores over its 128 columns of Q and K,
+// the two partial S tiles are exchanged through LDS and added (both waves then hold the same S
+// and run the same softmax), and each accumulates its own 128 columns of O.  8 waves, 128 rows
+// per workgroup, 32-key tiles, one workgroup per CU.
+template <typename T>
+struct ILCfgPair {
+    static constexpr int D = 256, BN = 32;
+    static constexpr bool kPair = true;
+    static constexpr int kThreads = 512;
+    static constexpr int kWaves = 8;
+    static constexpr int BM = (kWaves / 2) * 32;
+    static constexpr int DH = D / 2;
+    static constexpr int NB = BN / 32;
+    static constexpr int KS = DH / 16;
+    static constexpr int DB = DH / 32;
+    static constexpr int PT = BN / 16;
+    static constexpr int CPR = D / 8;
+    static constexpr int ROWB = D * 2;
+    static constexpr int TILE = BN * ROWB;
+    static constexpr int NS = 2;
+    static constexpr int LOADS = BN * CPR / kThreads;
+    static constexpr int ROWS_PER_PASS = kThreads / CPR;
+    static constexpr int PASSB = kThreads * 16;
+    static constexpr int XCH = NB * 16 * 64 * 4;            // one partial S tile of a wave, fp32
+    static constexpr int SMEM = 2 * NS * TILE + kWaves * 2 * XCH;   // rings, then two exchange tiles per wave
+    static_assert((BN * CPR) % kThreads == 0, "tile shape");
+};
+
+template <typename T, typename C>
+__global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParams kp) {
+    constexpr int D = C::D, BN = C::BN;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_fwd_params& p = kp.p;
@@ -93,8 +128,10 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
     const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
     const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
 
-    const int r0 = m0 + wave * 32;                // first query row of this wave
+    // first query row of this wave, and the first head-dim column it owns
+    const int r0 = m0 + (C::kPair ? (wave >> 1) : wave) * 32;
     const int row = r0 + l32;
+    const int dcol0 = C::kPair ? (wave & 1) * C::DH : 0;
 
     v8 qf[C::KS];
     {
@@ -102,7 +139,7 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
         const T* qrow = qg + (int64_t)row * p.q_row_stride;
 #pragma unroll
         for (int dk = 0; dk < C::KS; dk++) {
-            const int d0 = dk * 16 + 8 * hh;
+            const int d0 = dcol0 + dk * 16 + 8 * hh;
             u32x4 raw = {0, 0, 0, 0};
             if (valid && d0 < p.d) raw = ld_global16(qrow + d0);
             qf[dk] = __builtin_bit_cast(v8, raw);
@@ -181,12 +218,12 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
     // ---- LDS fragment addressing
     int kofs[C::KS];
 #pragma unroll
-    for (int dk = 0; dk < C::KS; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dk * 2 + hh, l32) * 16;
+    for (int dk = 0; dk < C::KS; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dcol0 / 8 + dk * 2 + hh, l32) * 16;
     const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
     int vofs[C::DB];
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
-        vofs[db] = (4 * hh + tj) * C::ROWB + swz_v<D>(db * 4 + dhalf * 2 + (tq >> 1), 4 * hh + tj) * 16 + (tq & 1) * 8;
+        vofs[db] = (4 * hh + tj) * C::ROWB + swz_v<D>(dcol0 / 8 + db * 4 + dhalf * 2 + (tq >> 1), 4 * hh + tj) * 16 + (tq & 1) * 8;
 
     constexpr int LA = FA_IL_LA;
     constexpr int NFV = C::PT * C::DB;             // V fragments in (t16, db) order
@@ -311,6 +348,36 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
         }
     };
 
+    // Pair mode: the partial S tile of step i lives in exchange slot i & 1 of the wave that made it
+    // (same lane, same register order on both sides, so writer and reader use identical addresses).
+    // A slot written at the end of step i-1 is read by the partner at the start of step i and
+    // rewritten at the end of step i+1; the barriers closing steps i-1 and i order the three.
+    auto xch_ptr = [&](int w, int i) { return smem + 2 * C::NS * C::TILE + (w * 2 + (i & 1)) * C::XCH + lane * 16; };
+    auto xch_write = [&](int i, const f32x16 (&s)[C::NB]) __attribute__((always_inline)) {
+        if constexpr (C::kPair) {
+            char* base = xch_ptr(wave, i);
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    const f32x4 v = {s[nb][4 * r4], s[nb][4 * r4 + 1], s[nb][4 * r4 + 2], s[nb][4 * r4 + 3]};
+                    *reinterpret_cast<f32x4*>(base + (nb * 4 + r4) * 1024) = v;
+                }
+        }
+    };
+    auto xch_read_add = [&](int i, f32x16 (&s)[C::NB]) __attribute__((always_inline)) {
+        if constexpr (C::kPair) {
+            const char* base = xch_ptr(wave ^ 1, i);
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(base + (nb * 4 + r4) * 1024);
+                    s[nb][4 * r4] += v[0]; s[nb][4 * r4 + 1] += v[1]; s[nb][4 * r4 + 2] += v[2]; s[nb][4 * r4 + 3] += v[3];
+                }
+        }
+    };
+
     f32x16 sA[C::NB], sB[C::NB];
     v8 pA[C::PT], pB[C::PT];
 #pragma unroll
@@ -336,7 +403,7 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
     // read LA chunks ahead, and a slice of the softmax of S(i) (running max in the first chunks,
     // then the decision about the reference max, then the exponentials two at a time).  Scheduling
     // barriers between the chunks keep the compiler from regrouping them.
-    auto fast_step = [&](int i, const f32x16 (&s_cur)[C::NB], f32x16 (&s_nxt)[C::NB], const v8 (&p_prev)[C::PT],
+    auto fast_step = [&](int i, f32x16 (&s_cur)[C::NB], f32x16 (&s_nxt)[C::NB], const v8 (&p_prev)[C::PT],
                          v8 (&p_cur)[C::PT]) __attribute__((always_inline)) {
         constexpr int NF = NFV + NFK;
         constexpr int NE = C::NB * 16;             // S elements per lane
@@ -346,6 +413,7 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
         constexpr int CE = CD + 1;                 // first chunk with exponentials
         static_assert(NF > CE + 1, "tile too small for the chunked step");
         open_step(i);
+        xch_read_add(i, s_cur);
         // an opaque copy of the scale keeps the vector work in this block (behind the barrier)
         float sc = sl2;
         asm volatile("" : "+v"(sc));
@@ -431,14 +499,19 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
         }
         asm volatile("" : "+v"(l_run));
         rescale(corr, move);
+        xch_write(i + 1, s_nxt);
         advance_ring(i);
     };
     // Plain step (first, last and masked tiles): the same pieces one after the other; S stays in sA
     // and P in pA.
     auto plain_step = [&](int i) __attribute__((always_inline)) {
         open_step(i);
+        xch_read_add(i, sA);
         if (i > 0) mma(std::true_type(), std::false_type(), i - 1, 0, pA, sB);
-        if (i + 1 < nt) mma(std::false_type(), std::true_type(), 0, i + 1, pA, sB);
+        if (i + 1 < nt) {
+            mma(std::false_type(), std::true_type(), 0, i + 1, pA, sB);
+            xch_write(i + 1, sB);
+        }
         mask_tile(i, sA);
         float corr; bool move;
         probs(sA, pA, corr, move, sl2);
@@ -455,6 +528,7 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
         wait_vmcnt<0>();
         __syncthreads();
         mma(std::false_type(), std::true_type(), 0, 0, pA, sA);
+        xch_write(0, sA);
         __syncthreads();      // K(0)'s ring slot is refilled when step 0 opens
 
         // steps [i_fb, i_fe) visit tiles that need no masking for this wave, an even number of them
@@ -477,11 +551,12 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
     const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
     const float inv = dead ? 1.f : 1.f / l_tot;
     const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
-    if (hh == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
-    // output tile of the wave through LDS (whole rows per store instruction); all ring reads are
+    if (hh == 0 && dcol0 == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
+    // output tile of the wave (32 rows x DH columns) through LDS (whole rows per store instruction); all ring reads are
     // behind the last barrier and each wave uses its own region
     {
-        constexpr int PITCH = C::ROWB + 16;
+        constexpr int PITCH = C::DH * 2 + 16;
+        constexpr int OCPR = C::DH / 8;                 // 16 B chunks per output row of the wave
         static_assert(C::kWaves * 32 * PITCH <= C::SMEM, "staging region");
         char* stage = smem + wave * (32 * PITCH);
 #pragma unroll
@@ -493,32 +568,36 @@ __global__ void __launch_bounds__(256, 2) prefill_il_kernel(const KParams kp) {
                                  pack2<T>(o_acc[db][4 * q4 + 2] * inv, o_acc[db][4 * q4 + 3] * inv)};
                 *reinterpret_cast<u32x2*>(stage + l32 * PITCH + d0 * 2) = v;
             }
-        constexpr int RPP = 64 / C::CPR;
-        const int srow = lane / C::CPR, sch = lane % C::CPR;
-        T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + sch * 8;
+        constexpr int RPP = 64 / OCPR;
+        const int srow = lane / OCPR, sch = lane % OCPR;
+        T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + dcol0 + sch * 8;
 #pragma unroll
         for (int j = 0; j < 32 / RPP; j++) {
             const int rr = j * RPP + srow;
             const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
-            if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
+            if (r0 + rr < si.sq && dcol0 + sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
         }
     }
 }
 
-template <typename T, int D, int BN>
-int launch_prefill_il(KParams kp, hipStream_t stream) {
-    typedef ILCfg<T, D, BN> C;
+template <typename T, typename C>
+int launch_prefill_il_cfg(KParams kp, hipStream_t stream) {
     kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
     if (total <= 0) return 0;
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
     dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
-    auto kern = prefill_il_kernel<T, D, BN>;
+    auto kern = prefill_il_kernel<T, C>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
+
+template <typename T, int D, int BN>
+int launch_prefill_il(const KParams& kp, hipStream_t stream) { return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream); }
+template <typename T>
+int launch_prefill_il_pair(const KParams& kp, hipStream_t stream) { return launch_prefill_il_cfg<T, ILCfgPair<T>>(kp, stream); }
 
 }  // namespace fa

@@ -3,7 +3,9 @@ the split path): at least 512 query rows and at least 256 row blocks in the laun
 
   * software-pipelined kernel (fa_prefill_il.h): head dim <= 64 at any length, head dim <= 128 up to
     4096 keys (causal / windowed) or 2048 keys (full attention);
-  * ping-pong kernel (fa_prefill_pp.h): head dim 65..128 beyond those key counts.
+  * ping-pong kernel (fa_prefill_pp.h): head dim 65..128 beyond those key counts;
+  * the pair form of the software-pipelined kernel (two waves split the head dimension): head dim
+    129..256.
 
 Cases follow the reference's own test dimensions (tests/test_flash_attn.py:530-657, 1295-1402): ragged
 lengths, seqlen_q != seqlen_k both ways, causal / local masks, MQA/GQA, padded head dims, fp16 and
@@ -104,7 +106,21 @@ def test_pingpong_kernel(case):
     _check(out, lse, q, k, v, causal=causal, window_size=window)
 
 
-@pytest.mark.parametrize("s,d", [(1024, 64), (2304, 128)])
+@pytest.mark.parametrize("d", [136, 160, 192, 224, 256])
+@pytest.mark.parametrize("sq,sk,mode", [(777, 777, "causal"), (512, 512, "full"), (600, 1500, "causal"),
+                                         (1500, 600, "local"), (1024, 1024, "local")])
+def test_pair_kernel_head_dims_above_128(d, sq, sk, mode):
+    _say("pair kernel", d, sq, sk, mode)
+    dtype = torch.float16 if d in (160, 224) else torch.bfloat16
+    b, h, hk = 4, 16, 2
+    q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
+    window = _window(mode, sk, d * 31 + sq)
+    out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
+                                        window_size=window, return_attn_probs=True)
+    _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
+
+
+@pytest.mark.parametrize("s,d", [(1024, 64), (2304, 128), (1024, 256)])
 def test_long_kernels_take_strided_packed_input(s, d):
     """q, k, v as strided views of one (b, s, 3, h, d) tensor: row stride 3*h*d."""
     _say("packed long", s, d)
@@ -115,7 +131,7 @@ def test_long_kernels_take_strided_packed_input(s, d):
     _check(out, lse, qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], causal=True)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 256])
 def test_varlen_long_with_empty_and_tiny_sequences(d):
     _say("varlen long", d)
     dtype, h = torch.bfloat16, 16
