@@ -37,6 +37,7 @@ def units():
                       ["-DFA_T_BF16=%d" % bf, "-DFA_D=%d" % d]))
     u.append(("fa_decode.hip", "decode.o", []))
     u.append(("fa_aux.hip", "aux.o", []))
+    u.append(("fa_rotary.hip", "rotary.o", []))
     u.append(("fa_api.hip", "api.o", []))
     return u
 

@@ -23,6 +23,7 @@ _LIB_PATH = os.environ.get("FLASH_ATTN_MI355X_LIB") or os.path.join(_HERE, "libf
 
 FA_DTYPE_FP16 = 0
 FA_DTYPE_BF16 = 1
+FA_DTYPE_FP32 = 2
 
 
 class FaFwdParams(ctypes.Structure):
@@ -43,6 +44,19 @@ class FaFwdParams(ctypes.Structure):
             "window_left", "window_right", "is_causal", "is_seqlens_k_cumulative",
             "is_rotary_interleaved", "num_splits", "dtype")]
         + [("softmax_scale", ctypes.c_float)]
+    )
+
+
+class FaRotaryParams(ctypes.Structure):
+    """Mirror of `fa_rotary_params` in include/fa_mi355x.h (field order matters)."""
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in ("x", "out", "cos", "sin", "cu_seqlens", "seqlen_offsets")]
+        + [(n, ctypes.c_int64) for n in (
+            "x_batch_stride", "x_row_stride", "x_head_stride",
+            "o_batch_stride", "o_row_stride", "o_head_stride", "cs_row_stride")]
+        + [(n, ctypes.c_int32) for n in (
+            "b", "seqlen", "h", "d", "rotary_dim", "seqlen_ro", "seqlen_offset",
+            "interleaved", "conjugate", "dtype", "cs_dtype")]
     )
 
 
@@ -67,6 +81,13 @@ def _load():
     lib.fa_version.restype = ctypes.c_int32
     lib.fa_sizeof_params.argtypes = []
     lib.fa_sizeof_params.restype = ctypes.c_int32
+    lib.fa_rotary.argtypes = [ctypes.POINTER(FaRotaryParams), ctypes.c_void_p]
+    lib.fa_rotary.restype = ctypes.c_int
+    lib.fa_sizeof_rotary_params.argtypes = []
+    lib.fa_sizeof_rotary_params.restype = ctypes.c_int32
+    if lib.fa_sizeof_rotary_params() != ctypes.sizeof(FaRotaryParams):
+        raise ImportError("flash_attn: fa_rotary_params layout mismatch between %s and its Python mirror; "
+                          "rebuild the library" % _LIB_PATH)
     if lib.fa_sizeof_params() != ctypes.sizeof(FaFwdParams):
         raise ImportError("flash_attn: fa_fwd_params layout mismatch between %s (%d bytes) and its "
                           "Python mirror (%d bytes); rebuild the library" %

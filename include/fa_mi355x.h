@@ -21,6 +21,7 @@ extern "C" {
 
 #define FA_DTYPE_FP16 0
 #define FA_DTYPE_BF16 1
+#define FA_DTYPE_FP32 2   /* rotary tables only */
 
 #define FA_MAX_SPLITS 128
 
@@ -135,6 +136,40 @@ int32_t fa_version(void);
 /* sizeof(fa_fwd_params) as the library was compiled: lets a foreign-language binding verify its
  * mirror of the struct.  No counterpart in the reference (pybind11 passes tensors). */
 int32_t fa_sizeof_params(void);
+
+/*
+ * Standalone rotary embedding: out[..., :rotary_dim] = x * cos + rotate_half(x) * sin per
+ * (token, head) row, remaining columns copied through; math in fp32, one rounding to the dtype of
+ * x.  Replaces the reference's Triton op apply_rotary (flash_attn/ops/triton/rotary.py:144-240)
+ * behind apply_rotary_emb (flash_attn/layers/rotary.py:34-124): same arguments.
+ *   x, out        (b, seqlen, h, d) with the strides below, or packed (total, h, d) when
+ *                 cu_seqlens != NULL (then seqlen = max_seqlen); out may be x (in place)
+ *   cos, sin      (seqlen_ro, rotary_dim/2), row stride cs_row_stride, dtype cs_dtype
+ *   position of token t of batch entry i: t + (seqlen_offsets ? seqlen_offsets[i] : seqlen_offset);
+ *                 positions outside the table leave the row unrotated
+ *   interleaved   pairs (2i, 2i+1) instead of (i, i + rotary_dim/2)
+ *   conjugate     rotate by -angle (the backward of the operation)
+ * d % 8 == 0, rotary_dim % 16 == 0, rotary_dim <= d.
+ */
+typedef struct fa_rotary_params {
+    const void *x;
+    void *out;
+    const void *cos, *sin;
+    const int32_t *cu_seqlens;       /* (b+1) or NULL */
+    const int32_t *seqlen_offsets;   /* (b) or NULL */
+    int64_t x_batch_stride, x_row_stride, x_head_stride;
+    int64_t o_batch_stride, o_row_stride, o_head_stride;
+    int64_t cs_row_stride;
+    int32_t b, seqlen, h, d, rotary_dim, seqlen_ro, seqlen_offset;
+    int32_t interleaved, conjugate;
+    int32_t dtype;                   /* FA_DTYPE_FP16 / FA_DTYPE_BF16 */
+    int32_t cs_dtype;                /* FA_DTYPE_FP16 / FA_DTYPE_BF16 / FA_DTYPE_FP32 */
+} fa_rotary_params;
+
+int fa_rotary(const fa_rotary_params *p, void *hip_stream);
+
+/* sizeof(fa_rotary_params) as compiled, for foreign-language bindings (no reference counterpart). */
+int32_t fa_sizeof_rotary_params(void);
 
 #ifdef __cplusplus
 }
