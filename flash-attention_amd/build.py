@@ -35,6 +35,8 @@ def units():
         for d in (64, 128, 256):
             u.append(("fa_prefill_inst.hip", "prefill_%s_%d.o" % ("bf16" if bf else "fp16", d),
                       ["-DFA_T_BF16=%d" % bf, "-DFA_D=%d" % d]))
+            u.append(("fa_bwd_inst.hip", "bwd_%s_%d.o" % ("bf16" if bf else "fp16", d),
+                      ["-DFA_T_BF16=%d" % bf, "-DFA_D=%d" % d]))
     u.append(("fa_decode.hip", "decode.o", []))
     u.append(("fa_aux.hip", "aux.o", []))
     u.append(("fa_rotary.hip", "rotary.o", []))

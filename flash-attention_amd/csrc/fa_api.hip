@@ -9,6 +9,7 @@
 #include <vector>
 #include <algorithm>
 #include "fa_prefill.h"
+#include "fa_bwd.h"
 #include "fa_launch.h"
 
 namespace fa {
@@ -171,6 +172,50 @@ static int resolve_splits(KParams& kp, const fa_fwd_params& p, bool allow_split)
     return 0;
 }
 
+// Backward: host-side counterpart of mha_bwd / mha_varlen_bwd after tensor unpacking
+// (flash_api.cpp:609-832, 834-1036) and of run_mha_bwd's dispatch (:587-607).
+static int run_bwd(const fa_bwd_params* p, bool varlen, hipStream_t stream) {
+    if (!p) return fail("params is NULL");
+    if (!p->dout || !p->q || !p->k || !p->v || !p->out || !p->softmax_lse || !p->dq || !p->dk || !p->dv || !p->softmax_d)
+        return fail("dout, q, k, v, out, softmax_lse, dq, dk, dv and softmax_d must be set");
+    if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return fail("FlashAttention only support fp16 and bf16 data type");
+    if (p->b <= 0) return fail("batch size must be positive");
+    if (p->d <= 0 || p->d > 256) return fail("FlashAttention backward only supports head dimension at most 256");
+    if (p->d % 8 != 0) return fail("head_size should be a multiple of 8");
+    if (p->h <= 0 || p->h_k <= 0 || p->h % p->h_k != 0) return fail("Number of heads in key/value must divide number of heads in query");
+    if (p->seqlen_q < 0 || p->seqlen_k < 0) return fail("sequence lengths must be non-negative");
+    if (p->seqlen_q_rounded < p->seqlen_q) return fail("seqlen_q_rounded must be at least seqlen_q");
+    if (varlen && (!p->cu_seqlens_q || !p->cu_seqlens_k)) return fail("fa_varlen_bwd needs cu_seqlens_q and cu_seqlens_k");
+    if (!varlen && (p->cu_seqlens_q || p->cu_seqlens_k)) return fail("fa_bwd takes dense batches; use fa_varlen_bwd");
+    const int64_t strides[] = {p->q_row_stride, p->q_head_stride, p->k_row_stride, p->k_head_stride, p->v_row_stride,
+                               p->v_head_stride, p->o_row_stride, p->o_head_stride, p->do_row_stride, p->do_head_stride,
+                               p->dq_row_stride, p->dq_head_stride, p->dk_row_stride, p->dk_head_stride,
+                               p->dv_row_stride, p->dv_head_stride, p->q_batch_stride, p->k_batch_stride, p->v_batch_stride,
+                               p->o_batch_stride, p->do_batch_stride, p->dq_batch_stride, p->dk_batch_stride, p->dv_batch_stride};
+    for (int64_t st : strides) if (st % 4 != 0) return fail("strides must be multiples of 4 elements");
+    const int64_t in_strides[] = {p->q_row_stride, p->q_head_stride, p->k_row_stride, p->k_head_stride, p->v_row_stride,
+                                  p->v_head_stride, p->o_row_stride, p->o_head_stride, p->do_row_stride, p->do_head_stride,
+                                  p->q_batch_stride, p->k_batch_stride, p->v_batch_stride, p->o_batch_stride, p->do_batch_stride};
+    for (int64_t st : in_strides) if (st % 8 != 0) return fail("input strides must be multiples of 8 elements (16-byte rows)");
+
+    BwdKParams kp;
+    kp.p = *p;
+    if (kp.p.is_causal) kp.p.window_right = 0;     // flash_api.cpp:627
+    kp.has_left = kp.p.window_left >= 0;
+    kp.has_right = kp.p.window_right >= 0;
+    kp.scale_log2 = p->softmax_scale * (float)M_LOG2E;
+    const bool bf = p->dtype == FA_DTYPE_BF16;
+    int e = bf ? launch_bwd_dot_bf16(kp, stream) : launch_bwd_dot_fp16(kp, stream);
+    if (e) return fail_hip(e, "backward preprocess kernel launch");
+    switch (bucket(p->d)) {
+        case 64: e = bf ? launch_bwd_bf16_64(kp, stream) : launch_bwd_fp16_64(kp, stream); break;
+        case 128: e = bf ? launch_bwd_bf16_128(kp, stream) : launch_bwd_fp16_128(kp, stream); break;
+        default: e = bf ? launch_bwd_bf16_256(kp, stream) : launch_bwd_fp16_256(kp, stream); break;
+    }
+    if (e) return fail_hip(e, "backward kernel launch");
+    return 0;
+}
+
 }  // namespace fa
 
 using namespace fa;
@@ -293,6 +338,18 @@ int fa_rotary(const fa_rotary_params* p, void* hip_stream) {
     for (const void* q : ptrs) if ((uintptr_t)q % 16 != 0) return fail("rotary needs 16-byte aligned x, out, cos and sin");
     if (int e = launch_rotary(*p, (hipStream_t)hip_stream)) return fail_hip(e, "rotary kernel launch");
     return 0;
+}
+
+int32_t fa_sizeof_bwd_params(void) { return (int32_t)sizeof(fa_bwd_params); }
+
+int fa_bwd(const fa_bwd_params* p, void* hip_stream) {
+    g_err.clear();
+    return run_bwd(p, false, (hipStream_t)hip_stream);
+}
+
+int fa_varlen_bwd(const fa_bwd_params* p, void* hip_stream) {
+    g_err.clear();
+    return run_bwd(p, true, (hipStream_t)hip_stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,550 @@
+// Backward kernels for gfx950: dQ by one pass over query tiles, dK / dV by one pass over key tiles.
+// Counterpart of the reference's compute_dq_dk_dv_1colblock (csrc/flash_attn/src/flash_bwd_kernel.h:
+// 79-780) and its dot_do_o / convert_dQ passes (flash_bwd_preprocess_kernel.h), re-designed so that
+// nothing is accumulated through global atomics and no fp32 dq buffer exists:
+//
+//   D_i   = sum_d dO[i,d] O[i,d]                                   (bwd_dot_kernel)
+//   P     = exp(scale * Q K^T - lse),   dP = dO V^T,   dS = P o (dP - D)
+//   dQ    = scale * dS K                                           (bwd_dq_kernel: per query tile)
+//   dV    = P^T dO,   dK = scale * dS^T Q                          (bwd_dkv_kernel: per key tile)
+//
+// Both kernels keep the forward kernels' register geometry: every product is computed TRANSPOSED with
+// v_mfma_f32_32x32x16 so that the accumulator gives each lane ONE row of the resident operand (a
+// query row in the dQ kernel, a key row in the dK/dV kernel) and 16 rows of the streamed tile; the
+// accumulator layout is then already the B-operand layout of the next product, so P and dS never
+// leave registers.  Streamed tiles are read from LDS twice, row-wise (ds_read_b128) as the A operand
+// of the score-shaped products and transposed (ds_read_b64_tr_b16) as the A operand of the
+// gradient-shaped ones; one swizzle (swz_u) keeps both conflict free.  The sum of dK / dV over the
+// query heads of a GQA group is a loop inside the key-tile kernel.
+#pragma once
+#include "fa_common.h"
+
+namespace fa {
+
+struct BwdKParams {
+    fa_bwd_params p;
+    float scale_log2;             // softmax_scale * log2(e)
+    int32_t has_left, has_right;  // window bounds active (after causal normalisation)
+};
+
+struct BwdSeq {
+    int sq, sk;
+    int64_t q_off, k_off, v_off, o_off, do_off, dq_off, dk_off, dv_off;   // element offsets of (row 0, head 0)
+};
+FA_DEV BwdSeq bwd_seq(const fa_bwd_params& p, int b) {
+    BwdSeq s;
+    if (p.cu_seqlens_q) {
+        const int64_t r0 = p.cu_seqlens_q[b];
+        s.sq = p.cu_seqlens_q[b + 1] - (int)r0;
+        s.q_off = r0 * p.q_row_stride; s.o_off = r0 * p.o_row_stride;
+        s.do_off = r0 * p.do_row_stride; s.dq_off = r0 * p.dq_row_stride;
+    } else {
+        s.sq = p.seqlen_q;
+        s.q_off = (int64_t)b * p.q_batch_stride; s.o_off = (int64_t)b * p.o_batch_stride;
+        s.do_off = (int64_t)b * p.do_batch_stride; s.dq_off = (int64_t)b * p.dq_batch_stride;
+    }
+    if (p.cu_seqlens_k) {
+        const int64_t r0 = p.cu_seqlens_k[b];
+        s.sk = p.cu_seqlens_k[b + 1] - (int)r0;
+        s.k_off = r0 * p.k_row_stride; s.v_off = r0 * p.v_row_stride;
+        s.dk_off = r0 * p.dk_row_stride; s.dv_off = r0 * p.dv_row_stride;
+    } else {
+        s.sk = p.seqlen_k;
+        s.k_off = (int64_t)b * p.k_batch_stride; s.v_off = (int64_t)b * p.v_batch_stride;
+        s.dk_off = (int64_t)b * p.dk_batch_stride; s.dv_off = (int64_t)b * p.dv_batch_stride;
+    }
+    return s;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// A operand, row-wise: rows [row0, row0+32) of a swizzled tile, columns [16 dk, 16 dk + 16)
+template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_a_rows(const char* tile, int row, int dk, int hh) {
+    const int c = dk * 2 + hh;
+    const u32x4 raw = *reinterpret_cast<const u32x4*>(tile + row * (D * 2) + swz_u<D>(c, row) * 16);
+    return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+// A operand, transposed: columns [32 db, 32 db + 32) of tile rows [16 t16, 16 t16 + 16), in the row
+// order that matches a packed accumulator (rows 4hh..4hh+3 and 8+4hh..8+4hh+3 of the 16)
+template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_a_cols(const char* tile, int t16, int db, int lane) {
+    const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1, hh = lane >> 5;
+    const int row = t16 * 16 + 4 * hh + tj;
+    const int c = db * 4 + dhalf * 2 + (tq >> 1);
+    const u32x2 lo = lds_read_tr16(tile + row * (D * 2) + swz_u<D>(c, row) * 16 + (tq & 1) * 8);
+    const u32x2 hi = lds_read_tr16(tile + (row + 8) * (D * 2) + swz_u<D>(c, row + 8) * 16 + (tq & 1) * 8);
+    const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+// accumulator registers [r8, r8+8) -> B operand of the next product
+template <typename T> FA_DEV typename Elem<T>::v8 pack_acc8(const f32x16& a, int r8) {
+    u32x4 pk;
+#pragma unroll
+    for (int e = 0; e < 4; e++) pk[e] = pack2<T>(a[r8 + 2 * e], a[r8 + 2 * e + 1]);
+    return __builtin_bit_cast(typename Elem<T>::v8, pk);
+}
+
+// ------------------------------------------------------------------------------------------------
+// D_i = rowsum(dO o O).  16 lanes per (row, head); HBM-bound, reads dO and O once.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdKParams kp) {
+    const fa_bwd_params& p = kp.p;
+    const int b = blockIdx.z, head = blockIdx.y;
+    const int row = blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int sub = threadIdx.x & 15;
+    const BwdSeq si = bwd_seq(p, b);
+    float acc = 0.f;
+    if (row < si.sq) {
+        const T* o = reinterpret_cast<const T*>(p.out) + si.o_off + (int64_t)row * p.o_row_stride + (int64_t)head * p.o_head_stride;
+        const T* g = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)row * p.do_row_stride + (int64_t)head * p.do_head_stride;
+        for (int c = sub; c * 8 < p.d; c += 16) {
+            float a[8], bb[8];
+            unpack8<T>(ld_global16(o + c * 8), a);
+            unpack8<T>(ld_global16(g + c * 8), bb);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc += a[e] * bb[e];
+        }
+    }
+#pragma unroll
+    for (int m = 8; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 16);
+    if (sub == 0 && row < p.seqlen_q_rounded)
+        p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + row] = row < si.sq ? acc : 0.f;
+}
+
+// ------------------------------------------------------------------------------------------------
+// dQ: a workgroup owns 128 query rows of one (batch, head) and streams K / V tiles of BN keys.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int D, int BN>
+struct BwdDqCfg {
+    static constexpr int kThreads = 256, kWaves = 4, BM = 128;
+    static constexpr int NB = BN / 32, KS = D / 16, DB = D / 32, PT = BN / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int TILE_BYTES = BN * ROWB;
+    static constexpr int LOADS = BN * CPR / kThreads;
+    static constexpr int SMEM = 4 * TILE_BYTES;   // {K, V} x 2 stages
+    static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
+};
+
+template <typename T, int D, int BN, int MINW>
+__global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) {
+    typedef BwdDqCfg<T, D, BN> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_bwd_params& p = kp.p;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+
+    // logical order: heads of one group adjacent, then query tiles, then kv heads, then batch; runs of
+    // the order go to one XCD so that workgroups streaming the same K / V share an L2
+    const int G = p.h / p.h_k;
+    const int num_m_blocks = (p.seqlen_q + C::BM - 1) / C::BM;
+    const int64_t total = (int64_t)num_m_blocks * p.h * p.b;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int g = (int)(w % G); w /= G;
+    const int mb = num_m_blocks - 1 - (int)(w % num_m_blocks); w /= num_m_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+    const int head = hk * G + g;
+
+    const BwdSeq si = bwd_seq(p, b);
+    const int m0 = mb * C::BM;
+    if (m0 >= si.sq) return;
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    int n_hi = si.sk;
+    if (has_right) n_hi = min(n_hi, min(m0 + C::BM, si.sq) + shift + wr);
+    const int n_lo = has_left ? max(0, m0 + shift - wl) : 0;
+    const int t_lo = n_lo / BN;
+    const int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
+
+    const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
+    const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
+
+    // resident operands: this lane's query row of Q and dO, its log-sum-exp and D
+    const int r0w = m0 + wave * 32;
+    const int row = r0w + l32;
+    const bool row_ok = row < si.sq;
+    v8 qf[C::KS], gf[C::KS];
+    {
+        const T* qrow = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)row * p.q_row_stride + (int64_t)head * p.q_head_stride;
+        const T* grow = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)row * p.do_row_stride + (int64_t)head * p.do_head_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 a = {0, 0, 0, 0}, c = {0, 0, 0, 0};
+            if (row_ok && d0 < p.d) { a = ld_global16(qrow + d0); c = ld_global16(grow + d0); }
+            qf[dk] = __builtin_bit_cast(v8, a);
+            gf[dk] = __builtin_bit_cast(v8, c);
+        }
+    }
+    // a row beyond the sequence, or one that saw no key (lse = +inf), gets P = exp2(-inf) = 0
+    const float lse2 = row_ok ? p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] * kLog2e : INFINITY;
+    const float dsum = row_ok ? p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + row] : 0.f;
+
+    f32x16 dq_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dq_acc[db][r] = 0.f;
+
+    u32x4 kr[C::LOADS], vr[C::LOADS];
+    const int d_last_chunk = p.d / 8 - 1;
+    auto load_tile = [&](int t) {
+        const int n0 = t * BN;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
+            const int n = min(n0 + r, si.sk - 1);
+            kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
+            vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
+        }
+    };
+    auto store_tile = [&](int buf, int t) {
+        char* kb = smem + buf * 2 * C::TILE_BYTES;
+        char* vb = kb + C::TILE_BYTES;
+        const int n0 = t * BN;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = f % C::CPR;
+            const bool ok = (n0 + r < si.sk) && (c <= d_last_chunk);
+            const u32x4 z = {0, 0, 0, 0};
+            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
+            *reinterpret_cast<u32x4*>(kb + off) = ok ? kr[i] : z;
+            *reinterpret_cast<u32x4*>(vb + off) = ok ? vr[i] : z;
+        }
+    };
+
+    const float sl2 = kp.scale_log2;
+    if (t_hi > t_lo) { load_tile(t_lo); store_tile(0, t_lo); }
+    __syncthreads();
+    int buf = 0;
+    for (int t = t_lo; t < t_hi; ++t) {
+        const bool has_next = t + 1 < t_hi;
+        if (has_next) load_tile(t + 1);
+        const int n0 = t * BN;
+        const char* kb = smem + buf * 2 * C::TILE_BYTES;
+        const char* vb = kb + C::TILE_BYTES;
+        const bool skip = (has_right && n0 > r0w + 31 + shift + wr) || (has_left && n0 + BN - 1 < r0w + shift - wl) ||
+                          (r0w >= si.sq);
+        if (!skip) {
+            f32x16 s_acc[C::NB], dp_acc[C::NB];
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) { s_acc[nb][r] = 0.f; dp_acc[nb][r] = 0.f; }
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                for (int dk = 0; dk < C::KS; dk++) {
+                    s_acc[nb] = Elem<T>::mfma32(lds_a_rows<T, D>(kb, nb * 32 + l32, dk, hh), qf[dk], s_acc[nb]);
+                    dp_acc[nb] = Elem<T>::mfma32(lds_a_rows<T, D>(vb, nb * 32 + l32, dk, hh), gf[dk], dp_acc[nb]);
+                }
+            const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0w + shift + wr) ||
+                                   (has_left && n0 < r0w + 31 + shift - wl);
+            if (need_mask) {
+                int lim_hi = si.sk - 1;
+                if (has_right) lim_hi = min(lim_hi, row + shift + wr);
+                const int lim_lo = has_left ? row + shift - wl : 0;
+#pragma unroll
+                for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                        if (n > lim_hi || n < lim_lo) s_acc[nb][r] = -INFINITY;
+                    }
+            }
+            v8 dsf[C::PT];
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float pv = fast_exp2(s_acc[nb][r] * sl2 - lse2);
+                    s_acc[nb][r] = pv * (dp_acc[nb][r] - dsum);
+                }
+                dsf[2 * nb] = pack_acc8<T>(s_acc[nb], 0);
+                dsf[2 * nb + 1] = pack_acc8<T>(s_acc[nb], 8);
+            }
+            // dQ^T += K^T dS^T
+#pragma unroll
+            for (int t16 = 0; t16 < C::PT; t16++)
+#pragma unroll
+                for (int db = 0; db < C::DB; db++)
+                    dq_acc[db] = Elem<T>::mfma32(lds_a_cols<T, D>(kb, t16, db, lane), dsf[t16], dq_acc[db]);
+        }
+        if (has_next) store_tile(buf ^ 1, t + 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    if (!row_ok) return;
+    T* orow = reinterpret_cast<T*>(p.dq) + si.dq_off + (int64_t)row * p.dq_row_stride + (int64_t)head * p.dq_head_stride;
+    const float sc = p.softmax_scale;
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const int d0 = db * 32 + 8 * q4 + 4 * hh;
+            if (d0 < p.d) {
+                u32x2 v = {pack2<T>(dq_acc[db][4 * q4] * sc, dq_acc[db][4 * q4 + 1] * sc),
+                           pack2<T>(dq_acc[db][4 * q4 + 2] * sc, dq_acc[db][4 * q4 + 3] * sc)};
+                st_global8(orow + d0, v);
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK, dV: a workgroup owns 128 keys of one (batch, kv head) and streams the Q / dO tiles (BM query
+// rows) of every query head of the group.  With DPARTS = 2 a workgroup accumulates only half of the
+// head dimension (the scores are computed in full by both halves): head dim 256 would otherwise
+// need more than 512 registers per lane.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int D, int BM, int DPARTS>
+struct BwdDkvCfg {
+    static constexpr int kThreads = 256, kWaves = 4, BNW = 128;
+    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32 / DPARTS, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int TILE_BYTES = BM * ROWB;
+    static constexpr int LOADS = BM * CPR / kThreads;
+    static constexpr int STAGE = 2 * TILE_BYTES + 2 * BM * 4;   // Q, dO, lse (log2 units), D
+    static constexpr int SMEM = 2 * STAGE;
+    static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
+};
+
+template <typename T, int D, int BM, int DPARTS, int MINW>
+__global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp) {
+    typedef BwdDkvCfg<T, D, BM, DPARTS> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_bwd_params& p = kp.p;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+
+    const int G = p.h / p.h_k;
+    const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
+    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b * DPARTS;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int dpart = (int)(w % DPARTS); w /= DPARTS;
+    const int nblk = (int)(w % num_n_blocks); w /= num_n_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+
+    const BwdSeq si = bwd_seq(p, b);
+    const int n0 = nblk * C::BNW;
+    if (n0 >= si.sk) return;
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    // query rows that see at least one of this workgroup's keys
+    int i_lo = 0, i_hi = si.sq;
+    if (has_right) i_lo = max(0, n0 - shift - wr);
+    if (has_left) i_hi = min(si.sq, min(n0 + C::BNW, si.sk) - shift + wl);
+    const int t_lo = i_lo / BM;
+    const int t_hi = i_hi > i_lo ? (i_hi + BM - 1) / BM : t_lo;
+    const int nt = t_hi - t_lo;
+    const int iters = nt * G;
+
+    // resident operands: this lane's key row of K and V
+    const int j0w = n0 + wave * 32;
+    const int key = j0w + l32;
+    const bool key_ok = key < si.sk;
+    v8 kf[C::KS], vf[C::KS];
+    {
+        const T* krow = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)key * p.k_row_stride + (int64_t)hk * p.k_head_stride;
+        const T* vrow = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)key * p.v_row_stride + (int64_t)hk * p.v_head_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 a = {0, 0, 0, 0}, c = {0, 0, 0, 0};
+            if (key_ok && d0 < p.d) { a = ld_global16(krow + d0); c = ld_global16(vrow + d0); }
+            kf[dk] = __builtin_bit_cast(v8, a);
+            vf[dk] = __builtin_bit_cast(v8, c);
+        }
+    }
+
+    f32x16 dk_acc[C::DB], dv_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) { dk_acc[db][r] = 0.f; dv_acc[db][r] = 0.f; }
+
+    u32x4 qr[C::LOADS], gr[C::LOADS];
+    float aux = 0.f;
+    const int d_last_chunk = p.d / 8 - 1;
+    auto load_tile = [&](int it) {
+        const int head = hk * G + it / nt;
+        const int i0 = (t_lo + it % nt) * BM;
+        const T* qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
+        const T* gg = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
+            const int n = min(i0 + r, si.sq - 1);
+            qr[i] = ld_global16(qg + (int64_t)n * p.q_row_stride + c * 8);
+            gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
+        }
+        if (tid < 2 * BM) {
+            const int r = i0 + (tid < BM ? tid : tid - BM);
+            if (r < si.sq)
+                aux = tid < BM ? p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + r] * kLog2e
+                               : p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + r];
+            else
+                aux = tid < BM ? INFINITY : 0.f;
+        }
+    };
+    auto store_tile = [&](int buf, int it) {
+        char* qb = smem + buf * C::STAGE;
+        char* gb = qb + C::TILE_BYTES;
+        const int i0 = (t_lo + it % nt) * BM;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = f % C::CPR;
+            const bool ok = (i0 + r < si.sq) && (c <= d_last_chunk);
+            const u32x4 z = {0, 0, 0, 0};
+            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
+            *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
+            *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
+        }
+        if (tid < 2 * BM) reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = aux;
+    };
+
+    const float sl2 = kp.scale_log2;
+    if (iters > 0) { load_tile(0); store_tile(0, 0); }
+    __syncthreads();
+    int buf = 0;
+    for (int it = 0; it < iters; ++it) {
+        const bool has_next = it + 1 < iters;
+        if (has_next) load_tile(it + 1);
+        const int i0 = (t_lo + it % nt) * BM;
+        const char* qb = smem + buf * C::STAGE;
+        const char* gb = qb + C::TILE_BYTES;
+        const float* lse_s = reinterpret_cast<const float*>(gb + C::TILE_BYTES);
+        const float* dsum_s = lse_s + BM;
+
+        // keys of this wave against the rows of the tile: nothing visible -> nothing to add
+        const bool wave_skip = (has_right && j0w > i0 + BM - 1 + shift + wr) || (has_left && j0w + 31 < i0 + shift - wl) ||
+                               (j0w >= si.sk);
+        if (!wave_skip) {
+            f32x16 s_acc[C::MBK], dp_acc[C::MBK];
+#pragma unroll
+            for (int mb = 0; mb < C::MBK; mb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) { s_acc[mb][r] = 0.f; dp_acc[mb][r] = 0.f; }
+#pragma unroll
+            for (int mb = 0; mb < C::MBK; mb++)
+#pragma unroll
+                for (int dk = 0; dk < C::KS; dk++) {
+                    s_acc[mb] = Elem<T>::mfma32(lds_a_rows<T, D>(qb, mb * 32 + l32, dk, hh), kf[dk], s_acc[mb]);
+                    dp_acc[mb] = Elem<T>::mfma32(lds_a_rows<T, D>(gb, mb * 32 + l32, dk, hh), vf[dk], dp_acc[mb]);
+                }
+            v8 pf[C::PT], dsf[C::PT];
+#pragma unroll
+            for (int mb = 0; mb < C::MBK; mb++) {
+                const int ib = i0 + mb * 32;
+                const bool need_mask = (has_right && j0w + 31 > ib + shift + wr) || (has_left && j0w < ib + 31 + shift - wl);
+                if (need_mask) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int i = ib + 8 * (r >> 2) + 4 * hh + (r & 3);
+                        const bool hidden = (has_right && key > i + shift + wr) || (has_left && key < i + shift - wl);
+                        if (hidden) s_acc[mb][r] = -INFINITY;
+                    }
+                }
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int r = 4 * q4 + e;
+                        const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
+                        s_acc[mb][r] = pv;
+                        dp_acc[mb][r] = pv * (dp_acc[mb][r] - d4[e]);
+                    }
+                }
+                pf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
+                pf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
+                dsf[2 * mb] = pack_acc8<T>(dp_acc[mb], 0);
+                dsf[2 * mb + 1] = pack_acc8<T>(dp_acc[mb], 8);
+            }
+            // dV^T += dO^T P,  dK^T += Q^T dS   (columns of this workgroup's part of the head dim)
+#pragma unroll
+            for (int t16 = 0; t16 < C::PT; t16++)
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) {
+                    dv_acc[db] = Elem<T>::mfma32(lds_a_cols<T, D>(gb, t16, dpart * C::DB + db, lane), pf[t16], dv_acc[db]);
+                    dk_acc[db] = Elem<T>::mfma32(lds_a_cols<T, D>(qb, t16, dpart * C::DB + db, lane), dsf[t16], dk_acc[db]);
+                }
+        }
+        if (has_next) store_tile(buf ^ 1, it + 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    if (!key_ok) return;
+    T* dkrow = reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride;
+    T* dvrow = reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
+    const float sc = p.softmax_scale;
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const int d0 = (dpart * C::DB + db) * 32 + 8 * q4 + 4 * hh;
+            if (d0 < p.d) {
+                u32x2 a = {pack2<T>(dk_acc[db][4 * q4] * sc, dk_acc[db][4 * q4 + 1] * sc),
+                           pack2<T>(dk_acc[db][4 * q4 + 2] * sc, dk_acc[db][4 * q4 + 3] * sc)};
+                u32x2 c = {pack2<T>(dv_acc[db][4 * q4], dv_acc[db][4 * q4 + 1]),
+                           pack2<T>(dv_acc[db][4 * q4 + 2], dv_acc[db][4 * q4 + 3])};
+                st_global8(dkrow + d0, a);
+                st_global8(dvrow + d0, c);
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------------
+template <typename K> static int bwd_set_smem(K kern, int bytes) {
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+template <typename T, int D, int BN, int MINW>
+int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
+    typedef BwdDqCfg<T, D, BN> C;
+    const int64_t total = (int64_t)((kp.p.seqlen_q + C::BM - 1) / C::BM) * kp.p.h * kp.p.b;
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    auto kern = bwd_dq_kernel<T, D, BN, MINW>;
+    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int D, int BM, int DPARTS, int MINW>
+int launch_bwd_dkv(const BwdKParams& kp, hipStream_t stream) {
+    typedef BwdDkvCfg<T, D, BM, DPARTS> C;
+    const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b * DPARTS;
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    auto kern = bwd_dkv_kernel<T, D, BM, DPARTS, MINW>;
+    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+int launch_bwd_dot(const BwdKParams& kp, hipStream_t stream) {
+    const fa_bwd_params& p = kp.p;
+    if (p.b <= 0 || p.h <= 0 || p.seqlen_q_rounded <= 0) return 0;
+    dim3 grid((unsigned)((p.seqlen_q_rounded + 15) / 16), (unsigned)p.h, (unsigned)p.b);
+    hipLaunchKernelGGL(bwd_dot_kernel<T>, grid, dim3(256), 0, stream, kp);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fa

@@ -1,0 +1,35 @@
+// Backward kernels, one translation unit per (dtype, head-dim bucket): compiled with
+// -DFA_T_BF16=0/1 -DFA_D=64/128/256.
+#include "fa_bwd.h"
+#include "fa_launch.h"
+
+namespace fa {
+#if FA_T_BF16
+typedef __bf16 InstT;
+#define FA_INST_NAME2(d) launch_bwd_bf16_##d
+#else
+typedef _Float16 InstT;
+#define FA_INST_NAME2(d) launch_bwd_fp16_##d
+#endif
+#define FA_INST_NAME(d) FA_INST_NAME2(d)
+
+// dQ pass then dK/dV pass on the same stream; both read softmax_d, which the caller's stream has
+// already filled (launch_bwd_dot).
+int FA_INST_NAME(FA_D)(const BwdKParams& kp, hipStream_t stream) {
+#if FA_D <= 128
+    if (int e = launch_bwd_dq<InstT, FA_D, 64, 1>(kp, stream)) return e;
+    return launch_bwd_dkv<InstT, FA_D, 64, 1, 1>(kp, stream);
+#else
+    if (int e = launch_bwd_dq<InstT, FA_D, 32, 1>(kp, stream)) return e;
+    return launch_bwd_dkv<InstT, FA_D, 32, 2, 1>(kp, stream);
+#endif
+}
+
+#if FA_D == 64
+#if FA_T_BF16
+int launch_bwd_dot_bf16(const BwdKParams& kp, hipStream_t stream) { return launch_bwd_dot<__bf16>(kp, stream); }
+#else
+int launch_bwd_dot_fp16(const BwdKParams& kp, hipStream_t stream) { return launch_bwd_dot<_Float16>(kp, stream); }
+#endif
+#endif
+}  // namespace fa

@@ -115,6 +115,16 @@ template <int D> FA_DEV int swz_v(int chunk, int row) {
     else return chunk;                       // D == 32: four rows fill the 256 B bank window
 }
 
+// One swizzle that serves BOTH read patterns on the same tile (the backward kernels read every
+// streamed tile row-wise as one MFMA operand and transposed as another): a bijection of the rows that
+// share a bank window for the row-wise read, whose upper bits separate the 4 consecutive rows of a
+// transposing read.
+template <int D> FA_DEV int swz_u(int chunk, int row) {
+    if constexpr (D >= 128) return chunk ^ (((row & 3) << 2) | ((row >> 2) & 3));
+    else if constexpr (D == 64) return chunk ^ ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+    else return chunk ^ ((row >> 2) & 3);   // D == 32
+}
+
 // Rotary embedding of 8 consecutive elements [d0, d0+8) of one row, fp32 math.
 // `x` are the row's own values, `row_ptr` points at the row start (to fetch the partner half for
 // the non-interleaved form), cos/sin point at the table row for this token.

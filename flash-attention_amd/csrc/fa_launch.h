@@ -3,6 +3,7 @@
 #include "fa_common.h"
 
 namespace fa {
+struct BwdKParams;
 #define FA_DECL_PREFILL(name) int name(const KParams& kp, hipStream_t stream);
 FA_DECL_PREFILL(launch_prefill_bf16_64)
 FA_DECL_PREFILL(launch_prefill_bf16_128)
@@ -20,4 +21,15 @@ int launch_zero_counter(int32_t* c, hipStream_t stream);     // ticket counter o
 int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials
 int launch_append_kv(const KParams& kp, hipStream_t stream);   // k_new/v_new (+rotary) -> cache
 int launch_rotary(const fa_rotary_params& p, hipStream_t stream);   // standalone rotary embedding
+
+#define FA_DECL_BWD(name) int name(const BwdKParams& kp, hipStream_t stream);
+FA_DECL_BWD(launch_bwd_bf16_64)
+FA_DECL_BWD(launch_bwd_bf16_128)
+FA_DECL_BWD(launch_bwd_bf16_256)
+FA_DECL_BWD(launch_bwd_fp16_64)
+FA_DECL_BWD(launch_bwd_fp16_128)
+FA_DECL_BWD(launch_bwd_fp16_256)
+FA_DECL_BWD(launch_bwd_dot_bf16)    // rowsum(dO o O) -> softmax_d
+FA_DECL_BWD(launch_bwd_dot_fp16)
+#undef FA_DECL_BWD
 }  // namespace fa

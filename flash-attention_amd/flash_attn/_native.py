@@ -60,6 +60,19 @@ class FaRotaryParams(ctypes.Structure):
     )
 
 
+class FaBwdParams(ctypes.Structure):
+    """Mirror of `fa_bwd_params` in include/fa_mi355x.h (field order matters)."""
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in ("dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv",
+                                        "softmax_d", "cu_seqlens_q", "cu_seqlens_k")]
+        + [("%s_%s_stride" % (t, a), ctypes.c_int64) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv")
+           for a in ("batch", "row", "head")]
+        + [(n, ctypes.c_int32) for n in ("b", "seqlen_q", "seqlen_k", "h", "h_k", "d", "seqlen_q_rounded")]
+        + [("softmax_scale", ctypes.c_float)]
+        + [(n, ctypes.c_int32) for n in ("is_causal", "window_left", "window_right", "dtype")]
+    )
+
+
 def _load():
     if not os.path.exists(_LIB_PATH):
         raise ImportError(
@@ -81,6 +94,15 @@ def _load():
     lib.fa_version.restype = ctypes.c_int32
     lib.fa_sizeof_params.argtypes = []
     lib.fa_sizeof_params.restype = ctypes.c_int32
+    for name in ("fa_bwd", "fa_varlen_bwd"):
+        f = getattr(lib, name)
+        f.argtypes = [ctypes.POINTER(FaBwdParams), ctypes.c_void_p]
+        f.restype = ctypes.c_int
+    lib.fa_sizeof_bwd_params.argtypes = []
+    lib.fa_sizeof_bwd_params.restype = ctypes.c_int32
+    if lib.fa_sizeof_bwd_params() != ctypes.sizeof(FaBwdParams):
+        raise ImportError("flash_attn: fa_bwd_params layout mismatch between %s and its Python mirror; "
+                          "rebuild the library" % _LIB_PATH)
     lib.fa_rotary.argtypes = [ctypes.POINTER(FaRotaryParams), ctypes.c_void_p]
     lib.fa_rotary.restype = ctypes.c_int
     lib.fa_sizeof_rotary_params.argtypes = []
@@ -302,6 +324,130 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
             out_.copy_(out)
     rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
     return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, None, rng_state]
+
+
+def _set_strides(p, name, t):
+    """(batch, row, head) element strides of a (b, s, h, d) tensor, or (0, row, head) of a packed (total, h, d) one."""
+    st = t.stride()
+    b, r, h = (st[0], st[1], st[2]) if t.dim() == 4 else (0, st[0], st[1])
+    setattr(p, name + "_batch_stride", b)
+    setattr(p, name + "_row_stride", r)
+    setattr(p, name + "_head_stride", h)
+
+
+def _bwd_common(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, what):
+    if p_dropout != 0.0:
+        raise NotImplementedError("dropout is not implemented in the MI355X backward path")
+    q_dtype = q.dtype
+    dt = _dtype_code(q_dtype)
+    _check(k.dtype == q_dtype, "query and key must have the same dtype")
+    _check(v.dtype == q_dtype, "query and value must have the same dtype")
+    _check(out.dtype == q_dtype, "query and out must have the same dtype")
+    _check(dout.dtype == q_dtype, "query and dout must have the same dtype")
+    _check_device(q, k, v, out, dout, softmax_lse)
+    for t in (q, k, v):
+        _check(t.stride(-1) == 1, "Input tensor must have contiguous last dimension")
+    _check(out.stride(-1) == 1, "out tensor must have contiguous last dimension")
+    _check(dout.stride(-1) == 1, "dout tensor must have contiguous last dimension")
+    head_size_og, head_size = dout.shape[-1], q.shape[-1]
+    _check(head_size % 8 == 0, "head_size should be a multiple of 8")
+    _check(head_size <= 256, "FlashAttention backward only supports head dimension at most 256")
+    _check(q.shape[-2] % k.shape[-2] == 0, "Number of heads in key/value must divide number of heads in query")
+    _check(head_size == _round_up(head_size_og, 8), "head_size must be head_size_og rounded to a multiple of 8")
+    _check(tuple(k.shape[:-2]) == tuple(v.shape[:-2]) and k.shape[-2:] == v.shape[-2:] and k.shape[-1] == head_size,
+           "k and v must have the same shape and q's head size")
+    _check(tuple(out.shape) == tuple(q.shape), "out must have the shape of q")
+    _check(tuple(dout.shape) == tuple(q.shape[:-1]) + (head_size_og,), "dout must have the shape of out")
+    grads = []
+    for g_, like, name in ((dq_, q, "dq"), (dk_, k, "dk"), (dv_, v, "dv")):
+        if g_ is None:
+            g_ = torch.empty_like(like)
+        else:
+            _check(g_.dtype == q_dtype, name + " must have the same dtype as q")
+            _check_device(g_)
+            _check(g_.stride(-1) == 1, name + " must have contiguous last dimension")
+            _check(tuple(g_.shape) == tuple(like.shape), name + " has the wrong shape")
+        grads.append(g_)
+    dout_padded = _pad8(dout)
+    return dt, dout_padded, grads
+
+
+def _slice_grads(dq, dk, dv, head_size_og):
+    """Gradients at the caller's head size when it was padded to a multiple of 8 (flash_api.cpp:803-807)."""
+    if head_size_og % 8 != 0:
+        return [dq[..., :head_size_og], dk[..., :head_size_og], dv[..., :head_size_og]]
+    return [dq, dk, dv]
+
+
+def _fill_bwd(p, dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal, wl, wr, dt):
+    p.dout, p.q, p.k, p.v, p.out = dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.softmax_lse, p.softmax_d = softmax_lse.data_ptr(), softmax_d.data_ptr()
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", out), ("do", dout), ("dq", dq), ("dk", dk), ("dv", dv)):
+        _set_strides(p, name, t)
+    p.h, p.h_k, p.d = q.shape[-2], k.shape[-2], q.shape[-1]
+    p.softmax_scale = softmax_scale
+    p.is_causal, p.window_left, p.window_right = int(is_causal), wl, (0 if is_causal else wr)
+    p.dtype = dt
+
+
+def bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, softmax_scale, is_causal,
+        window_size_left, window_size_right, gen_, rng_state):
+    """Dense batch backward; mirrors mha_bwd (flash_api.cpp:609-832).  Returns [dq, dk, dv, softmax_d]."""
+    _check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be 4-dimensional")
+    dt, dout_padded, (dq, dk, dv) = _bwd_common(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, "bwd")
+    batch_size, seqlen_q, num_heads, _ = q.shape
+    seqlen_k = k.shape[1]
+    _check(batch_size > 0, "batch size must be positive")
+    _check(k.shape[0] == batch_size, "k must have q's batch size")
+    _check(tuple(softmax_lse.shape) == (batch_size, num_heads, seqlen_q) and softmax_lse.dtype == torch.float32
+           and softmax_lse.is_contiguous(), "softmax_lse must be a contiguous fp32 (batch, nheads, seqlen_q) tensor")
+    seqlen_q_rounded = _round_up(seqlen_q, 128)
+    with torch.cuda.device(q.device):
+        softmax_d = torch.empty((batch_size, num_heads, seqlen_q_rounded), dtype=torch.float32, device=q.device)
+        p = FaBwdParams()
+        _fill_bwd(p, dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal,
+                  window_size_left, window_size_right, dt)
+        p.b, p.seqlen_q, p.seqlen_k, p.seqlen_q_rounded = batch_size, seqlen_q, seqlen_k, seqlen_q_rounded
+        if seqlen_q > 0 and seqlen_k > 0:
+            _call(lib.fa_bwd, p, _stream(q.device))
+        else:       # nothing to attend to: all gradients are zero
+            dq.zero_(); dk.zero_(); dv.zero_(); softmax_d.zero_()
+    return _slice_grads(dq, dk, dv, dout.shape[-1]) + [softmax_d]
+
+
+def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
+               max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, window_size_left,
+               window_size_right, gen_, rng_state):
+    """Packed variable-length backward; mirrors mha_varlen_bwd (flash_api.cpp:834-1036)."""
+    _check(q.dim() == 3 and k.dim() == 3 and v.dim() == 3, "q, k, v must be 3-dimensional")
+    dt, dout_padded, (dq, dk, dv) = _bwd_common(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, "varlen_bwd")
+    _check(cu_seqlens_q.dtype == torch.int32, "cu_seqlens_q must have dtype int32")
+    _check(cu_seqlens_k.dtype == torch.int32, "cu_seqlens_k must have dtype int32")
+    _check_device(cu_seqlens_q, cu_seqlens_k)
+    _check(cu_seqlens_q.is_contiguous(), "cu_seqlens_q must be contiguous")
+    _check(cu_seqlens_k.is_contiguous(), "cu_seqlens_k must be contiguous")
+    total_q, num_heads, _ = q.shape
+    batch_size = cu_seqlens_q.numel() - 1
+    _check(batch_size > 0, "batch size must be positive")
+    _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
+    _check(tuple(softmax_lse.shape) == (batch_size, num_heads, max_seqlen_q) and softmax_lse.dtype == torch.float32
+           and softmax_lse.is_contiguous(), "softmax_lse must be a contiguous fp32 (batch, nheads, max_seqlen_q) tensor")
+    seqlen_q_rounded = _round_up(max_seqlen_q, 128)
+    with torch.cuda.device(q.device):
+        softmax_d = torch.empty((batch_size, num_heads, seqlen_q_rounded), dtype=torch.float32, device=q.device)
+        if zero_tensors:
+            dq.zero_(); dk.zero_(); dv.zero_(); softmax_d.zero_()
+        p = FaBwdParams()
+        _fill_bwd(p, dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal,
+                  window_size_left, window_size_right, dt)
+        p.cu_seqlens_q, p.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
+        p.b, p.seqlen_q, p.seqlen_k, p.seqlen_q_rounded = batch_size, max_seqlen_q, max_seqlen_k, seqlen_q_rounded
+        if max_seqlen_q > 0 and max_seqlen_k > 0 and total_q > 0 and k.shape[0] > 0:
+            _call(lib.fa_varlen_bwd, p, _stream(q.device))
+        else:
+            dq.zero_(); dk.zero_(); dv.zero_(); softmax_d.zero_()
+    return _slice_grads(dq, dk, dv, dout.shape[-1]) + [softmax_d]
 
 
 def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_,

@@ -171,6 +171,55 @@ int fa_rotary(const fa_rotary_params *p, void *hip_stream);
 /* sizeof(fa_rotary_params) as compiled, for foreign-language bindings (no reference counterpart). */
 int32_t fa_sizeof_rotary_params(void);
 
+/*
+ * Backward pass: gradients of q, k, v given the gradient of the output.  Replaces the reference's
+ * mha_bwd and mha_varlen_bwd (csrc/flash_attn/flash_api.cpp:609-832, 834-1036); the struct is the
+ * POD counterpart of Flash_bwd_params (csrc/flash_attn/src/flash.h:134-175).
+ *
+ * Layouts as in fa_fwd_params: q, out, dout, dq are (b, seqlen_q, h, d) or packed (total_q, h, d)
+ * with cu_seqlens_q; k, v, dk, dv are (b, seqlen_k, h_k, d) or packed (total_k, h_k, d) with
+ * cu_seqlens_k.  softmax_lse is the forward's (b, h, seqlen_q) fp32 result (seqlen_q = max_seqlen_q
+ * for packed input).  softmax_d is caller-provided work space AND a result, as in the reference:
+ * (b, h, seqlen_q_rounded) fp32, seqlen_q_rounded >= seqlen_q, receiving rowsum(dout * out).
+ * dk and dv are written at h_k heads: the sum over the query heads of a group happens inside the
+ * kernel, no expanded buffer is needed.  Dropout is not supported.  Results are deterministic (no
+ * atomics): dq is produced by one pass over query tiles, dk / dv by one pass over key tiles.
+ */
+typedef struct fa_bwd_params {
+    const void *dout, *q, *k, *v, *out;
+    const float *softmax_lse;
+    void *dq, *dk, *dv;
+    float *softmax_d;
+    const int32_t *cu_seqlens_q;    /* (b+1) prefix sums, or NULL for a dense batch */
+    const int32_t *cu_seqlens_k;    /* (b+1) prefix sums, or NULL for a dense batch */
+
+    int64_t q_batch_stride, q_row_stride, q_head_stride;
+    int64_t k_batch_stride, k_row_stride, k_head_stride;
+    int64_t v_batch_stride, v_row_stride, v_head_stride;
+    int64_t o_batch_stride, o_row_stride, o_head_stride;
+    int64_t do_batch_stride, do_row_stride, do_head_stride;
+    int64_t dq_batch_stride, dq_row_stride, dq_head_stride;
+    int64_t dk_batch_stride, dk_row_stride, dk_head_stride;
+    int64_t dv_batch_stride, dv_row_stride, dv_head_stride;
+
+    int32_t b, seqlen_q, seqlen_k;  /* seqlen_* are the maxima for packed input */
+    int32_t h, h_k, d;              /* d a multiple of 8, <= 256 */
+    int32_t seqlen_q_rounded;       /* row pitch of softmax_d */
+    float softmax_scale;
+    int32_t is_causal;
+    int32_t window_left, window_right;
+    int32_t dtype;                  /* FA_DTYPE_* */
+} fa_bwd_params;
+
+/* mha_bwd (flash_api.cpp:609-832): dense batch; cu_seqlens_* must be NULL. */
+int fa_bwd(const fa_bwd_params *p, void *hip_stream);
+
+/* mha_varlen_bwd (flash_api.cpp:834-1036): packed sequences; both cu_seqlens_* required. */
+int fa_varlen_bwd(const fa_bwd_params *p, void *hip_stream);
+
+/* sizeof(fa_bwd_params) as compiled into the library. */
+int32_t fa_sizeof_bwd_params(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,4 @@
-"""CPU oracle for the FlashAttention-2 forward path.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the FlashAttention-2 forward and backward path.  TEST INFRASTRUCTURE ONLY.
 
 This module is the checker, never the product: only the test-suite, the smoke entry and the
 benchmark's CPU-baseline leg may import it.  Nothing in the shipped package routes through it.
@@ -16,7 +16,11 @@ It restates, in plain PyTorch on the CPU, the semantics that the reference pins 
   (`flash_attn/flash_attn_interface.py:922-1042`, `tests/test_flash_attn.py:1759-1834`);
 * packed variable-length attention as "each sequence attends alone"
   (`tests/test_flash_attn.py:229-258`);
-* the reference's split-count heuristic (`csrc/flash_attn/flash_api.cpp:212-246`).
+* the reference's split-count heuristic (`csrc/flash_attn/flash_api.cpp:212-246`);
+* the gradients of q, k, v by the formulas the backward kernel evaluates
+  (`csrc/flash_attn/src/flash_bwd_kernel.h:79-780`: dV = P^T dO, dP = dO V^T, dS = P o (dP - D) with
+  D = rowsum(dO o O), dQ = scale dS K, dK = scale dS^T Q), pinned against torch autograd through
+  the forward restatement and against central finite differences in fp64.
 
 How each function is pinned (none is "parity unpinned"): see tests/test_oracle.py -- library
 routine `scaled_dot_product_attention`, brute-force scalar loops on tiny shapes, the docstring
@@ -129,6 +133,53 @@ def attention_forward(q, k, v, causal=False, window_size=(-1, -1), softmax_scale
             out[ib, :, h0:h1] = o.to(dtype_og)
             lse[ib, h0:h1] = lse_blk
     return out, lse
+
+
+def attention_backward(q, k, v, dout, causal=False, window_size=(-1, -1), softmax_scale=None,
+                       seqlens_q=None, seqlens_k=None, dtype=torch.float32):
+    """(dq, dk, dv) in `dtype` (fp32, or fp64 for the finite-difference check), unrounded.
+
+    The backward kernel's own formulas (`csrc/flash_attn/src/flash_bwd_kernel.h:79-780`), evaluated per
+    (batch, head) on the full score matrix: P = softmax(scale Q K^T) over the visible keys (0 for a row
+    that sees none), dV = P^T dO, dP = dO V^T, D_i = sum_d dO[i,d] O[i,d], dS = P o (dP - D),
+    dQ = scale dS K, dK = scale dS^T Q; with GQA / MQA the dK, dV of a key head are summed over the
+    query heads that read it (`csrc/flash_attn/flash_api.cpp:799-803`).  Padded query rows
+    (seqlens_q) contribute nothing and get dQ = 0; padded keys get dK = dV = 0."""
+    b, sq, h, d = q.shape
+    _, sk, hk, _ = k.shape
+    g = h // hk
+    scale = (1.0 / math.sqrt(d)) if softmax_scale is None else float(softmax_scale)
+    qf, kf, vf, gf = q.to(dtype), k.to(dtype), v.to(dtype), dout.to(dtype)
+    dq, dk, dv = torch.zeros_like(qf), torch.zeros_like(kf), torch.zeros_like(vf)
+    vis_all = visible_mask(sq, sk, window_size, causal, seqlens_q, seqlens_k)
+    for ib in range(b):
+        vis = vis_all[ib] if vis_all.dim() == 3 else vis_all
+        if seqlens_q is not None:
+            vis = vis & (torch.arange(sq) < int(seqlens_q[ib])).view(-1, 1)
+        dead = ~vis.any(dim=-1, keepdim=True)
+        for ih in range(h):
+            jk = ih // g
+            s = (qf[ib, :, ih] @ kf[ib, :, jk].T) * scale
+            s = s.masked_fill(~vis, float("-inf"))
+            p = torch.softmax(s, dim=-1).masked_fill(dead, 0.0)
+            o = p @ vf[ib, :, jk]
+            do = gf[ib, :, ih]
+            dv[ib, :, jk] += p.T @ do
+            dp = do @ vf[ib, :, jk].T
+            dsum = (do * o).sum(dim=-1, keepdim=True)
+            ds = p * (dp - dsum)
+            dq[ib, :, ih] = scale * (ds @ kf[ib, :, jk])
+            dk[ib, :, jk] += scale * (ds.T @ qf[ib, :, ih])
+    return dq, dk, dv
+
+
+def attention_backward_autograd(q, k, v, dout, upcast=True, reorder_ops=False, **kw):
+    """(dq, dk, dv) by torch autograd through `attention_forward`.  With upcast=False,
+    reorder_ops=True this is the ordinary low-precision implementation whose error supplies the
+    right-hand side of the gradient tolerance rule (`tests/test_flash_attn.py:1006-1008`)."""
+    q, k, v = [t.detach().clone().requires_grad_() for t in (q, k, v)]
+    out, _ = attention_forward(q, k, v, upcast=upcast, reorder_ops=reorder_ops, **kw)
+    return torch.autograd.grad(out, (q, k, v), dout.to(out.dtype))
 
 
 def attention_reference_pair(q, k, v, **kw):

@@ -29,7 +29,8 @@ def declared_symbols():
 def test_header_symbols_exported(lib):
     names = declared_symbols()
     assert {"fa_fwd", "fa_varlen_fwd", "fa_fwd_kvcache", "fa_plan_splits", "fa_last_error",
-            "fa_num_splits_heuristic_reference", "fa_version", "fa_sizeof_params"} <= set(names)
+            "fa_num_splits_heuristic_reference", "fa_version", "fa_sizeof_params", "fa_bwd", "fa_varlen_bwd",
+            "fa_sizeof_bwd_params", "fa_rotary", "fa_sizeof_rotary_params"} <= set(names)
     for n in names:
         assert hasattr(lib, n), "library does not export %s" % n
 
@@ -38,6 +39,31 @@ def test_struct_mirror_size(lib):
     import flash_attn._native as nat
     lib.fa_sizeof_params.restype = ctypes.c_int32
     assert lib.fa_sizeof_params() == ctypes.sizeof(nat.FaFwdParams)
+    lib.fa_sizeof_bwd_params.restype = ctypes.c_int32
+    assert lib.fa_sizeof_bwd_params() == ctypes.sizeof(nat.FaBwdParams)
+    lib.fa_sizeof_rotary_params.restype = ctypes.c_int32
+    assert lib.fa_sizeof_rotary_params() == ctypes.sizeof(nat.FaRotaryParams)
+
+
+def test_backward_argument_errors_do_not_abort(lib):
+    import flash_attn._native as nat
+    p = nat.FaBwdParams()
+    lib.fa_bwd.argtypes = [ctypes.POINTER(nat.FaBwdParams), ctypes.c_void_p]
+    lib.fa_bwd.restype = ctypes.c_int
+    lib.fa_varlen_bwd.argtypes = [ctypes.POINTER(nat.FaBwdParams), ctypes.c_void_p]
+    lib.fa_varlen_bwd.restype = ctypes.c_int
+    lib.fa_last_error.restype = ctypes.c_char_p
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"must be set" in lib.fa_last_error()
+    for n in ("dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "softmax_d"):
+        setattr(p, n, 16)                       # never dereferenced: the checks below fail first
+    p.b, p.h, p.h_k, p.d, p.seqlen_q, p.seqlen_k, p.seqlen_q_rounded, p.dtype = 1, 4, 3, 64, 8, 8, 128, 1
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"Number of heads" in lib.fa_last_error()
+    p.h_k, p.d = 2, 260
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"at most 256" in lib.fa_last_error()
+    p.d = 64
+    assert lib.fa_varlen_bwd(ctypes.byref(p), None) != 0 and b"cu_seqlens" in lib.fa_last_error()
+    p.q_row_stride = 4
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"strides" in lib.fa_last_error()
 
 
 def test_reference_heuristic_matches_oracle(lib):

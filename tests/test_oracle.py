@@ -258,3 +258,86 @@ def test_tolerance_rule_detects_errors():
     ok, _, _ = orc.tolerance_ok(ref + 0.05, ref, pt)
     assert not ok
     assert orc.lse_ok(lse * (1 + 5e-4), lse)[0] and not orc.lse_ok(lse * 1.01, lse)[0]
+
+
+# ---------------------------------------------------------------------------------------------
+# backward restatement
+# ---------------------------------------------------------------------------------------------
+def _loss(q, k, v, w, **kw):
+    """sum(out * w) with out from a scalar-loop softmax attention in fp64: the function whose gradient
+    the backward restatement claims to be."""
+    b, sq, h, d = q.shape
+    sk, hk = k.shape[1], k.shape[2]
+    g = h // hk
+    scale = kw.get("softmax_scale") or d ** -0.5
+    vis = orc.visible_mask(sq, sk, kw.get("window_size", (-1, -1)), kw.get("causal", False))
+    total = 0.0
+    for ib in range(b):
+        for ih in range(h):
+            s = (q[ib, :, ih] @ k[ib, :, ih // g].T) * scale
+            for i in range(sq):
+                cols = [j for j in range(sk) if vis[i, j]]
+                if not cols:
+                    continue
+                e = torch.exp(s[i, cols] - s[i, cols].max())
+                p = e / e.sum()
+                total = total + ((p[:, None] * v[ib, cols, ih // g]).sum(0) * w[ib, i, ih]).sum()
+    return total
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(causal=True), dict(window_size=(2, 1)), dict(window_size=(-1, 0), softmax_scale=0.3)])
+def test_backward_against_central_differences(kw):
+    """Every entry of dq, dk, dv against (L(x + e) - L(x - e)) / 2e of a scalar-loop forward in fp64;
+    seqlen_q > seqlen_k under causal gives rows that see nothing (gradient exactly zero)."""
+    g = torch.Generator().manual_seed(3)
+    b, sq, sk, h, hk, d = 1, 5, 4, 2, 1, 3
+    q = torch.randn(b, sq, h, d, generator=g, dtype=torch.float64)
+    k = torch.randn(b, sk, hk, d, generator=g, dtype=torch.float64)
+    v = torch.randn(b, sk, hk, d, generator=g, dtype=torch.float64)
+    w = torch.randn(b, sq, h, d, generator=g, dtype=torch.float64)
+    grads = orc.attention_backward(q, k, v, w, dtype=torch.float64, **kw)
+    eps = 1e-6
+    for x, gx in zip((q, k, v), grads):
+        flat = x.view(-1)
+        for idx in range(flat.numel()):
+            old = flat[idx].item()
+            flat[idx] = old + eps
+            up = _loss(q, k, v, w, **kw)
+            flat[idx] = old - eps
+            dn = _loss(q, k, v, w, **kw)
+            flat[idx] = old
+            assert abs((up - dn).item() / (2 * eps) - gx.view(-1)[idx].item()) < 1e-7
+
+
+@pytest.mark.parametrize("kw", [dict(causal=True), dict(window_size=(5, 3)), dict(),
+                                dict(causal=True, seqlens_q=torch.tensor([7, 13]), seqlens_k=torch.tensor([17, 6]))])
+def test_backward_against_autograd(kw):
+    """Library check: torch autograd through the forward restatement (fp64, GQA, padded lengths)."""
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(2, 13, 6, 16, generator=g, dtype=torch.float64)
+    k = torch.randn(2, 17, 2, 16, generator=g, dtype=torch.float64)
+    v = torch.randn(2, 17, 2, 16, generator=g, dtype=torch.float64)
+    do = torch.randn(2, 13, 6, 16, generator=g, dtype=torch.float64)
+    a = orc.attention_backward(q, k, v, do, dtype=torch.float64, **kw)
+    c = orc.attention_backward_autograd(q, k, v, do, upcast=False, **kw)
+    for x, y in zip(a, c):
+        assert (x - y).abs().max() < 1e-12
+
+
+def test_backward_closed_forms():
+    """One key: P = 1, so dV = sum of dO over rows and heads of the group, dQ = dK = 0.
+    Zero queries: uniform attention, dV[j] = mean-weighted sum of dO and dK = 0 exactly when dO V^T is
+    constant along keys (V rows equal)."""
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(2, 6, 4, 8, generator=g); do = torch.randn(2, 6, 4, 8, generator=g)
+    k = torch.randn(2, 1, 2, 8, generator=g); v = torch.randn(2, 1, 2, 8, generator=g)
+    dq, dk, dv = orc.attention_backward(q, k, v, do)
+    assert dq.abs().max() < 1e-6 and dk.abs().max() < 1e-6
+    want = do.view(2, 6, 2, 2, 8).sum(dim=(1, 3))
+    assert torch.allclose(dv[:, 0], want, atol=1e-5)
+    sk = 5
+    k = torch.randn(2, sk, 2, 8, generator=g)
+    v = torch.randn(2, 1, 2, 8, generator=g).expand(2, sk, 2, 8).contiguous()
+    dq, dk, dv = orc.attention_backward(torch.zeros_like(q), k, v, do)
+    assert dk.abs().max() < 1e-6
+    assert torch.allclose(dv, (want / sk)[:, None].expand_as(dv), atol=1e-5)
