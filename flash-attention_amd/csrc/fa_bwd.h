@@ -58,6 +58,12 @@ FA_DEV BwdSeq bwd_seq(const fa_bwd_params& p, int b) {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// accumulate step dk of a product; step 0 starts from an inline zero instead of a cleared accumulator
+template <typename T> FA_DEV void mfma_step(f32x16& acc, typename Elem<T>::v8 a, typename Elem<T>::v8 b, int dk) {
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    acc = Elem<T>::mfma32(a, b, dk == 0 ? zero : acc);
+}
+
 // A operand, row-wise: rows [row0, row0+32) of a swizzled tile, columns [16 dk, 16 dk + 16)
 template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_a_rows(const char* tile, int row, int dk, int hh) {
     const int c = dk * 2 + hh;
@@ -130,7 +136,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_bwd_params& p = kp.p;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
 
     // logical order: heads of one group adjacent, then query tiles, then kv heads, then batch; runs of
     // the order go to one XCD so that workgroups streaming the same K / V share an L2
@@ -234,13 +240,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 #pragma unroll
             for (int nb = 0; nb < C::NB; nb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) { s_acc[nb][r] = 0.f; dp_acc[nb][r] = 0.f; }
-#pragma unroll
-            for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
                 for (int dk = 0; dk < C::KS; dk++) {
-                    s_acc[nb] = Elem<T>::mfma32(lds_a_rows<T, D>(kb, nb * 32 + l32, dk, hh), qf[dk], s_acc[nb]);
-                    dp_acc[nb] = Elem<T>::mfma32(lds_a_rows<T, D>(vb, nb * 32 + l32, dk, hh), gf[dk], dp_acc[nb]);
+                    mfma_step<T>(s_acc[nb], lds_a_rows<T, D>(kb, nb * 32 + l32, dk, hh), qf[dk], dk);
+                    mfma_step<T>(dp_acc[nb], lds_a_rows<T, D>(vb, nb * 32 + l32, dk, hh), gf[dk], dk);
                 }
             const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0w + shift + wr) ||
                                    (has_left && n0 < r0w + 31 + shift - wl);
@@ -318,7 +320,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_bwd_params& p = kp.p;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
 
     const int G = p.h / p.h_k;
     const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
@@ -373,9 +375,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
     u32x4 qr[C::LOADS], gr[C::LOADS];
     float aux = 0.f;
     const int d_last_chunk = p.d / 8 - 1;
-    auto load_tile = [&](int it) {
-        const int head = hk * G + it / nt;
-        const int i0 = (t_lo + it % nt) * BM;
+    auto load_tile = [&](int g, int t) {
+        const int head = hk * G + g;
+        const int i0 = t * BM;
         const T* qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
         const T* gg = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride;
 #pragma unroll
@@ -395,10 +397,10 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
                 aux = tid < BM ? INFINITY : 0.f;
         }
     };
-    auto store_tile = [&](int buf, int it) {
+    auto store_tile = [&](int buf, int t) {
         char* qb = smem + buf * C::STAGE;
         char* gb = qb + C::TILE_BYTES;
-        const int i0 = (t_lo + it % nt) * BM;
+        const int i0 = t * BM;
 #pragma unroll
         for (int i = 0; i < C::LOADS; i++) {
             const int f = tid + i * C::kThreads;
@@ -413,13 +415,19 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
     };
 
     const float sl2 = kp.scale_log2;
-    if (iters > 0) { load_tile(0); store_tile(0, 0); }
+    const int rel_hi = has_right ? shift + wr : 0x3fffffff;
+    const int rel_lo = has_left ? shift - wl : -0x3fffffff;
+    if (iters > 0) { load_tile(0, t_lo); store_tile(0, t_lo); }
     __syncthreads();
     int buf = 0;
+    int cur_t = t_lo, nxt_g = 0, nxt_t = t_lo;       // (head of group, query tile) walked without divisions
     for (int it = 0; it < iters; ++it) {
         const bool has_next = it + 1 < iters;
-        if (has_next) load_tile(it + 1);
-        const int i0 = (t_lo + it % nt) * BM;
+        if (has_next) {
+            if (++nxt_t == t_hi) { nxt_t = t_lo; ++nxt_g; }
+            load_tile(nxt_g, nxt_t);
+        }
+        const int i0 = cur_t * BM;
         const char* qb = smem + buf * C::STAGE;
         const char* gb = qb + C::TILE_BYTES;
         const float* lse_s = reinterpret_cast<const float*>(gb + C::TILE_BYTES);
@@ -433,13 +441,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
 #pragma unroll
             for (int mb = 0; mb < C::MBK; mb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) { s_acc[mb][r] = 0.f; dp_acc[mb][r] = 0.f; }
-#pragma unroll
-            for (int mb = 0; mb < C::MBK; mb++)
-#pragma unroll
                 for (int dk = 0; dk < C::KS; dk++) {
-                    s_acc[mb] = Elem<T>::mfma32(lds_a_rows<T, D>(qb, mb * 32 + l32, dk, hh), kf[dk], s_acc[mb]);
-                    dp_acc[mb] = Elem<T>::mfma32(lds_a_rows<T, D>(gb, mb * 32 + l32, dk, hh), vf[dk], dp_acc[mb]);
+                    mfma_step<T>(s_acc[mb], lds_a_rows<T, D>(qb, mb * 32 + l32, dk, hh), kf[dk], dk);
+                    mfma_step<T>(dp_acc[mb], lds_a_rows<T, D>(gb, mb * 32 + l32, dk, hh), vf[dk], dk);
                 }
             v8 pf[C::PT], dsf[C::PT];
 #pragma unroll
@@ -447,11 +451,12 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
                 const int ib = i0 + mb * 32;
                 const bool need_mask = (has_right && j0w + 31 > ib + shift + wr) || (has_left && j0w < ib + 31 + shift - wl);
                 if (need_mask) {
+                    // key - row must lie in [rel_lo, rel_hi]; the row of register r is ib + 4 hh + c_r
+                    const int rel = key - ib - 4 * hh;
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const int i = ib + 8 * (r >> 2) + 4 * hh + (r & 3);
-                        const bool hidden = (has_right && key > i + shift + wr) || (has_left && key < i + shift - wl);
-                        if (hidden) s_acc[mb][r] = -INFINITY;
+                        const int c_r = 8 * (r >> 2) + (r & 3);
+                        s_acc[mb][r] = (rel > rel_hi + c_r || rel < rel_lo + c_r) ? -INFINITY : s_acc[mb][r];
                     }
                 }
 #pragma unroll
@@ -480,9 +485,10 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
                     dk_acc[db] = Elem<T>::mfma32(lds_a_cols<T, D>(qb, t16, dpart * C::DB + db, lane), dsf[t16], dk_acc[db]);
                 }
         }
-        if (has_next) store_tile(buf ^ 1, it + 1);
+        if (has_next) store_tile(buf ^ 1, nxt_t);
         __syncthreads();
         buf ^= 1;
+        cur_t = nxt_t;
     }
 
     if (!key_ok) return;
@@ -501,6 +507,225 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
                            pack2<T>(dv_acc[db][4 * q4 + 2], dv_acc[db][4 * q4 + 3])};
                 st_global8(dkrow + d0, a);
                 st_global8(dvrow + d0, c);
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK, dV with the two gradients on different waves (head dim <= 128).  8 waves: wave w < 4 computes dV
+// of key block w (S, P, dV^T += dO^T P), wave w + 4 computes dK of the same keys (S, dP, dS,
+// dK^T += Q^T dS).  Each wave then fits 256 registers, so a SIMD holds one wave of each kind and
+// the exp / pack work of one overlaps the matrix products of the other; the price is that S is
+// computed by both (5 tile products instead of 4).  The streamed Q / dO tiles are shared.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int D, int BM>
+struct BwdDkv2Cfg {
+    static constexpr int kThreads = 512, kWaves = 8, BNW = 128;
+    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int TILE_BYTES = BM * ROWB;
+    static constexpr int LOADS = BM * CPR / kThreads;
+    static constexpr int STAGE = 2 * TILE_BYTES + 2 * BM * 4;   // Q, dO, lse (log2 units), D
+    static constexpr int SMEM = 2 * STAGE;
+    static_assert(BM % 32 == 0 && D % 32 == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
+};
+
+template <typename T, int D, int BM>
+__global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
+    typedef BwdDkv2Cfg<T, D, BM> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_bwd_params& p = kp.p;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const bool role_k = wave >= 4;          // wave-uniform
+    const int kblk = wave & 3;
+
+    const int G = p.h / p.h_k;
+    const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
+    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int nblk = (int)(w % num_n_blocks); w /= num_n_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+
+    const BwdSeq si = bwd_seq(p, b);
+    const int n0 = nblk * C::BNW;
+    if (n0 >= si.sk) return;
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    int i_lo = 0, i_hi = si.sq;
+    if (has_right) i_lo = max(0, n0 - shift - wr);
+    if (has_left) i_hi = min(si.sq, min(n0 + C::BNW, si.sk) - shift + wl);
+    const int t_lo = i_lo / BM;
+    const int t_hi = i_hi > i_lo ? (i_hi + BM - 1) / BM : t_lo;
+    const int nt = t_hi - t_lo;
+    const int iters = nt * G;
+
+    const int j0w = n0 + kblk * 32;
+    const int key = j0w + l32;
+    const bool key_ok = key < si.sk;
+    v8 kf[C::KS], vf[C::KS];
+    {
+        const T* krow = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)key * p.k_row_stride + (int64_t)hk * p.k_head_stride;
+        const T* vrow = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)key * p.v_row_stride + (int64_t)hk * p.v_head_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 a = {0, 0, 0, 0}, c = {0, 0, 0, 0};
+            if (key_ok && d0 < p.d) {
+                a = ld_global16(krow + d0);
+                if (role_k) c = ld_global16(vrow + d0);
+            }
+            kf[dk] = __builtin_bit_cast(v8, a);
+            vf[dk] = __builtin_bit_cast(v8, c);
+        }
+    }
+
+    f32x16 acc[C::DB];      // dV^T of this wave's keys (role V) or dK^T (role K)
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+
+    u32x4 qr[C::LOADS], gr[C::LOADS];
+    float aux = 0.f;
+    const int d_last_chunk = p.d / 8 - 1;
+    auto load_tile = [&](int g, int t) {
+        const int head = hk * G + g;
+        const int i0 = t * BM;
+        const T* qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
+        const T* gg = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
+            const int n = min(i0 + r, si.sq - 1);
+            qr[i] = ld_global16(qg + (int64_t)n * p.q_row_stride + c * 8);
+            gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
+        }
+        if (tid < 2 * BM) {
+            const int r = i0 + (tid < BM ? tid : tid - BM);
+            if (r < si.sq)
+                aux = tid < BM ? p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + r] * kLog2e
+                               : p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + r];
+            else
+                aux = tid < BM ? INFINITY : 0.f;
+        }
+    };
+    auto store_tile = [&](int buf, int t) {
+        char* qb = smem + buf * C::STAGE;
+        char* gb = qb + C::TILE_BYTES;
+        const int i0 = t * BM;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = f % C::CPR;
+            const bool ok = (i0 + r < si.sq) && (c <= d_last_chunk);
+            const u32x4 z = {0, 0, 0, 0};
+            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
+            *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
+            *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
+        }
+        if (tid < 2 * BM) reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = aux;
+    };
+
+    const float sl2 = kp.scale_log2;
+    const int rel_hi = has_right ? shift + wr : 0x3fffffff;
+    const int rel_lo = has_left ? shift - wl : -0x3fffffff;
+    if (iters > 0) { load_tile(0, t_lo); store_tile(0, t_lo); }
+    __syncthreads();
+    int buf = 0;
+    int cur_t = t_lo, nxt_g = 0, nxt_t = t_lo;       // (head of group, query tile) walked without divisions
+    for (int it = 0; it < iters; ++it) {
+        const bool has_next = it + 1 < iters;
+        if (has_next) {
+            if (++nxt_t == t_hi) { nxt_t = t_lo; ++nxt_g; }
+            load_tile(nxt_g, nxt_t);
+        }
+        const int i0 = cur_t * BM;
+        const char* qb = smem + buf * C::STAGE;
+        const char* gb = qb + C::TILE_BYTES;
+        const float* lse_s = reinterpret_cast<const float*>(gb + C::TILE_BYTES);
+        const float* dsum_s = lse_s + BM;
+
+        const bool wave_skip = (has_right && j0w > i0 + BM - 1 + shift + wr) || (has_left && j0w + 31 < i0 + shift - wl) ||
+                               (j0w >= si.sk);
+        if (!wave_skip) {
+            f32x16 s_acc[C::MBK], dp_acc[C::MBK];
+#pragma unroll
+            for (int mb = 0; mb < C::MBK; mb++)
+#pragma unroll
+                for (int dk = 0; dk < C::KS; dk++)
+                    mfma_step<T>(s_acc[mb], lds_a_rows<T, D>(qb, mb * 32 + l32, dk, hh), kf[dk], dk);
+            if (role_k) {
+#pragma unroll
+                for (int mb = 0; mb < C::MBK; mb++)
+#pragma unroll
+                    for (int dk = 0; dk < C::KS; dk++)
+                        mfma_step<T>(dp_acc[mb], lds_a_rows<T, D>(gb, mb * 32 + l32, dk, hh), vf[dk], dk);
+            }
+            v8 bf[C::PT];       // P (role V) or dS (role K), packed as the B operand
+#pragma unroll
+            for (int mb = 0; mb < C::MBK; mb++) {
+                const int ib = i0 + mb * 32;
+                const bool need_mask = (has_right && j0w + 31 > ib + shift + wr) || (has_left && j0w < ib + 31 + shift - wl);
+                if (need_mask) {
+                    // key - row must lie in [rel_lo, rel_hi]; the row of register r is ib + 4 hh + c_r
+                    const int rel = key - ib - 4 * hh;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int c_r = 8 * (r >> 2) + (r & 3);
+                        s_acc[mb][r] = (rel > rel_hi + c_r || rel < rel_lo + c_r) ? -INFINITY : s_acc[mb][r];
+                    }
+                }
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        s_acc[mb][4 * q4 + e] = fast_exp2(s_acc[mb][4 * q4 + e] * sl2 - l4[e]);
+                }
+                if (role_k) {
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            s_acc[mb][4 * q4 + e] *= dp_acc[mb][4 * q4 + e] - d4[e];
+                    }
+                }
+                bf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
+                bf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
+            }
+            // role V: dV^T += dO^T P;  role K: dK^T += Q^T dS
+            const char* tb = role_k ? qb : gb;
+#pragma unroll
+            for (int t16 = 0; t16 < C::PT; t16++)
+#pragma unroll
+                for (int db = 0; db < C::DB; db++)
+                    acc[db] = Elem<T>::mfma32(lds_a_cols<T, D>(tb, t16, db, lane), bf[t16], acc[db]);
+        }
+        if (has_next) store_tile(buf ^ 1, nxt_t);
+        __syncthreads();
+        buf ^= 1;
+        cur_t = nxt_t;
+    }
+
+    if (!key_ok) return;
+    T* orow = role_k ? reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride
+                     : reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
+    const float sc = role_k ? p.softmax_scale : 1.f;
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const int d0 = db * 32 + 8 * q4 + 4 * hh;
+            if (d0 < p.d) {
+                u32x2 a = {pack2<T>(acc[db][4 * q4] * sc, acc[db][4 * q4 + 1] * sc),
+                           pack2<T>(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc)};
+                st_global8(orow + d0, a);
             }
         }
 }
@@ -533,6 +758,19 @@ int launch_bwd_dkv(const BwdKParams& kp, hipStream_t stream) {
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
     auto kern = bwd_dkv_kernel<T, D, BM, DPARTS, MINW>;
+    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int D, int BM>
+int launch_bwd_dkv2(const BwdKParams& kp, hipStream_t stream) {
+    typedef BwdDkv2Cfg<T, D, BM> C;
+    const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b;
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    auto kern = bwd_dkv2_kernel<T, D, BM>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();

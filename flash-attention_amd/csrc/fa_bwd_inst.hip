@@ -17,8 +17,9 @@ typedef _Float16 InstT;
 // already filled (launch_bwd_dot).
 int FA_INST_NAME(FA_D)(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
-    if (int e = launch_bwd_dq<InstT, FA_D, 64, 1>(kp, stream)) return e;
-    return launch_bwd_dkv<InstT, FA_D, 64, 1, 1>(kp, stream);
+    // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers
+    if (int e = launch_bwd_dq<InstT, FA_D, (FA_D > 64 ? 32 : 64), 2>(kp, stream)) return e;
+    return launch_bwd_dkv2<InstT, FA_D, 64>(kp, stream);
 #else
     if (int e = launch_bwd_dq<InstT, FA_D, 32, 1>(kp, stream)) return e;
     return launch_bwd_dkv<InstT, FA_D, 32, 2, 1>(kp, stream);
