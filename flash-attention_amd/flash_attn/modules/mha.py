@@ -1,0 +1,150 @@
+"""Self-attention layer with a KV cache: the caller of `flash_attn_with_kvcache` during generation.
+
+Covers the decoding glue of the reference's flash_attn/modules/mha.py: `_update_kv_cache` (:296-322),
+`MHA.allocate_inference_cache` (:422-434), `MHA._apply_rotary_update_kvcache_attention` (:442-479),
+`MHA._update_kvcache_attention` (:481-507) and the self-attention branches of `MHA.forward`
+(:515-653): packed QKV projection, rotary, MHA / GQA / MQA, causal mask.  Not carried over (the
+reference's options outside the attention path): cross-attention, depthwise convolution, dropout,
+ALiBi, fused dense layers, the non-flash attention fallbacks, activation checkpointing and the
+tensor-parallel variant.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from flash_attn import flash_attn_kvpacked_func, flash_attn_qkvpacked_func, flash_attn_with_kvcache
+from flash_attn.layers.rotary import RotaryEmbedding
+
+
+def _update_kv_cache(kv, inference_params, layer_idx):
+    """Write kv (batch, seqlen, 2, nheads_kv, head_dim) at [batch_size_offset, seqlen_offset) of the
+    layer's cache (allocated on first use) and return the filled part (batch, seqlen_offset + seqlen, ...)."""
+    num_heads, head_dim = kv.shape[-2:]
+    if layer_idx not in inference_params.key_value_memory_dict:
+        inference_params.key_value_memory_dict[layer_idx] = torch.empty(
+            inference_params.max_batch_size, inference_params.max_seqlen, 2, num_heads, head_dim,
+            dtype=kv.dtype, device=kv.device)
+    kv_cache = inference_params.key_value_memory_dict[layer_idx]
+    b0 = inference_params.batch_size_offset
+    b1 = b0 + kv.shape[0]
+    s0 = inference_params.seqlen_offset
+    s1 = s0 + kv.shape[1]
+    assert b1 <= kv_cache.shape[0]
+    assert s1 <= kv_cache.shape[1]
+    kv_cache[b0:b1, s0:s1, ...] = kv
+    return kv_cache[b0:b1, :s1, ...]
+
+
+class MHA(nn.Module):
+    """Multi-head self-attention on the flash attention kernels, with the reference's constructor
+    arguments for the options that are supported."""
+
+    def __init__(self, embed_dim, num_heads, num_heads_kv=None, qkv_proj_bias=True, out_proj_bias=True,
+                 softmax_scale=None, causal=False, layer_idx=None, rotary_emb_dim=0, rotary_emb_base=10000.0,
+                 rotary_emb_scale_base=None, rotary_emb_interleaved=False, window_size=(-1, -1), device=None,
+                 dtype=None):
+        factory_kwargs = {"device": device, "dtype": dtype}
+        super().__init__()
+        self.embed_dim = embed_dim
+        self.causal = causal
+        self.layer_idx = layer_idx
+        self.rotary_emb_dim = rotary_emb_dim
+        self.softmax_scale = softmax_scale
+        self.window_size = window_size
+        self.use_flash_attn = True
+        self.num_heads = num_heads
+        self.num_heads_kv = num_heads_kv if num_heads_kv is not None else num_heads
+        assert self.num_heads % self.num_heads_kv == 0, "num_heads must be divisible by num_heads_kv"
+        assert self.embed_dim % num_heads == 0, "embed_dim must be divisible by num_heads"
+        self.head_dim = self.embed_dim // num_heads
+        qkv_dim = self.head_dim * (self.num_heads + 2 * self.num_heads_kv)
+        if self.rotary_emb_dim > 0:
+            self.rotary_emb = RotaryEmbedding(self.rotary_emb_dim, base=rotary_emb_base, scale_base=rotary_emb_scale_base,
+                                              interleaved=rotary_emb_interleaved, device=device)
+        self.Wqkv = nn.Linear(embed_dim, qkv_dim, bias=qkv_proj_bias, **factory_kwargs)
+        self.out_proj = nn.Linear(embed_dim, embed_dim, bias=out_proj_bias, **factory_kwargs)
+
+    def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None):
+        dtype = self.out_proj.weight.dtype if dtype is None else dtype
+        return torch.empty(batch_size, max_seqlen, 2, self.num_heads_kv, self.head_dim, dtype=dtype,
+                           device=self.out_proj.weight.device)
+
+    def _update_kv_cache(self, kv, inference_params):
+        assert self.layer_idx is not None, "Generation requires layer_idx in the constructor"
+        return _update_kv_cache(kv, inference_params, self.layer_idx)
+
+    def _cache_and_lengths(self, batch, inference_params):
+        kv_cache = inference_params.key_value_memory_dict[self.layer_idx][:batch]
+        lengths = inference_params.lengths_per_sample
+        return kv_cache, (lengths[:batch] if lengths is not None else inference_params.seqlen_offset)
+
+    def _apply_rotary_update_kvcache_attention(self, q, kv, inference_params):
+        """One kernel sequence for: rotate q and the new k at each sequence's current length, append
+        the new k / v to the cache, attend to the cache.  q (batch, seqlen_q, nheads, head_dim),
+        kv (batch, seqlen_new, 2, nheads_kv, head_dim)."""
+        assert inference_params is not None and inference_params.seqlen_offset > 0
+        rotary_cos = rotary_sin = None
+        if self.rotary_emb_dim > 0:
+            assert self.rotary_emb.scale is None, "This code path does not support xPos"
+            self.rotary_emb._update_cos_sin_cache(inference_params.max_seqlen, device=q.device, dtype=q.dtype)
+            rotary_cos, rotary_sin = self.rotary_emb._cos_cached, self.rotary_emb._sin_cached
+        kv_cache, cache_seqlens = self._cache_and_lengths(q.shape[0], inference_params)
+        return flash_attn_with_kvcache(
+            q, kv_cache[:, :, 0], kv_cache[:, :, 1], kv[:, :, 0], kv[:, :, 1], rotary_cos=rotary_cos,
+            rotary_sin=rotary_sin, cache_seqlens=cache_seqlens, softmax_scale=self.softmax_scale, causal=self.causal,
+            window_size=self.window_size,
+            rotary_interleaved=self.rotary_emb.interleaved if self.rotary_emb_dim > 0 else False)
+
+    def _update_kvcache_attention(self, q, kv, inference_params):
+        """q and kv already rotated (or no rotary).  The prompt pass (nothing cached yet) writes the
+        cache and attends within the prompt; later steps append and attend to the cache."""
+        if inference_params.seqlen_offset == 0:
+            kv = self._update_kv_cache(kv, inference_params)
+            return flash_attn_kvpacked_func(q, kv, softmax_scale=self.softmax_scale, causal=self.causal,
+                                            window_size=self.window_size)
+        kv_cache, cache_seqlens = self._cache_and_lengths(q.shape[0], inference_params)
+        return flash_attn_with_kvcache(q, kv_cache[:, :, 0], kv_cache[:, :, 1], kv[:, :, 0], kv[:, :, 1],
+                                       cache_seqlens=cache_seqlens, softmax_scale=self.softmax_scale, causal=self.causal,
+                                       window_size=self.window_size)
+
+    def forward(self, x, inference_params=None):
+        """x (batch, seqlen, embed_dim) -> (batch, seqlen, embed_dim)."""
+        if inference_params is None:
+            seqlen_offset, rotary_max_seqlen = 0, None
+        else:
+            lengths = inference_params.lengths_per_sample
+            seqlen_offset = lengths if lengths is not None else inference_params.seqlen_offset
+            rotary_max_seqlen = inference_params.max_seqlen
+        batch, seqlen = x.shape[:2]
+        qkv = self.Wqkv(x)
+        # the fused rotary + append path needs something cached and a rotary_dim the kernel takes
+        fused = (inference_params is not None and inference_params.seqlen_offset > 0
+                 and self.rotary_emb_dim > 0 and self.rotary_emb_dim % 16 == 0)
+        if self.num_heads_kv == self.num_heads:
+            qkv = qkv.view(batch, seqlen, 3, self.num_heads, self.head_dim)
+            if fused:
+                context = self._apply_rotary_update_kvcache_attention(qkv[:, :, 0], qkv[:, :, 1:], inference_params)
+            else:
+                if self.rotary_emb_dim > 0:
+                    qkv = self.rotary_emb(qkv, seqlen_offset=seqlen_offset, max_seqlen=rotary_max_seqlen)
+                if inference_params is None:
+                    context = flash_attn_qkvpacked_func(qkv, softmax_scale=self.softmax_scale, causal=self.causal,
+                                                        window_size=self.window_size)
+                else:
+                    context = self._update_kvcache_attention(qkv[:, :, 0], qkv[:, :, 1:], inference_params)
+        else:
+            nq = self.num_heads * self.head_dim
+            q = qkv[..., :nq].reshape(batch, seqlen, self.num_heads, self.head_dim)
+            kv = qkv[..., nq:].reshape(batch, seqlen, 2, self.num_heads_kv, self.head_dim)
+            if fused:
+                context = self._apply_rotary_update_kvcache_attention(q, kv, inference_params)
+            else:
+                if self.rotary_emb_dim > 0:
+                    q, kv = self.rotary_emb(q, kv, seqlen_offset=seqlen_offset, max_seqlen=rotary_max_seqlen)
+                if inference_params is None:
+                    context = flash_attn_kvpacked_func(q, kv, softmax_scale=self.softmax_scale, causal=self.causal,
+                                                       window_size=self.window_size)
+                else:
+                    context = self._update_kvcache_attention(q, kv, inference_params)
+        return self.out_proj(context.reshape(batch, seqlen, self.embed_dim))
