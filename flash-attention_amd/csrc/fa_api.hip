@@ -38,7 +38,7 @@ static const int kNumCU = 256;   // MI355X
 
 // The small-q streaming kernel packs seqlen_q x (h / h_k) rows into 16 MFMA columns.
 static bool use_decode_kernel(const fa_fwd_params& p) {
-    return p.cu_seqlens_q == nullptr && (int64_t)p.seqlen_q * (p.h / p.h_k) <= 16;
+    return p.cu_seqlens_q == nullptr && (int64_t)p.seqlen_q * (p.h / p.h_k) <= 16 && p.p_dropout == 0.f;
 }
 
 static int check_common(const fa_fwd_params* p) {
@@ -51,6 +51,9 @@ static int check_common(const fa_fwd_params* p) {
     if (p->h <= 0 || p->h_k <= 0 || p->h % p->h_k != 0) return fail("Number of heads in key/value must divide number of heads in query");
     if (p->seqlen_q < 0 || p->seqlen_k < 0) return fail("sequence lengths must be non-negative");
     if (p->num_splits < 0 || p->num_splits > FA_MAX_SPLITS) return fail("num_splits > 128 not supported");
+    if (!(p->p_dropout >= 0.f && p->p_dropout < 1.f)) return fail("p_dropout must be in [0, 1)");
+    if (p->p_dropout > 0.f && !p->rng_state) return fail("rng_state is required when p_dropout > 0");
+    if (p->s_dmask && (p->sdm_rows < p->seqlen_q || p->sdm_cols < p->seqlen_k)) return fail("s_dmask is smaller than (seqlen_q, seqlen_k)");
     return 0;
 }
 
@@ -71,6 +74,7 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
     auto rup = [](int64_t x, int64_t m) { return (int)((x + m - 1) / m * m); };
     int splits = 1;
     bool automatic = false;
+    if (p.p_dropout > 0.f) allow_split = false;      // as the reference (flash_api.cpp:380)
     if (allow_split && sk > 0) {
         if (p.num_splits > 1) {
             splits = p.num_splits;
@@ -158,6 +162,10 @@ static int run_attention(KParams& kp, hipStream_t stream) {
         e = launch_combine(kp, stream);
         if (e) return fail_hip(e, "combine kernel launch");
     }
+    if (p.s_dmask) {
+        e = launch_attn_probs(kp, stream);
+        if (e) return fail_hip(e, "attention probability kernel launch");
+    }
     return 0;
 }
 
@@ -187,6 +195,8 @@ static int run_bwd(const fa_bwd_params* p, bool varlen, hipStream_t stream) {
     if (p->seqlen_q_rounded < p->seqlen_q) return fail("seqlen_q_rounded must be at least seqlen_q");
     if (varlen && (!p->cu_seqlens_q || !p->cu_seqlens_k)) return fail("fa_varlen_bwd needs cu_seqlens_q and cu_seqlens_k");
     if (!varlen && (p->cu_seqlens_q || p->cu_seqlens_k)) return fail("fa_bwd takes dense batches; use fa_varlen_bwd");
+    if (!(p->p_dropout >= 0.f && p->p_dropout < 1.f)) return fail("p_dropout must be in [0, 1)");
+    if (p->p_dropout > 0.f && !p->rng_state) return fail("rng_state is required when p_dropout > 0");
     const int64_t strides[] = {p->q_row_stride, p->q_head_stride, p->k_row_stride, p->k_head_stride, p->v_row_stride,
                                p->v_head_stride, p->o_row_stride, p->o_head_stride, p->do_row_stride, p->do_head_stride,
                                p->dq_row_stride, p->dq_head_stride, p->dk_row_stride, p->dk_head_stride,
@@ -287,6 +297,7 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
     g_err.clear();
     if (int r = check_common(p)) return r;
     if (p->cu_seqlens_q) return fail("fa_fwd_kvcache takes a dense q batch");
+    if (p->p_dropout != 0.f || p->s_dmask) return fail("fa_fwd_kvcache has no dropout");
     if (p->cu_seqlens_k && p->is_seqlens_k_cumulative) return fail("cache_seqlens must be per-batch lengths, not prefix sums");
     const bool has_new = p->k_new != nullptr;
     if (has_new) {

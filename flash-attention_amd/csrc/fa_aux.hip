@@ -113,4 +113,53 @@ int launch_append_kv(const KParams& kp, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// Testing aid behind return_softmax (the reference's S_dmask, csrc/flash_attn/flash_api.cpp:351-357):
+// s_dmask[b, h, i, j] = exp(scale q_i . k_j - lse_i), negated where dropout removed the entry, 0 where
+// the mask hides it or outside (seqlen_q, seqlen_k).  Runs after the attention kernel, so lse is
+// final and the value is the normalised probability.  One thread per entry, scalar dot product.
+template <typename T>
+__global__ void __launch_bounds__(256) attn_probs_kernel(const KParams kp) {
+    const fa_fwd_params& p = kp.p;
+    const int b = blockIdx.z / p.h, head = blockIdx.z % p.h;
+    const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int j = blockIdx.x * 16 + (threadIdx.x & 15);
+    if (i >= p.sdm_rows || j >= p.sdm_cols) return;
+    const SeqInfo si = seq_info(p, b);
+    const int hk = head / (p.h / p.h_k);
+    const int shift = si.sk - si.sq;
+    bool vis = i < si.sq && j < si.sk;
+    if (kp.has_right) vis = vis && j <= i + shift + p.window_right;
+    if (kp.has_left) vis = vis && j >= i + shift - p.window_left;
+    float val = 0.f;
+    if (vis) {
+        const T* q = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)i * p.q_row_stride + (int64_t)head * p.q_head_stride;
+        const T* k = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)j * p.k_row_stride + (int64_t)hk * p.k_head_stride;
+        float dot = 0.f;
+        for (int c = 0; c < p.d; c += 8) {
+            float a[8], bb[8];
+            unpack8<T>(ld_global16(q + c), a);
+            unpack8<T>(ld_global16(k + c), bb);
+#pragma unroll
+            for (int e = 0; e < 8; e++) dot += a[e] * bb[e];
+        }
+        const float lse = p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + i];
+        val = __expf(dot * p.softmax_scale - lse);
+        if (p.p_dropout > 0.f) {
+            const Drop drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
+            if (!drop_keep(drop, i, j)) val = -val;
+        }
+    }
+    reinterpret_cast<T*>(p.s_dmask)[(((int64_t)b * p.h + head) * p.sdm_rows + i) * p.sdm_cols + j] = (T)val;
+}
+
+int launch_attn_probs(const KParams& kp, hipStream_t stream) {
+    const fa_fwd_params& p = kp.p;
+    if (p.sdm_rows <= 0 || p.sdm_cols <= 0) return 0;
+    dim3 grid((unsigned)((p.sdm_cols + 15) / 16), (unsigned)((p.sdm_rows + 15) / 16), (unsigned)(p.b * p.h));
+    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(attn_probs_kernel<__bf16>, grid, dim3(256), 0, stream, kp);
+    else hipLaunchKernelGGL(attn_probs_kernel<_Float16>, grid, dim3(256), 0, stream, kp);
+    return (int)hipGetLastError();
+}
+
+
 }  // namespace fa

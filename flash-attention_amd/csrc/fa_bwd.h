@@ -130,7 +130,7 @@ struct BwdDqCfg {
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
 };
 
-template <typename T, int D, int BN, int MINW>
+template <typename T, int D, int BN, int MINW, bool DROPOUT>
 __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) {
     typedef BwdDqCfg<T, D, BN> C;
     typedef typename Elem<T>::v8 v8;
@@ -224,6 +224,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     };
 
     const float sl2 = kp.scale_log2;
+    Drop drop = {0, 0, 256, 1.f};
+    if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
     if (t_hi > t_lo) { load_tile(t_lo); store_tile(0, t_lo); }
     __syncthreads();
     int buf = 0;
@@ -261,10 +263,14 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
             v8 dsf[C::PT];
 #pragma unroll
             for (int nb = 0; nb < C::NB; nb++) {
+                uint32_t keep = 0xffffu;
+                if constexpr (DROPOUT) keep = drop_keep16_row(drop, row, n0 + nb * 32, hh);
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const float pv = fast_exp2(s_acc[nb][r] * sl2 - lse2);
-                    s_acc[nb][r] = pv * (dp_acc[nb][r] - dsum);
+                    float dpv = dp_acc[nb][r];
+                    if constexpr (DROPOUT) dpv = (keep >> r) & 1u ? dpv * drop.rp : 0.f;   // gradient through the dropped P
+                    s_acc[nb][r] = pv * (dpv - dsum);
                 }
                 dsf[2 * nb] = pack_acc8<T>(s_acc[nb], 0);
                 dsf[2 * nb + 1] = pack_acc8<T>(s_acc[nb], 8);
@@ -314,7 +320,7 @@ struct BwdDkvCfg {
     static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
 };
 
-template <typename T, int D, int BM, int DPARTS, int MINW>
+template <typename T, int D, int BM, int DPARTS, int MINW, bool DROPOUT>
 __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp) {
     typedef BwdDkvCfg<T, D, BM, DPARTS> C;
     typedef typename Elem<T>::v8 v8;
@@ -420,7 +426,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
     if (iters > 0) { load_tile(0, t_lo); store_tile(0, t_lo); }
     __syncthreads();
     int buf = 0;
-    int cur_t = t_lo, nxt_g = 0, nxt_t = t_lo;       // (head of group, query tile) walked without divisions
+    int cur_t = t_lo, cur_g = 0, nxt_g = 0, nxt_t = t_lo;   // (head of group, query tile) walked without divisions
+    Drop drop = {0, 0, 256, 1.f};
     for (int it = 0; it < iters; ++it) {
         const bool has_next = it + 1 < iters;
         if (has_next) {
@@ -428,6 +435,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
             load_tile(nxt_g, nxt_t);
         }
         const int i0 = cur_t * BM;
+        if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, hk * G + cur_g, p.h);
         const char* qb = smem + buf * C::STAGE;
         const char* gb = qb + C::TILE_BYTES;
         const float* lse_s = reinterpret_cast<const float*>(gb + C::TILE_BYTES);
@@ -459,6 +467,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
                         s_acc[mb][r] = (rel > rel_hi + c_r || rel < rel_lo + c_r) ? -INFINITY : s_acc[mb][r];
                     }
                 }
+                uint32_t keep = 0xffffu;
+                if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
                     const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
@@ -467,8 +477,11 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
                     for (int e = 0; e < 4; e++) {
                         const int r = 4 * q4 + e;
                         const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
-                        s_acc[mb][r] = pv;
-                        dp_acc[mb][r] = pv * (dp_acc[mb][r] - d4[e]);
+                        const bool kept = (keep >> r) & 1u;
+                        float dpv = dp_acc[mb][r];
+                        if constexpr (DROPOUT) dpv = kept ? dpv * drop.rp : 0.f;
+                        s_acc[mb][r] = (!DROPOUT || kept) ? pv : 0.f;
+                        dp_acc[mb][r] = pv * (dpv - d4[e]);
                     }
                 }
                 pf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
@@ -489,12 +502,14 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
         __syncthreads();
         buf ^= 1;
         cur_t = nxt_t;
+        cur_g = nxt_g;
     }
 
     if (!key_ok) return;
     T* dkrow = reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride;
     T* dvrow = reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
     const float sc = p.softmax_scale;
+    const float rp = DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f;
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
@@ -503,8 +518,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
             if (d0 < p.d) {
                 u32x2 a = {pack2<T>(dk_acc[db][4 * q4] * sc, dk_acc[db][4 * q4 + 1] * sc),
                            pack2<T>(dk_acc[db][4 * q4 + 2] * sc, dk_acc[db][4 * q4 + 3] * sc)};
-                u32x2 c = {pack2<T>(dv_acc[db][4 * q4], dv_acc[db][4 * q4 + 1]),
-                           pack2<T>(dv_acc[db][4 * q4 + 2], dv_acc[db][4 * q4 + 3])};
+                u32x2 c = {pack2<T>(dv_acc[db][4 * q4] * rp, dv_acc[db][4 * q4 + 1] * rp),
+                           pack2<T>(dv_acc[db][4 * q4 + 2] * rp, dv_acc[db][4 * q4 + 3] * rp)};
                 st_global8(dkrow + d0, a);
                 st_global8(dvrow + d0, c);
             }
@@ -529,7 +544,7 @@ struct BwdDkv2Cfg {
     static_assert(BM % 32 == 0 && D % 32 == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
 };
 
-template <typename T, int D, int BM>
+template <typename T, int D, int BM, bool DROPOUT>
 __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
     typedef BwdDkv2Cfg<T, D, BM> C;
     typedef typename Elem<T>::v8 v8;
@@ -637,7 +652,8 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
     if (iters > 0) { load_tile(0, t_lo); store_tile(0, t_lo); }
     __syncthreads();
     int buf = 0;
-    int cur_t = t_lo, nxt_g = 0, nxt_t = t_lo;       // (head of group, query tile) walked without divisions
+    int cur_t = t_lo, cur_g = 0, nxt_g = 0, nxt_t = t_lo;   // (head of group, query tile) walked without divisions
+    Drop drop = {0, 0, 256, 1.f};
     for (int it = 0; it < iters; ++it) {
         const bool has_next = it + 1 < iters;
         if (has_next) {
@@ -645,6 +661,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
             load_tile(nxt_g, nxt_t);
         }
         const int i0 = cur_t * BM;
+        if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, hk * G + cur_g, p.h);
         const char* qb = smem + buf * C::STAGE;
         const char* gb = qb + C::TILE_BYTES;
         const float* lse_s = reinterpret_cast<const float*>(gb + C::TILE_BYTES);
@@ -687,14 +704,22 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
                     for (int e = 0; e < 4; e++)
                         s_acc[mb][4 * q4 + e] = fast_exp2(s_acc[mb][4 * q4 + e] * sl2 - l4[e]);
                 }
+                uint32_t keep = 0xffffu;
+                if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);
                 if (role_k) {
 #pragma unroll
                     for (int q4 = 0; q4 < 4; q4++) {
                         const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
 #pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            s_acc[mb][4 * q4 + e] *= dp_acc[mb][4 * q4 + e] - d4[e];
+                        for (int e = 0; e < 4; e++) {
+                            float dpv = dp_acc[mb][4 * q4 + e];
+                            if constexpr (DROPOUT) dpv = (keep >> (4 * q4 + e)) & 1u ? dpv * drop.rp : 0.f;
+                            s_acc[mb][4 * q4 + e] *= dpv - d4[e];
+                        }
                     }
+                } else if constexpr (DROPOUT) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s_acc[mb][r] = (keep >> r) & 1u ? s_acc[mb][r] : 0.f;
                 }
                 bf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
                 bf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
@@ -711,12 +736,13 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
         __syncthreads();
         buf ^= 1;
         cur_t = nxt_t;
+        cur_g = nxt_g;
     }
 
     if (!key_ok) return;
     T* orow = role_k ? reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride
                      : reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
-    const float sc = role_k ? p.softmax_scale : 1.f;
+    const float sc = role_k ? p.softmax_scale : (DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f);
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
@@ -737,40 +763,40 @@ template <typename K> static int bwd_set_smem(K kern, int bytes) {
     return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-template <typename T, int D, int BN, int MINW>
+template <typename T, int D, int BN, int MINW, bool DROPOUT>
 int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDqCfg<T, D, BN> C;
     const int64_t total = (int64_t)((kp.p.seqlen_q + C::BM - 1) / C::BM) * kp.p.h * kp.p.b;
     if (total <= 0) return 0;
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    auto kern = bwd_dq_kernel<T, D, BN, MINW>;
+    auto kern = bwd_dq_kernel<T, D, BN, MINW, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
 
-template <typename T, int D, int BM, int DPARTS, int MINW>
+template <typename T, int D, int BM, int DPARTS, int MINW, bool DROPOUT>
 int launch_bwd_dkv(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDkvCfg<T, D, BM, DPARTS> C;
     const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b * DPARTS;
     if (total <= 0) return 0;
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    auto kern = bwd_dkv_kernel<T, D, BM, DPARTS, MINW>;
+    auto kern = bwd_dkv_kernel<T, D, BM, DPARTS, MINW, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
 
-template <typename T, int D, int BM>
+template <typename T, int D, int BM, bool DROPOUT>
 int launch_bwd_dkv2(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDkv2Cfg<T, D, BM> C;
     const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b;
     if (total <= 0) return 0;
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    auto kern = bwd_dkv2_kernel<T, D, BM>;
+    auto kern = bwd_dkv2_kernel<T, D, BM, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();

@@ -15,15 +15,20 @@ typedef _Float16 InstT;
 
 // dQ pass then dK/dV pass on the same stream; both read softmax_d, which the caller's stream has
 // already filled (launch_bwd_dot).
-int FA_INST_NAME(FA_D)(const BwdKParams& kp, hipStream_t stream) {
+template <bool DROPOUT>
+static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers
-    if (int e = launch_bwd_dq<InstT, FA_D, (FA_D > 64 ? 32 : 64), 2>(kp, stream)) return e;
-    return launch_bwd_dkv2<InstT, FA_D, 64>(kp, stream);
+    if (int e = launch_bwd_dq<InstT, FA_D, (FA_D > 64 ? 32 : 64), 2, DROPOUT>(kp, stream)) return e;
+    return launch_bwd_dkv2<InstT, FA_D, 64, DROPOUT>(kp, stream);
 #else
-    if (int e = launch_bwd_dq<InstT, FA_D, 32, 1>(kp, stream)) return e;
-    return launch_bwd_dkv<InstT, FA_D, 32, 2, 1>(kp, stream);
+    if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
+    return launch_bwd_dkv<InstT, FA_D, 32, 2, 1, DROPOUT>(kp, stream);
 #endif
+}
+
+int FA_INST_NAME(FA_D)(const BwdKParams& kp, hipStream_t stream) {
+    return kp.p.p_dropout > 0.f ? run<true>(kp, stream) : run<false>(kp, stream);
 }
 
 #if FA_D == 64

@@ -125,6 +125,75 @@ template <int D> FA_DEV int swz_u(int chunk, int row) {
     else return chunk ^ ((row >> 2) & 3);   // D == 32
 }
 
+// ------------------------------------------------------------------------------------------------
+// Dropout mask.  keep(b, h, i, j) is a pure function of (seed, offset, b, h, i, j): one 32-bit hash
+// per 2 x 2 block of (row, key) supplies four random bytes, byte (i & 1) * 2 + (j & 1) belongs to
+// element (i, j), and the element is kept iff its byte is below `thresh` (keep probability in 1/256
+// steps, csrc/flash_attn/flash_api.cpp:104).  The 2 x 2 unit costs the same number of hashes in
+// both register geometries: a lane that owns one row and 4 consecutive keys (forward, dQ kernel)
+// and a lane that owns one key and 4 consecutive rows (dK / dV kernel).
+// ------------------------------------------------------------------------------------------------
+struct Drop {
+    uint32_t k0, k1;     // per (batch, head) keys derived from seed and offset
+    uint32_t thresh;     // 1..256
+    float rp;            // 1 / (1 - p_dropout)
+};
+FA_DEV uint32_t fmix32(uint32_t h) {
+    h ^= h >> 16; h *= 0x85ebca6bu; h ^= h >> 13; h *= 0xc2b2ae35u; h ^= h >> 16;
+    return h;
+}
+FA_DEV Drop drop_init(const uint64_t* rng_state, float p_dropout, int b, int h, int nheads) {
+    Drop d;
+    const uint64_t seed = rng_state[0], off = rng_state[1];
+    const uint32_t bh = (uint32_t)(b * nheads + h);
+    d.k0 = fmix32((uint32_t)seed ^ fmix32((uint32_t)(seed >> 32) + bh * 0x9e3779b1u));
+    d.k1 = fmix32(d.k0 + (uint32_t)off * 0x7f4a7c15u + fmix32((uint32_t)(off >> 32) ^ 0x2545f491u));
+    const float keep = 1.f - p_dropout;
+    d.thresh = (uint32_t)floorf(keep * 255.f) + 1u;
+    d.rp = 1.f / keep;
+    return d;
+}
+FA_DEV uint32_t drop_hash(const Drop& d, uint32_t i2, uint32_t j2) {
+    return fmix32((i2 * 0x9e3779b1u + d.k0) ^ (j2 * 0x85ebca77u + d.k1));
+}
+FA_DEV bool drop_keep(const Drop& d, int i, int j) {          // one element (any kernel)
+    const uint32_t w = drop_hash(d, (uint32_t)i >> 1, (uint32_t)j >> 1);
+    return ((w >> (8 * ((i & 1) * 2 + (j & 1)))) & 0xffu) < d.thresh;
+}
+// Bit r of the result = keep for accumulator register r of a 32 x 32 block whose lane owns ROW `row`
+// and whose registers walk keys kb0 + 8 (r >> 2) + 4 hh + (r & 3)   (kb0 a multiple of 32).
+FA_DEV uint32_t drop_keep16_row(const Drop& d, int row, int kb0, int hh) {
+    uint32_t bits = 0;
+    const uint32_t sh = (row & 1) * 16;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const uint32_t j2 = (uint32_t)(kb0 + 8 * q + 4 * hh) >> 1;
+        const uint32_t wa = drop_hash(d, (uint32_t)row >> 1, j2) >> sh;
+        const uint32_t wb = drop_hash(d, (uint32_t)row >> 1, j2 + 1) >> sh;
+        bits |= (uint32_t)((wa & 0xffu) < d.thresh) << (4 * q);
+        bits |= (uint32_t)(((wa >> 8) & 0xffu) < d.thresh) << (4 * q + 1);
+        bits |= (uint32_t)((wb & 0xffu) < d.thresh) << (4 * q + 2);
+        bits |= (uint32_t)(((wb >> 8) & 0xffu) < d.thresh) << (4 * q + 3);
+    }
+    return bits;
+}
+// Same for a block whose lane owns KEY `key` and whose registers walk rows rb0 + 8 (r >> 2) + 4 hh + (r & 3).
+FA_DEV uint32_t drop_keep16_key(const Drop& d, int key, int rb0, int hh) {
+    uint32_t bits = 0;
+    const uint32_t sh = (key & 1) * 8;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const uint32_t i2 = (uint32_t)(rb0 + 8 * q + 4 * hh) >> 1;
+        const uint32_t wa = drop_hash(d, i2, (uint32_t)key >> 1) >> sh;
+        const uint32_t wb = drop_hash(d, i2 + 1, (uint32_t)key >> 1) >> sh;
+        bits |= (uint32_t)((wa & 0xffu) < d.thresh) << (4 * q);
+        bits |= (uint32_t)(((wa >> 16) & 0xffu) < d.thresh) << (4 * q + 1);
+        bits |= (uint32_t)((wb & 0xffu) < d.thresh) << (4 * q + 2);
+        bits |= (uint32_t)(((wb >> 16) & 0xffu) < d.thresh) << (4 * q + 3);
+    }
+    return bits;
+}
+
 // Rotary embedding of 8 consecutive elements [d0, d0+8) of one row, fp32 math.
 // `x` are the row's own values, `row_ptr` points at the row start (to fetch the partner half for
 // the non-interleaved form), cos/sin point at the table row for this token.

@@ -20,6 +20,7 @@ int launch_decode(const KParams& kp, hipStream_t stream);      // small-q split-
 int launch_zero_counter(int32_t* c, hipStream_t stream);     // ticket counter of the persistent decode
 int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials
 int launch_append_kv(const KParams& kp, hipStream_t stream);   // k_new/v_new (+rotary) -> cache
+int launch_attn_probs(const KParams& kp, hipStream_t stream);  // s_dmask: signed softmax probabilities (testing)
 int launch_rotary(const fa_rotary_params& p, hipStream_t stream);   // standalone rotary embedding
 
 #define FA_DECL_BWD(name) int name(const BwdKParams& kp, hipStream_t stream);

@@ -37,7 +37,7 @@ struct PrefillCfg {
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
 };
 
-template <typename T, int D, int RB, int BN, int MINW, bool SPLIT>
+template <typename T, int D, int RB, int BN, int MINW, bool SPLIT, bool DROPOUT = false>
 __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     typedef PrefillCfg<T, D, RB, BN> C;
     typedef typename Elem<T>::v8 v8;
@@ -161,6 +161,8 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
 
     const float sl2 = kp.scale_log2;
+    Drop drop = {0, 0, 256, 1.f};
+    if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
 
     if (t_hi > t_lo) {
         load_tile(t_hi - 1);
@@ -252,6 +254,16 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                     }
                 l_run[rb] = l_run[rb] * corr + sum;
                 m_run[rb] = m_new;
+                if constexpr (DROPOUT) {
+                    // the row sum above is of the undropped probabilities; dropped entries leave the
+                    // second product only, and 1 / (1 - p) is applied once in the epilogue
+#pragma unroll
+                    for (int nb = 0; nb < C::NB; nb++) {
+                        const uint32_t keep = drop_keep16_row(drop, r0 + l32, n0 + nb * 32, hh);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) s_acc[rb][nb][r] = (keep >> r) & 1u ? s_acc[rb][nb][r] : 0.f;
+                    }
+                }
                 if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
 #pragma unroll
                     for (int db = 0; db < C::DB; db++)
@@ -300,7 +312,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
         const int row = m0 + (wave * RB + rb) * 32 + l32;
         const float l_tot = xhalf_sum(l_run[rb]);
         const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
-        const float inv = dead ? 1.f : 1.f / l_tot;
+        const float inv = dead ? 1.f : drop.rp / l_tot;
         const float lse = dead ? (SPLIT ? -INFINITY : INFINITY) : m_run[rb] * p.softmax_scale + __logf(l_tot);
         if (row >= si.sq) continue;
         if (SPLIT) {
@@ -349,6 +361,11 @@ int launch_prefill(KParams kp, hipStream_t stream) {
     hipError_t e;
     if (split) {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, true>;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    } else if (kp.p.p_dropout > 0.f) {
+        auto kern = prefill_kernel<T, D, RB, BN, MINW, false, true>;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);

@@ -43,7 +43,9 @@ class FaFwdParams(ctypes.Structure):
             "b", "h", "h_k", "seqlen_q", "seqlen_k", "seqlen_knew", "d", "rotary_dim",
             "window_left", "window_right", "is_causal", "is_seqlens_k_cumulative",
             "is_rotary_interleaved", "num_splits", "dtype")]
-        + [("softmax_scale", ctypes.c_float)]
+        + [("softmax_scale", ctypes.c_float), ("p_dropout", ctypes.c_float),
+           ("rng_state", ctypes.c_void_p), ("s_dmask", ctypes.c_void_p),
+           ("sdm_rows", ctypes.c_int32), ("sdm_cols", ctypes.c_int32)]
     )
 
 
@@ -70,6 +72,7 @@ class FaBwdParams(ctypes.Structure):
         + [(n, ctypes.c_int32) for n in ("b", "seqlen_q", "seqlen_k", "h", "h_k", "d", "seqlen_q_rounded")]
         + [("softmax_scale", ctypes.c_float)]
         + [(n, ctypes.c_int32) for n in ("is_causal", "window_left", "window_right", "dtype")]
+        + [("p_dropout", ctypes.c_float), ("rng_state", ctypes.c_void_p)]
     )
 
 
@@ -158,6 +161,28 @@ def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def _dropout_state(p, p_dropout, return_softmax, gen_, batch, heads, seqlen_q, seqlen_k, dtype, device):
+    """Seed / offset of the dropout mask taken from (and advancing) torch's generator for the device,
+    like the reference does with its Philox state (flash_api.cpp:396-408), and the optional
+    probability tensor behind return_softmax (:351-357).  Returns (rng_state, s_dmask)."""
+    _check(0.0 <= p_dropout < 1.0, "p_dropout must be in [0, 1)")
+    rng_state = torch.empty((2,), dtype=torch.int64, device=device)
+    s_dmask = None
+    if return_softmax:
+        _check(p_dropout > 0.0, "return_softmax is only supported when p_dropout > 0.0")
+        s_dmask = torch.empty((batch, heads, _round_up(seqlen_q, 128), _round_up(seqlen_k, 128)), dtype=dtype, device=device)
+        p.s_dmask, p.sdm_rows, p.sdm_cols = s_dmask.data_ptr(), s_dmask.shape[2], s_dmask.shape[3]
+    if p_dropout > 0.0:
+        gen = gen_ if gen_ is not None else torch.cuda.default_generators[device.index if device.index is not None
+                                                                       else torch.cuda.current_device()]
+        seed, offset = gen.initial_seed(), gen.get_offset()
+        gen.set_offset(offset + batch * heads * 32)
+        host = torch.tensor([ctypes.c_int64(seed).value, ctypes.c_int64(offset).value], dtype=torch.int64)
+        rng_state.copy_(host)
+        p.p_dropout, p.rng_state = p_dropout, rng_state.data_ptr()
+    return rng_state, s_dmask
+
+
 def _plan_and_alloc(params, api, batch, heads, seqlen_q, d, device):
     """Resolve the split count and allocate the fp32 partial buffers like the reference does
     (flash_api.cpp:373-389, 1241-1257).  The returned tensors must stay alive until launch."""
@@ -180,8 +205,6 @@ def _plan_and_alloc(params, api, batch, heads, seqlen_q, d, device):
 def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, window_size_right,
         return_softmax, gen_):
     """Dense batch forward; mirrors mha_fwd (flash_api.cpp:248-424)."""
-    if p_dropout != 0.0:
-        raise NotImplementedError("dropout is not implemented in the MI355X forward path")
     q_dtype = q.dtype
     dt = _dtype_code(q_dtype)
     _check(k.dtype == q_dtype, "query and key must have the same dtype")
@@ -197,7 +220,6 @@ def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, wi
     _check(num_heads % num_heads_k == 0, "Number of heads in key/value must divide number of heads in query")
     _check(tuple(k.shape) == (batch_size, seqlen_k, num_heads_k, head_size_og), "k must have shape (batch_size, seqlen_k, num_heads_k, head_size)")
     _check(tuple(v.shape) == (batch_size, seqlen_k, num_heads_k, head_size_og), "v must have shape (batch_size, seqlen_k, num_heads_k, head_size)")
-    _check(not return_softmax, "return_softmax is only supported when p_dropout > 0.0")
     if seqlen_q == 1:
         is_causal = False
     if is_causal:
@@ -232,6 +254,8 @@ def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, wi
         p.num_splits = 0
         p.dtype = dt
         p.softmax_scale = softmax_scale
+        rng_state, s_dmask = _dropout_state(p, p_dropout, return_softmax, gen_, batch_size, num_heads, seqlen_q,
+                                            seqlen_k, q_dtype, q.device)
         if seqlen_q > 0 and seqlen_k > 0:
             keep = _plan_and_alloc(p, 0, batch_size, num_heads, seqlen_q, head_size, q.device)
             _call(lib.fa_fwd, p, _stream(q.device))
@@ -239,22 +263,21 @@ def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, wi
         else:
             out.zero_()
             softmax_lse.fill_(float("inf"))
+            if s_dmask is not None:
+                s_dmask.zero_()
 
     out_padded = out
     if head_size_og % 8 != 0:
         out = out[..., :head_size_og]
         if out_ is not None:
             out_.copy_(out)
-    rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
-    return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, None, rng_state]
+    return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, s_dmask, rng_state]
 
 
 def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout,
                softmax_scale, zero_tensors, is_causal, window_size_left, window_size_right,
                return_softmax, gen_):
     """Packed variable-length forward; mirrors mha_varlen_fwd (flash_api.cpp:426-585)."""
-    if p_dropout != 0.0:
-        raise NotImplementedError("dropout is not implemented in the MI355X forward path")
     q_dtype = q.dtype
     dt = _dtype_code(q_dtype)
     _check(k.dtype == q_dtype, "query and key must have the same dtype")
@@ -277,7 +300,6 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
     _check(tuple(v.shape) == (total_k, num_heads_k, head_size_og), "v must have shape (total_k, num_heads_k, head_size)")
     _check(tuple(cu_seqlens_q.shape) == (batch_size + 1,), "cu_seqlens_q must have shape (batch_size + 1)")
     _check(tuple(cu_seqlens_k.shape) == (batch_size + 1,), "cu_seqlens_k must have shape (batch_size + 1)")
-    _check(not return_softmax, "return_softmax is only supported when p_dropout > 0.0")
     if is_causal:
         window_size_right = 0
 
@@ -314,16 +336,19 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
         p.num_splits = 1
         p.dtype = dt
         p.softmax_scale = softmax_scale
+        rng_state, s_dmask = _dropout_state(p, p_dropout, return_softmax, gen_, batch_size, num_heads, max_seqlen_q,
+                                            max_seqlen_k, q_dtype, q.device)
         if total_q > 0 and max_seqlen_q > 0:
             _call(lib.fa_varlen_fwd, p, _stream(q.device))
+        elif s_dmask is not None:
+            s_dmask.zero_()
 
     out_padded = out
     if head_size_og % 8 != 0:
         out = out[..., :head_size_og]
         if out_ is not None:
             out_.copy_(out)
-    rng_state = torch.empty((2,), dtype=torch.int64, device=q.device)
-    return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, None, rng_state]
+    return [out, q_padded, k_padded, v_padded, out_padded, softmax_lse, s_dmask, rng_state]
 
 
 def _set_strides(p, name, t):
@@ -336,8 +361,7 @@ def _set_strides(p, name, t):
 
 
 def _bwd_common(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, what):
-    if p_dropout != 0.0:
-        raise NotImplementedError("dropout is not implemented in the MI355X backward path")
+    _check(0.0 <= p_dropout < 1.0, "p_dropout must be in [0, 1)")
     q_dtype = q.dtype
     dt = _dtype_code(q_dtype)
     _check(k.dtype == q_dtype, "query and key must have the same dtype")
@@ -379,7 +403,12 @@ def _slice_grads(dq, dk, dv, head_size_og):
     return [dq, dk, dv]
 
 
-def _fill_bwd(p, dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal, wl, wr, dt):
+def _fill_bwd(p, dout, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal, wl, wr, dt,
+              p_dropout=0.0, rng_state=None):
+    if p_dropout > 0.0:
+        _check(rng_state is not None and rng_state.is_cuda and rng_state.dtype == torch.int64 and rng_state.numel() == 2,
+               "rng_state (the forward's, 2 x int64 on the GPU) is required when dropout_p > 0")
+        p.p_dropout, p.rng_state = p_dropout, rng_state.data_ptr()
     p.dout, p.q, p.k, p.v, p.out = dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     p.softmax_lse, p.softmax_d = softmax_lse.data_ptr(), softmax_d.data_ptr()
     p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
@@ -407,7 +436,7 @@ def bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, softmax_scale
         softmax_d = torch.empty((batch_size, num_heads, seqlen_q_rounded), dtype=torch.float32, device=q.device)
         p = FaBwdParams()
         _fill_bwd(p, dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal,
-                  window_size_left, window_size_right, dt)
+                  window_size_left, window_size_right, dt, p_dropout, rng_state)
         p.b, p.seqlen_q, p.seqlen_k, p.seqlen_q_rounded = batch_size, seqlen_q, seqlen_k, seqlen_q_rounded
         if seqlen_q > 0 and seqlen_k > 0:
             _call(lib.fa_bwd, p, _stream(q.device))
@@ -440,7 +469,7 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
             dq.zero_(); dk.zero_(); dv.zero_(); softmax_d.zero_()
         p = FaBwdParams()
         _fill_bwd(p, dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal,
-                  window_size_left, window_size_right, dt)
+                  window_size_left, window_size_right, dt, p_dropout, rng_state)
         p.cu_seqlens_q, p.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
         p.b, p.seqlen_q, p.seqlen_k, p.seqlen_q_rounded = batch_size, max_seqlen_q, max_seqlen_k, seqlen_q_rounded
         if max_seqlen_q > 0 and max_seqlen_k > 0 and total_q > 0 and k.shape[0] > 0:

@@ -85,6 +85,20 @@ typedef struct fa_fwd_params {
     int32_t num_splits;   /* request: 0 = library decides, 1 = never split, n = at most n chunks */
     int32_t dtype;        /* FA_DTYPE_* */
     float softmax_scale;
+
+    /* Dropout on the attention probabilities (fa_fwd and fa_varlen_fwd; csrc/flash_attn/flash_api.cpp:
+     * 99-107, 396-408).  p_dropout is the probability of DROPPING an entry, 0 = none.  The mask is a pure
+     * function of (rng_state[0] = seed, rng_state[1] = offset, batch, head, row, key): the backward
+     * regenerates it from the same two words.  The keep probability is quantised to 8 bits as in
+     * the reference (:104).  With dropout the key range is never split (:380). */
+    float p_dropout;
+    const uint64_t *rng_state;   /* device memory, 2 words; required when p_dropout > 0 */
+    /* Optional, for testing (the reference's return_softmax): (b, h, sdm_rows, sdm_cols) in the q
+     * dtype, row-major, receives the softmax probability of every (row, key), negated where dropout
+     * removed it, 0 outside the mask.  Unlike the reference's S_dmask (which is stored in the order
+     * of its CUDA MMA fragments) entry [i][j] is plainly row i, key j. */
+    void *s_dmask;
+    int32_t sdm_rows, sdm_cols;  /* >= seqlen_q, >= seqlen_k */
 } fa_fwd_params;
 
 /*
@@ -182,7 +196,7 @@ int32_t fa_sizeof_rotary_params(void);
  * for packed input).  softmax_d is caller-provided work space AND a result, as in the reference:
  * (b, h, seqlen_q_rounded) fp32, seqlen_q_rounded >= seqlen_q, receiving rowsum(dout * out).
  * dk and dv are written at h_k heads: the sum over the query heads of a group happens inside the
- * kernel, no expanded buffer is needed.  Dropout is not supported.  Results are deterministic (no
+ * kernel, no expanded buffer is needed.  Results are deterministic (no
  * atomics): dq is produced by one pass over query tiles, dk / dv by one pass over key tiles.
  */
 typedef struct fa_bwd_params {
@@ -209,6 +223,8 @@ typedef struct fa_bwd_params {
     int32_t is_causal;
     int32_t window_left, window_right;
     int32_t dtype;                  /* FA_DTYPE_* */
+    float p_dropout;                /* as in the forward; 0 = none */
+    const uint64_t *rng_state;      /* device memory, the forward's {seed, offset}; required when p_dropout > 0 */
 } fa_bwd_params;
 
 /* mha_bwd (flash_api.cpp:609-832): dense batch; cu_seqlens_* must be NULL. */

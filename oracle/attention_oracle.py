@@ -76,7 +76,8 @@ def visible_mask(seqlen_q: int, seqlen_k: int, window_size=(-1, -1), causal: boo
 # --------------------------------------------------------------------------------------------
 def attention_forward(q, k, v, causal=False, window_size=(-1, -1), softmax_scale=None,
                       seqlens_q=None, seqlens_k=None, upcast=True, reorder_ops=False,
-                      head_block: int = 4) -> Tuple[torch.Tensor, torch.Tensor]:
+                      head_block: int = 4, dropout_p: float = 0.0,
+                      dropout_mask=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """out (b, sq, h, d) in q's dtype and lse (b, h, sq) fp32.
 
     Follows the reference oracle (`tests/test_flash_attn.py:183-259`): with `upcast` the inputs are
@@ -86,6 +87,9 @@ def attention_forward(q, k, v, causal=False, window_size=(-1, -1), softmax_scale
     rounding noise of an ordinary low-precision implementation.  GQA/MQA: query head h reads
     key/value head h // (H / H_k) (`:222-223`).  seqlens_q / seqlens_k give per-batch valid lengths
     (the reference's padding masks, `:229-258`): padded keys are invisible, padded query rows give 0.
+    dropout_mask (b, h, sq, sk) bool, True = keep: probabilities are zeroed where False and the rest
+    scaled by 1 / (1 - dropout_p) AFTER the softmax, so the log-sum-exp is that of the undropped
+    scores (`:247-251`).
     """
     b, sq, h, d = q.shape
     _, sk, hk, _ = k.shape
@@ -126,6 +130,8 @@ def attention_forward(q, k, v, causal=False, window_size=(-1, -1), softmax_scale
                 p = p.masked_fill(dead, 0.0)
                 lse_blk = torch.where(dead.squeeze(-1).expand_as(lse_blk),
                                       torch.full_like(lse_blk, float("inf")), lse_blk)
+            if dropout_mask is not None:
+                p = p.masked_fill(~dropout_mask[ib, h0:h1], 0.0) * (1.0 / (1.0 - dropout_p))
             o = torch.einsum("hts,shd->thd", p, vh)
             if seqlens_q is not None:
                 pad_rows = torch.arange(sq) >= int(seqlens_q[ib])
@@ -136,7 +142,8 @@ def attention_forward(q, k, v, causal=False, window_size=(-1, -1), softmax_scale
 
 
 def attention_backward(q, k, v, dout, causal=False, window_size=(-1, -1), softmax_scale=None,
-                       seqlens_q=None, seqlens_k=None, dtype=torch.float32):
+                       seqlens_q=None, seqlens_k=None, dtype=torch.float32, dropout_p: float = 0.0,
+                       dropout_mask=None):
     """(dq, dk, dv) in `dtype` (fp32, or fp64 for the finite-difference check), unrounded.
 
     The backward kernel's own formulas (`csrc/flash_attn/src/flash_bwd_kernel.h:79-780`), evaluated per
@@ -144,7 +151,9 @@ def attention_backward(q, k, v, dout, causal=False, window_size=(-1, -1), softma
     that sees none), dV = P^T dO, dP = dO V^T, D_i = sum_d dO[i,d] O[i,d], dS = P o (dP - D),
     dQ = scale dS K, dK = scale dS^T Q; with GQA / MQA the dK, dV of a key head are summed over the
     query heads that read it (`csrc/flash_attn/flash_api.cpp:799-803`).  Padded query rows
-    (seqlens_q) contribute nothing and get dQ = 0; padded keys get dK = dV = 0."""
+    (seqlens_q) contribute nothing and get dQ = 0; padded keys get dK = dV = 0.
+    With dropout (mask M, r = 1 / (1 - p)): O = (P o M r) V, so dV = (P o M r)^T dO and
+    dP = (dO V^T) o M r, with D still rowsum(dO o O) (`flash_bwd_kernel.h:411-460`)."""
     b, sq, h, d = q.shape
     _, sk, hk, _ = k.shape
     g = h // hk
@@ -162,10 +171,16 @@ def attention_backward(q, k, v, dout, causal=False, window_size=(-1, -1), softma
             s = (qf[ib, :, ih] @ kf[ib, :, jk].T) * scale
             s = s.masked_fill(~vis, float("-inf"))
             p = torch.softmax(s, dim=-1).masked_fill(dead, 0.0)
-            o = p @ vf[ib, :, jk]
+            pd = p
+            if dropout_mask is not None:
+                keep = dropout_mask[ib, ih].to(dtype) * (1.0 / (1.0 - dropout_p))
+                pd = p * keep
+            o = pd @ vf[ib, :, jk]
             do = gf[ib, :, ih]
-            dv[ib, :, jk] += p.T @ do
+            dv[ib, :, jk] += pd.T @ do
             dp = do @ vf[ib, :, jk].T
+            if dropout_mask is not None:
+                dp = dp * keep
             dsum = (do * o).sum(dim=-1, keepdim=True)
             ds = p * (dp - dsum)
             dq[ib, :, ih] = scale * (ds @ kf[ib, :, jk])

@@ -64,6 +64,10 @@ def test_backward_argument_errors_do_not_abort(lib):
     assert lib.fa_varlen_bwd(ctypes.byref(p), None) != 0 and b"cu_seqlens" in lib.fa_last_error()
     p.q_row_stride = 4
     assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"strides" in lib.fa_last_error()
+    p.q_row_stride, p.p_dropout = 0, 0.1
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"rng_state" in lib.fa_last_error()
+    p.p_dropout = 1.0
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"p_dropout" in lib.fa_last_error()
 
 
 def test_reference_heuristic_matches_oracle(lib):

@@ -341,3 +341,24 @@ def test_backward_closed_forms():
     dq, dk, dv = orc.attention_backward(torch.zeros_like(q), k, v, do)
     assert dk.abs().max() < 1e-6
     assert torch.allclose(dv, (want / sk)[:, None].expand_as(dv), atol=1e-5)
+
+
+def test_dropout_restatement():
+    """Dropout in the oracle: the forward zeroes masked probabilities after the softmax and scales
+    by 1 / (1 - p) (so an all-kept mask with p = 0.5 doubles the output and leaves lse alone), and
+    the backward formulas with the mask equal autograd through that forward."""
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(2, 9, 4, 8, generator=g, dtype=torch.float64)
+    k = torch.randn(2, 11, 2, 8, generator=g, dtype=torch.float64)
+    v = torch.randn(2, 11, 2, 8, generator=g, dtype=torch.float64)
+    do = torch.randn(2, 9, 4, 8, generator=g, dtype=torch.float64)
+    o0, l0 = orc.attention_forward(q, k, v, causal=True, upcast=False)
+    o1, l1 = orc.attention_forward(q, k, v, causal=True, upcast=False, dropout_p=0.5,
+                                   dropout_mask=torch.ones(2, 4, 9, 11, dtype=torch.bool))
+    assert torch.allclose(o1, 2 * o0) and torch.equal(l0, l1)
+    m = torch.rand(2, 4, 9, 11, generator=g) > 0.3
+    # one dropped key: the output loses exactly that key's share
+    a = orc.attention_backward(q, k, v, do, dtype=torch.float64, causal=True, dropout_p=0.3, dropout_mask=m)
+    c = orc.attention_backward_autograd(q, k, v, do, upcast=False, causal=True, dropout_p=0.3, dropout_mask=m)
+    for x, y in zip(a, c):
+        assert (x - y).abs().max() < 1e-12
