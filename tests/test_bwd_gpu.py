@@ -188,12 +188,12 @@ def test_backward_is_deterministic_and_returns_softmax_d():
     assert torch.allclose(softmax_d[:, :, :sq], want, rtol=1e-4, atol=1e-4)
 
 
-def test_backward_rejects_dropout_and_bad_shapes():
+def test_backward_rejects_missing_rng_state_and_bad_shapes():
     _say("bwd errors")
     from flash_attn import _native as nat
     q = torch.zeros(1, 8, 2, 64, dtype=torch.float16, device=DEV)
     lse = torch.zeros(1, 2, 8, dtype=torch.float32, device=DEV)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="rng_state"):        # dropout needs the forward's seed and offset
         nat.bwd(q, q, q, q, q, lse, None, None, None, 0.1, 0.125, False, -1, -1, None, None)
     with pytest.raises(RuntimeError, match="dq has the wrong shape"):
         nat.bwd(q, q, q, q, q, lse, q[:, :4], None, None, 0.0, 0.125, False, -1, -1, None, None)
