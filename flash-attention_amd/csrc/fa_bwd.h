@@ -58,6 +58,12 @@ FA_DEV BwdSeq bwd_seq(const fa_bwd_params& p, int b) {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// s_waitcnt vmcnt(0): placed after the resident operands are loaded, before the tile loop.  Without it
+// the compiler cannot prove inside the loop that those loads have landed (a zero-trip path skips the
+// first tile's wait) and guards the first product of every step with vmcnt(0), which also waits for
+// the NEXT tile's prefetch, i.e. it serialises the prefetch with the products.
+FA_DEV void wait_resident_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // accumulate step dk of a product; step 0 starts from an inline zero instead of a cleared accumulator
 template <typename T> FA_DEV void mfma_step(f32x16& acc, typename Elem<T>::v8 a, typename Elem<T>::v8 b, int dk) {
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -87,6 +93,97 @@ template <typename T> FA_DEV typename Elem<T>::v8 pack_acc8(const f32x16& a, int
 #pragma unroll
     for (int e = 0; e < 4; e++) pk[e] = pack2<T>(a[r8 + 2 * e], a[r8 + 2 * e + 1]);
     return __builtin_bit_cast(typename Elem<T>::v8, pk);
+}
+
+// Per-lane LDS offsets of both read patterns, computed once: the swizzle only involves row & 15, so a
+// block of 32 rows (row-wise) or 16 rows (transposed) further down is a compile-time byte offset.
+template <int D, int KS, int DB>
+struct LdsOffs {
+    int r[KS];       // row-wise: row l32, k-step dk
+    int c[DB][2];    // transposed: column block db, rows 4hh + tj and 8 more
+    FA_DEV void init(int lane) {
+        const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+        for (int dk = 0; dk < KS; dk++) r[dk] = l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16;
+        const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
+        const int row = 4 * hh + tj;
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+            const int cc = db * 4 + dhalf * 2 + (tq >> 1);
+            c[db][0] = row * (D * 2) + swz_u<D>(cc, row) * 16 + (tq & 1) * 8;
+            c[db][1] = (row + 8) * (D * 2) + swz_u<D>(cc, row + 8) * 16 + (tq & 1) * 8;
+        }
+    }
+};
+template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_rows_at(const char* tile, int off, int blk32) {
+    const u32x4 raw = *reinterpret_cast<const u32x4*>(tile + off + blk32 * 32 * (D * 2));
+    return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_cols_at(const char* tile, int off_lo, int off_hi, int t16) {
+    const u32x2 lo = lds_read_tr16(tile + off_lo + t16 * 16 * (D * 2));
+    const u32x2 hi = lds_read_tr16(tile + off_hi + t16 * 16 * (D * 2));
+    const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+
+// Tile products whose A operands come from LDS, software-pipelined by hand: the operands of GRP MFMAs
+// are read one group ahead into a second register set, and a scheduling fence keeps every group's
+// reads in front of the previous group's MFMAs.  (Left to itself the compiler issues read, wait,
+// MFMA, read, wait, MFMA ... with one operand register set, and every MFMA pays an LDS round trip.)
+//
+// acc[blk] (+)= rows [32 blk, 32 blk + 32) of `tile`  x  bfrag[dk]   for blk < NBLK, dk < KS
+template <typename T, int D, int NBLK, int KS, int GRP>
+FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const typename Elem<T>::v8* bfrag) {
+    typedef typename Elem<T>::v8 v8;
+    constexpr int TOTAL = NBLK * KS, NG = TOTAL / GRP;
+    static_assert(TOTAL % GRP == 0 && KS % GRP == 0, "group shape");
+    v8 a[2][GRP];
+#pragma unroll
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_rows_at<T, D>(tile, offr[j % KS], j / KS);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        if (g + 1 < NG) {
+#pragma unroll
+            for (int j = 0; j < GRP; j++) {
+                const int st = (g + 1) * GRP + j;
+                a[(g + 1) & 1][j] = lds_rows_at<T, D>(tile, offr[st % KS], st / KS);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < GRP; j++) {
+            const int st = g * GRP + j;
+            mfma_step<T>(acc[st / KS], a[g & 1][j], bfrag[st % KS], st % KS);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+// acc[db] += columns [32 db, 32 db + 32) of tile rows [16 t16, 16 t16 + 16), transposed  x  bfrag[t16]
+template <typename T, int D, int PT, int DB, int GRP>
+FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], const typename Elem<T>::v8* bfrag, int db0 = 0) {
+    typedef typename Elem<T>::v8 v8;
+    constexpr int TOTAL = PT * DB, NG = TOTAL / GRP;
+    static_assert(TOTAL % GRP == 0, "group shape");
+    v8 a[2][GRP];
+#pragma unroll
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_cols_at<T, D>(tile, offc[db0 + j % DB][0], offc[db0 + j % DB][1], j / DB);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        if (g + 1 < NG) {
+#pragma unroll
+            for (int j = 0; j < GRP; j++) {
+                const int st = (g + 1) * GRP + j;
+                a[(g + 1) & 1][j] = lds_cols_at<T, D>(tile, offc[db0 + st % DB][0], offc[db0 + st % DB][1], st / DB);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < GRP; j++) {
+            const int st = g * GRP + j;
+            acc[st % DB] = Elem<T>::mfma32(a[g & 1][j], bfrag[st / DB], acc[st % DB]);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -188,6 +285,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     const float lse2 = row_ok ? p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] * kLog2e : INFINITY;
     const float dsum = row_ok ? p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + row] : 0.f;
 
+    wait_resident_loads();
     f32x16 dq_acc[C::DB];
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
@@ -226,6 +324,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     const float sl2 = kp.scale_log2;
     Drop drop = {0, 0, 256, 1.f};
     if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
+    LdsOffs<D, C::KS, C::DB> lo;
+    lo.init(lane);
     if (t_hi > t_lo) { load_tile(t_lo); store_tile(0, t_lo); }
     __syncthreads();
     int buf = 0;
@@ -239,13 +339,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
                           (r0w >= si.sq);
         if (!skip) {
             f32x16 s_acc[C::NB], dp_acc[C::NB];
-#pragma unroll
-            for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-                for (int dk = 0; dk < C::KS; dk++) {
-                    mfma_step<T>(s_acc[nb], lds_a_rows<T, D>(kb, nb * 32 + l32, dk, hh), qf[dk], dk);
-                    mfma_step<T>(dp_acc[nb], lds_a_rows<T, D>(vb, nb * 32 + l32, dk, hh), gf[dk], dk);
-                }
+            product_rows<T, D, C::NB, C::KS, 4>(s_acc, kb, lo.r, qf);
+            product_rows<T, D, C::NB, C::KS, 4>(dp_acc, vb, lo.r, gf);
             const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0w + shift + wr) ||
                                    (has_left && n0 < r0w + 31 + shift - wl);
             if (need_mask) {
@@ -276,11 +371,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
                 dsf[2 * nb + 1] = pack_acc8<T>(s_acc[nb], 8);
             }
             // dQ^T += K^T dS^T
-#pragma unroll
-            for (int t16 = 0; t16 < C::PT; t16++)
-#pragma unroll
-                for (int db = 0; db < C::DB; db++)
-                    dq_acc[db] = Elem<T>::mfma32(lds_a_cols<T, D>(kb, t16, db, lane), dsf[t16], dq_acc[db]);
+            product_cols<T, D, C::PT, C::DB, 4>(dq_acc, kb, lo.c, dsf);
         }
         if (has_next) store_tile(buf ^ 1, t + 1);
         __syncthreads();
@@ -371,6 +462,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
             vf[dk] = __builtin_bit_cast(v8, c);
         }
     }
+    wait_resident_loads();
 
     f32x16 dk_acc[C::DB], dv_acc[C::DB];
 #pragma unroll
@@ -395,12 +487,12 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
             gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
         }
         if (tid < 2 * BM) {
-            const int r = i0 + (tid < BM ? tid : tid - BM);
-            if (r < si.sq)
-                aux = tid < BM ? p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + r] * kLog2e
-                               : p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + r];
-            else
-                aux = tid < BM ? INFINITY : 0.f;
+            // raw value only: anything computed from it here would make the wave wait for the load
+            // (and, loads completing in order, for the whole tile) before the current tile's products
+            const int r = min(i0 + (tid < BM ? tid : tid - BM), si.sq - 1);
+            const float* src = tid < BM ? p.softmax_lse + ((int64_t)b * p.h + head) * p.seqlen_q
+                                        : p.softmax_d + ((int64_t)b * p.h + head) * p.seqlen_q_rounded;
+            aux = src[r];
         }
     };
     auto store_tile = [&](int buf, int t) {
@@ -417,7 +509,10 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
             *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
             *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
         }
-        if (tid < 2 * BM) reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = aux;
+        if (tid < 2 * BM) {
+            const bool in_range = i0 + (tid < BM ? tid : tid - BM) < si.sq;   // rows past the end: lse = +inf => P = 0
+            reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? aux : 0.f);
+        }
     };
 
     const float sl2 = kp.scale_log2;
@@ -597,6 +692,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
             vf[dk] = __builtin_bit_cast(v8, c);
         }
     }
+    wait_resident_loads();
 
     f32x16 acc[C::DB];      // dV^T of this wave's keys (role V) or dK^T (role K)
 #pragma unroll
@@ -621,12 +717,12 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
             gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
         }
         if (tid < 2 * BM) {
-            const int r = i0 + (tid < BM ? tid : tid - BM);
-            if (r < si.sq)
-                aux = tid < BM ? p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + r] * kLog2e
-                               : p.softmax_d[((int64_t)b * p.h + head) * p.seqlen_q_rounded + r];
-            else
-                aux = tid < BM ? INFINITY : 0.f;
+            // raw value only: anything computed from it here would make the wave wait for the load
+            // (and, loads completing in order, for the whole tile) before the current tile's products
+            const int r = min(i0 + (tid < BM ? tid : tid - BM), si.sq - 1);
+            const float* src = tid < BM ? p.softmax_lse + ((int64_t)b * p.h + head) * p.seqlen_q
+                                        : p.softmax_d + ((int64_t)b * p.h + head) * p.seqlen_q_rounded;
+            aux = src[r];
         }
     };
     auto store_tile = [&](int buf, int t) {
@@ -643,7 +739,10 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
             *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
             *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
         }
-        if (tid < 2 * BM) reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = aux;
+        if (tid < 2 * BM) {
+            const bool in_range = i0 + (tid < BM ? tid : tid - BM) < si.sq;   // rows past the end: lse = +inf => P = 0
+            reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? aux : 0.f);
+        }
     };
 
     const float sl2 = kp.scale_log2;
@@ -757,6 +856,277 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv2_kernel(const BwdKParams kp) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// dK, dV without repeating any product (head dim <= 128).  8 waves; wave w < 4 ("P wave") owns key
+// block w for S = Q K^T, P = exp(S - lse) and dV^T += dO^T P; wave w + 4 ("dS wave") owns the same keys
+// for dP = dO V^T, dS = P o (dP - D) and dK^T += Q^T dS.  P goes from the first to the second through
+// LDS in accumulator layout (both waves map lanes to keys and registers to query rows identically,
+// so the hand-over is lane to same lane, 16 bytes at a time, sign bit = dropped by dropout).
+// The dS wave runs ONE TILE BEHIND: in step t it forms dP of tile t (matrix pipe) and dS, dK of tile
+// t - 1 (P of that tile was published before the barrier that ended step t - 1), so no barrier is
+// added and its exp-free vector work overlaps its own products.  The Q ring therefore has three
+// stages (tile t + 1 arriving, t read by the P wave, t - 1 read transposed by the dS wave); dO has two.
+// ------------------------------------------------------------------------------------------------
+template <typename T, int D, int BM>
+struct BwdDkv3Cfg {
+    static constexpr int kThreads = 512, kWaves = 8, BNW = 128;
+    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int TILE_BYTES = BM * ROWB;
+    static constexpr int LOADS = BM * CPR / kThreads;
+    static constexpr int Q_OFF = 0;                                  // 3 stages
+    static constexpr int G_OFF = 3 * TILE_BYTES;                     // dO: 2 stages
+    static constexpr int AUX_OFF = 5 * TILE_BYTES;                   // 3 stages x {lse (log2 units), D} x BM floats
+    static constexpr int X_OFF = AUX_OFF + 3 * 2 * BM * 4;           // P hand-over: 2 buffers x 4 key blocks
+    static constexpr int XBLK = BM * 32 * 4;                         // one key block's P tile, fp32
+    static constexpr int SMEM = X_OFF + 2 * 4 * XBLK;
+    static_assert(BM % 32 == 0 && D % 32 == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
+    static_assert(SMEM <= 160 * 1024, "LDS budget");
+};
+
+template <typename T, int D, int BM, bool DROPOUT>
+__global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
+    typedef BwdDkv3Cfg<T, D, BM> C;
+    typedef typename Elem<T>::v8 v8;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_bwd_params& p = kp.p;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
+    const bool role_ds = wave >= 4;         // wave-uniform
+    const int kblk = wave & 3;
+
+    const int G = p.h / p.h_k;
+    const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
+    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b;
+    const int per_xcd = gridDim.x >> 3;
+    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (w >= total) return;
+    const int nblk = (int)(w % num_n_blocks); w /= num_n_blocks;
+    const int hk = (int)(w % p.h_k);
+    const int b = (int)(w / p.h_k);
+
+    const BwdSeq si = bwd_seq(p, b);
+    const int n0 = nblk * C::BNW;
+    if (n0 >= si.sk) return;
+    const int shift = si.sk - si.sq;
+    const int wl = p.window_left, wr = p.window_right;
+    const bool has_left = kp.has_left, has_right = kp.has_right;
+    int i_lo = 0, i_hi = si.sq;
+    if (has_right) i_lo = max(0, n0 - shift - wr);
+    if (has_left) i_hi = min(si.sq, min(n0 + C::BNW, si.sk) - shift + wl);
+    const int t_lo = i_lo / BM;
+    const int t_hi = i_hi > i_lo ? (i_hi + BM - 1) / BM : t_lo;
+    const int nt = t_hi - t_lo;
+    const int iters = nt * G;
+
+    // resident operand: this lane's key row of K (P wave) or of V (dS wave)
+    const int j0w = n0 + kblk * 32;
+    const int key = j0w + l32;
+    const bool key_ok = key < si.sk;
+    v8 rf[C::KS];
+    {
+        const T* row = role_ds
+            ? reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)key * p.v_row_stride + (int64_t)hk * p.v_head_stride
+            : reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)key * p.k_row_stride + (int64_t)hk * p.k_head_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 a = {0, 0, 0, 0};
+            if (key_ok && d0 < p.d) a = ld_global16(row + d0);
+            rf[dk] = __builtin_bit_cast(v8, a);
+        }
+    }
+    wait_resident_loads();
+
+    f32x16 acc[C::DB];      // dV^T (P wave) or dK^T (dS wave) of this wave's keys
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+
+    u32x4 qr[C::LOADS], gr[C::LOADS];
+    float aux = 0.f;
+    const int d_last_chunk = p.d / 8 - 1;
+    auto load_tile = [&](int g, int t) {
+        const int head = hk * G + g;
+        const int i0 = t * BM;
+        const T* qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
+        const T* gg = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
+            const int n = min(i0 + r, si.sq - 1);
+            qr[i] = ld_global16(qg + (int64_t)n * p.q_row_stride + c * 8);
+            gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
+        }
+        if (tid < 2 * BM) {
+            // raw value only: anything computed from it here would make the wave wait for the load
+            // (and, loads completing in order, for the whole tile) before the current tile's products
+            const int r = min(i0 + (tid < BM ? tid : tid - BM), si.sq - 1);
+            const float* src = tid < BM ? p.softmax_lse + ((int64_t)b * p.h + head) * p.seqlen_q
+                                        : p.softmax_d + ((int64_t)b * p.h + head) * p.seqlen_q_rounded;
+            aux = src[r];
+        }
+    };
+    auto store_tile = [&](int q3, int g2, int t) {
+        char* qb = smem + C::Q_OFF + q3 * C::TILE_BYTES;
+        char* gb = smem + C::G_OFF + g2 * C::TILE_BYTES;
+        const int i0 = t * BM;
+#pragma unroll
+        for (int i = 0; i < C::LOADS; i++) {
+            const int f = tid + i * C::kThreads;
+            const int r = f / C::CPR, c = f % C::CPR;
+            const bool ok = (i0 + r < si.sq) && (c <= d_last_chunk);
+            const u32x4 z = {0, 0, 0, 0};
+            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
+            *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
+            *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
+        }
+        if (tid < 2 * BM) {
+            const bool in_range = i0 + (tid < BM ? tid : tid - BM) < si.sq;   // rows past the end: lse = +inf => P = 0
+            reinterpret_cast<float*>(smem + C::AUX_OFF + q3 * 2 * BM * 4)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? aux : 0.f);
+        }
+    };
+    auto skip_tile = [&](int i0) {   // keys of this wave against the rows of a tile: nothing visible
+        return (has_right && j0w > i0 + BM - 1 + shift + wr) || (has_left && j0w + 31 < i0 + shift - wl) || (j0w >= si.sk);
+    };
+
+    const float sl2 = kp.scale_log2;
+    const int rel_hi = has_right ? shift + wr : 0x3fffffff;
+    const int rel_lo = has_left ? shift - wl : -0x3fffffff;
+    LdsOffs<D, C::KS, C::DB> lo;
+    lo.init(lane);
+
+    // The tile walk shared by both kinds of wave; `body(it, i0, g, live, prev_live, q3, q3_prev)` is the
+    // wave's own work of one step.  iters + 1 steps: the last one drains the dS wave's final tile.
+    auto walk = [&](auto&& body) {
+        if (iters > 0) { load_tile(0, t_lo); store_tile(0, 0, t_lo); }
+        __syncthreads();
+        int q3 = 0, q3_prev = 0;                     // Q / aux ring slots of the current and the previous tile
+        int cur_t = t_lo, cur_g = 0, nxt_g = 0, nxt_t = t_lo;
+        bool prev_live = false;                      // the previous tile was not skipped (its P is in the hand-over)
+        for (int it = 0; it <= iters; ++it) {
+            const bool has_next = it + 1 < iters;
+            if (has_next) {
+                if (++nxt_t == t_hi) { nxt_t = t_lo; ++nxt_g; }
+                load_tile(nxt_g, nxt_t);
+            }
+            const int i0 = cur_t * BM;
+            const bool live = it < iters && !skip_tile(i0);
+            body(it, i0, cur_g, live, prev_live, q3, q3_prev);
+            prev_live = live;
+            const int q3_next = q3 == 2 ? 0 : q3 + 1;
+            if (has_next) store_tile(q3_next, (it + 1) & 1, nxt_t);
+            __syncthreads();
+            q3_prev = q3;
+            q3 = q3_next;
+            cur_t = nxt_t;
+            cur_g = nxt_g;
+        }
+    };
+
+    if (!role_ds) {
+        walk([&](int it, int i0, int g, bool live, bool, int q3, int) {
+            if (live) {
+            const char* qb = smem + C::Q_OFF + q3 * C::TILE_BYTES;
+            const char* gb = smem + C::G_OFF + (it & 1) * C::TILE_BYTES;
+            const float* lse_s = reinterpret_cast<const float*>(smem + C::AUX_OFF + q3 * 2 * BM * 4);
+            char* xw = smem + C::X_OFF + ((it & 1) * 4 + kblk) * C::XBLK;
+            Drop drop = {0, 0, 256, 1.f};
+            if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, hk * G + g, p.h);
+            f32x16 s_acc[C::MBK];
+            product_rows<T, D, C::MBK, C::KS, 4>(s_acc, qb, lo.r, rf);
+            v8 pf[C::PT];
+#pragma unroll
+            for (int mb = 0; mb < C::MBK; mb++) {
+                const int ib = i0 + mb * 32;
+                const bool need_mask = (has_right && j0w + 31 > ib + shift + wr) || (has_left && j0w < ib + 31 + shift - wl);
+                if (need_mask) {
+                    const int rel = key - ib - 4 * hh;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int c_r = 8 * (r >> 2) + (r & 3);
+                        s_acc[mb][r] = (rel > rel_hi + c_r || rel < rel_lo + c_r) ? -INFINITY : s_acc[mb][r];
+                    }
+                }
+                uint32_t keep = 0xffffu;
+                if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
+                    f32x4 out4;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int r = 4 * q4 + e;
+                        const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
+                        const bool kept = !DROPOUT || ((keep >> r) & 1u);
+                        out4[e] = kept ? pv : -pv;             // sign bit = dropped
+                        s_acc[mb][r] = kept ? pv : 0.f;
+                    }
+                    *reinterpret_cast<f32x4*>(xw + ((mb * 4 + q4) * 64 + lane) * 16) = out4;
+                }
+                pf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
+                pf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
+            }
+            product_cols<T, D, C::PT, C::DB, 4>(acc, gb, lo.c, pf);
+            }
+        });
+    } else {
+        f32x16 dp[C::MBK];      // dP of the tile of the previous step, carried over the loop
+#pragma unroll
+        for (int mb = 0; mb < C::MBK; mb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) dp[mb][r] = 0.f;
+        walk([&](int it, int, int, bool live, bool prev_live, int, int q3_prev) {
+            // first the previous tile (consumes dp), then dP of this tile into the same registers
+            if (prev_live) {
+                const char* qp = smem + C::Q_OFF + q3_prev * C::TILE_BYTES;
+                const float* dsum_s = reinterpret_cast<const float*>(smem + C::AUX_OFF + q3_prev * 2 * BM * 4) + BM;
+                const char* xr = smem + C::X_OFF + (((it - 1) & 1) * 4 + kblk) * C::XBLK;
+                const float rp = DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f;
+                v8 dsf[C::PT];
+#pragma unroll
+                for (int mb = 0; mb < C::MBK; mb++) {
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const f32x4 p4 = *reinterpret_cast<const f32x4*>(xr + ((mb * 4 + q4) * 64 + lane) * 16);
+                        const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int r = 4 * q4 + e;
+                            float dpv = dp[mb][r];
+                            if constexpr (DROPOUT) dpv = __builtin_signbit(p4[e]) ? 0.f : dpv * rp;
+                            dp[mb][r] = fabsf(p4[e]) * (dpv - d4[e]);
+                        }
+                    }
+                    dsf[2 * mb] = pack_acc8<T>(dp[mb], 0);
+                    dsf[2 * mb + 1] = pack_acc8<T>(dp[mb], 8);
+                }
+                product_cols<T, D, C::PT, C::DB, 4>(acc, qp, lo.c, dsf);
+            }
+            if (live) {
+                const char* gb = smem + C::G_OFF + (it & 1) * C::TILE_BYTES;
+                product_rows<T, D, C::MBK, C::KS, 4>(dp, gb, lo.r, rf);
+            }
+        });
+    }
+
+    if (!key_ok) return;
+    T* orow = role_ds ? reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride
+                      : reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
+    const float sc = role_ds ? p.softmax_scale : (DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f);
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const int d0 = db * 32 + 8 * q4 + 4 * hh;
+            if (d0 < p.d) {
+                u32x2 a = {pack2<T>(acc[db][4 * q4] * sc, acc[db][4 * q4 + 1] * sc),
+                           pack2<T>(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc)};
+                st_global8(orow + d0, a);
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
 template <typename K> static int bwd_set_smem(K kern, int bytes) {
@@ -797,6 +1167,19 @@ int launch_bwd_dkv2(const BwdKParams& kp, hipStream_t stream) {
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
     auto kern = bwd_dkv2_kernel<T, D, BM, DROPOUT>;
+    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int D, int BM, bool DROPOUT>
+int launch_bwd_dkv3(const BwdKParams& kp, hipStream_t stream) {
+    typedef BwdDkv3Cfg<T, D, BM> C;
+    const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b;
+    if (total <= 0) return 0;
+    const int64_t per_xcd = (total + 7) / 8;
+    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    auto kern = bwd_dkv3_kernel<T, D, BM, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
