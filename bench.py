@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X FlashAttention forward path (one GPU).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-decode] [--no-backward] [--no-cpu]
 
 One "step" is one forward pass over one synthetic batch already resident in HBM:
   * prefill  -- flash_attn_func, bf16, batch 4, seqlen 8192, 32 heads, head dim 128, causal
@@ -10,6 +10,8 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
   * decode   -- flash_attn_with_kvcache, bf16, batch 64, 1 new token appended with rotary, caches
                 (64, 32768, 8, 128), 64 query heads, cache_seqlens uniform in [1024, 32767];
                 reported as achieved HBM GB/s over the algorithmic bytes.
+  * backward -- gradients of the prefill workload (rowsum(dO o O), dQ pass, dK/dV pass); reported under
+                "backward" at the conventional 2.5 x forward FLOP count.
 Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
 attention_ref) timed on the host cores on a bounded sample of the same workload.
 """
@@ -73,6 +75,29 @@ def bench_prefill(steps, warmup):
     }
 
 
+def bench_backward(steps, warmup):
+    import torch
+    from flash_attn import _native as nat
+    b, s, h, d = 4, 8192, 32, 128
+    torch.manual_seed(0)
+    q, k, v, dout = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16) for _ in range(4))
+    scale = d ** -0.5
+    out, _, _, _, _, lse, _, _ = nat.fwd(q, k, v, None, 0.0, scale, True, -1, -1, False, None)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    fn = lambda: nat.bwd(dout, q, k, v, out, lse, dq, dk, dv, 0.0, scale, True, -1, -1, None, None)
+    ms, wall_ms = time_steps(fn, steps, warmup)
+    flops = 2.5 * 4.0 * b * s * s * h * d / 2      # 5 products of 2 b h s^2 d / 2 (causal)
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {
+        "ms": ms, "wall_ms": wall_ms, "tflops": tflops,
+        "workload": "flash_attn_func bwd bf16 batch=4 seqlen=8192 nheads=32 headdim=128 causal (dot + dQ + dK/dV kernels)",
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "fa::bwd_dkv3_kernel<bf16,128,64> + fa::bwd_dq_kernel<bf16,128,32> (7 tile products executed for 5 counted)",
+                     "flops_per_launch": flops},
+    }
+
+
 def bench_decode(steps, warmup):
     import torch
     import flash_attn
@@ -132,6 +157,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
@@ -168,6 +194,8 @@ def main():
     if not a.no_decode:
         dec = bench_decode(a.steps, a.warmup)
         out["decode"] = dec
+    if not a.no_backward:
+        out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
