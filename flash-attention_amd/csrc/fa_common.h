@@ -227,6 +227,123 @@ FA_DEV void rotary8(float* x, const T* row_ptr, const T* cos_row, const T* sin_r
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Tile products with the A operand in LDS (shared by the general forward kernel and the backward
+// kernels)
+// ------------------------------------------------------------------------------------------------
+constexpr float kLog2e = 1.4426950408889634f;
+
+// s_waitcnt vmcnt(0): placed after the resident operands are loaded, before the tile loop.  Without it
+// the compiler cannot prove inside the loop that those loads have landed (a zero-trip path skips the
+// first tile's wait) and guards the first product of every step with vmcnt(0), which also waits for
+// the NEXT tile's prefetch, i.e. it serialises the prefetch with the products.
+FA_DEV void wait_resident_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// accumulate step dk of a product; step 0 starts from an inline zero instead of a cleared accumulator
+template <typename T> FA_DEV void mfma_step(f32x16& acc, typename Elem<T>::v8 a, typename Elem<T>::v8 b, int dk) {
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    acc = Elem<T>::mfma32(a, b, dk == 0 ? zero : acc);
+}
+
+// accumulator registers [r8, r8+8) -> B operand of the next product
+template <typename T> FA_DEV typename Elem<T>::v8 pack_acc8(const f32x16& a, int r8) {
+    u32x4 pk;
+#pragma unroll
+    for (int e = 0; e < 4; e++) pk[e] = pack2<T>(a[r8 + 2 * e], a[r8 + 2 * e + 1]);
+    return __builtin_bit_cast(typename Elem<T>::v8, pk);
+}
+
+// Per-lane LDS offsets of both read patterns, computed once: the swizzle only involves row & 15, so a
+// block of 32 rows (row-wise) or 16 rows (transposed) further down is a compile-time byte offset.
+template <int D, int KS, int DB>
+struct LdsOffs {
+    int r[KS];       // row-wise: row l32, k-step dk
+    int c[DB][2];    // transposed: column block db, rows 4hh + tj and 8 more
+    FA_DEV void init(int lane) {
+        const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+        for (int dk = 0; dk < KS; dk++) r[dk] = l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16;
+        const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
+        const int row = 4 * hh + tj;
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+            const int cc = db * 4 + dhalf * 2 + (tq >> 1);
+            c[db][0] = row * (D * 2) + swz_u<D>(cc, row) * 16 + (tq & 1) * 8;
+            c[db][1] = (row + 8) * (D * 2) + swz_u<D>(cc, row + 8) * 16 + (tq & 1) * 8;
+        }
+    }
+};
+template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_rows_at(const char* tile, int off, int blk32) {
+    const u32x4 raw = *reinterpret_cast<const u32x4*>(tile + off + blk32 * 32 * (D * 2));
+    return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_cols_at(const char* tile, int off_lo, int off_hi, int t16) {
+    const u32x2 lo = lds_read_tr16(tile + off_lo + t16 * 16 * (D * 2));
+    const u32x2 hi = lds_read_tr16(tile + off_hi + t16 * 16 * (D * 2));
+    const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+
+// Tile products whose A operands come from LDS, software-pipelined by hand: the operands of GRP MFMAs
+// are read one group ahead into a second register set, and a scheduling fence keeps every group's
+// reads in front of the previous group's MFMAs.  (Left to itself the compiler issues read, wait,
+// MFMA, read, wait, MFMA ... with one operand register set, and every MFMA pays an LDS round trip.)
+//
+// acc[blk] (+)= rows [32 blk, 32 blk + 32) of `tile`  x  bfrag[dk]   for blk < NBLK, dk < KS
+template <typename T, int D, int NBLK, int KS, int GRP>
+FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const typename Elem<T>::v8* bfrag) {
+    typedef typename Elem<T>::v8 v8;
+    constexpr int TOTAL = NBLK * KS, NG = TOTAL / GRP;
+    static_assert(TOTAL % GRP == 0 && KS % GRP == 0, "group shape");
+    v8 a[2][GRP];
+#pragma unroll
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_rows_at<T, D>(tile, offr[j % KS], j / KS);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        if (g + 1 < NG) {
+#pragma unroll
+            for (int j = 0; j < GRP; j++) {
+                const int st = (g + 1) * GRP + j;
+                a[(g + 1) & 1][j] = lds_rows_at<T, D>(tile, offr[st % KS], st / KS);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < GRP; j++) {
+            const int st = g * GRP + j;
+            mfma_step<T>(acc[st / KS], a[g & 1][j], bfrag[st % KS], st % KS);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+// acc[db] += columns [32 db, 32 db + 32) of tile rows [16 t16, 16 t16 + 16), transposed  x  bfrag[t16]
+template <typename T, int D, int PT, int DB, int GRP>
+FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], const typename Elem<T>::v8* bfrag, int db0 = 0) {
+    typedef typename Elem<T>::v8 v8;
+    constexpr int TOTAL = PT * DB, NG = TOTAL / GRP;
+    static_assert(TOTAL % GRP == 0, "group shape");
+    v8 a[2][GRP];
+#pragma unroll
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_cols_at<T, D>(tile, offc[db0 + j % DB][0], offc[db0 + j % DB][1], j / DB);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        if (g + 1 < NG) {
+#pragma unroll
+            for (int j = 0; j < GRP; j++) {
+                const int st = (g + 1) * GRP + j;
+                a[(g + 1) & 1][j] = lds_cols_at<T, D>(tile, offc[db0 + st % DB][0], offc[db0 + st % DB][1], st / DB);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < GRP; j++) {
+            const int st = g * GRP + j;
+            acc[st % DB] = Elem<T>::mfma32(a[g & 1][j], bfrag[st / DB], acc[st % DB]);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // Resolved per-(batch) sequence bookkeeping.  Mirrors the reference's BlockInfo
 // (csrc/flash_attn/src/block_info.h:11-42) with 64-bit offsets.
 struct SeqInfo {

@@ -11,9 +11,10 @@
 //    B-operand layout of the second product O^T = V^T P^T -- P never leaves registers.
 //  * O^T accumulators likewise hold one query row per lane: the online-softmax rescale is a
 //    per-lane scalar multiply, no broadcast.
-//  * K and V tiles are double-buffered in LDS with 16-byte-chunk XOR swizzles chosen so that the
+//  * K and V tiles are double-buffered in LDS with a 16-byte-chunk XOR swizzle under which both the
 //    K fragment reads (ds_read_b128) and the transposing V reads (ds_read_b64_tr_b16) are
-//    bank-conflict free; global loads are 128-bit, issued one tile ahead.
+//    bank-conflict free; global loads are 128-bit, issued one tile ahead; LDS operands are read one
+//    group of MFMAs ahead (product_rows / product_cols in fa_common.h).
 //  * Key tiles that a wave's rows cannot see (causal / sliding window) are skipped per wave.
 #pragma once
 #include "fa_common.h"
@@ -35,6 +36,7 @@ struct PrefillCfg {
     static constexpr int LOADS = BN * CPR / kThreads;  // 16 B loads per thread, per tensor, per tile
     static constexpr int SMEM = 4 * TILE_BYTES;   // {K,V} x 2 stages
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
+    static_assert(RB == 1, "one 32-row block per wave");
 };
 
 template <typename T, int D, int RB, int BN, int MINW, bool SPLIT, bool DROPOUT = false>
@@ -45,7 +47,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     const fa_fwd_params& p = kp.p;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int l32 = lane & 31, hh = lane >> 5;
 
     // ---- work decode: contiguous ranges of the logical order go to one XCD (block ids are
@@ -113,6 +115,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
         }
     }
 
+    wait_resident_loads();
     f32x16 o_acc[RB][C::DB];
     float m_run[RB], l_run[RB];
 #pragma unroll
@@ -151,14 +154,14 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
             const int row = f / C::CPR, c = f % C::CPR;
             const bool ok = (n0 + row < si.sk) && (c <= d_last_chunk);
             const u32x4 z = {0, 0, 0, 0};
-            *reinterpret_cast<u32x4*>(kb + row * C::ROWB + swz_k<D>(c, row) * 16) = ok ? kr[i] : z;
-            *reinterpret_cast<u32x4*>(vb + row * C::ROWB + swz_v<D>(c, row) * 16) = ok ? vr[i] : z;
+            const int off = row * C::ROWB + swz_u<D>(c, row) * 16;
+            *reinterpret_cast<u32x4*>(kb + off) = ok ? kr[i] : z;
+            *reinterpret_cast<u32x4*>(vb + off) = ok ? vr[i] : z;
         }
     };
 
-    // per-lane pieces of the transposing V read: within a 16-lane block lane 4*j+q addresses row j,
-    // columns 4q..4q+3 of a 4-key x 16-dim tile.
-    const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
+    LdsOffs<D, C::KS, C::DB> lo;
+    lo.init(lane);
 
     const float sl2 = kp.scale_log2;
     Drop drop = {0, 0, 256, 1.f};
@@ -191,25 +194,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
         if (any_work) {
             // ---- S^T = K Q^T
             f32x16 s_acc[RB][C::NB];
-#pragma unroll
-            for (int rb = 0; rb < RB; rb++)
-#pragma unroll
-                for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) s_acc[rb][nb][r] = 0.f;
-#pragma unroll
-            for (int nb = 0; nb < C::NB; nb++) {
-                const int krow = nb * 32 + l32;
-#pragma unroll
-                for (int dk = 0; dk < C::KS; dk++) {
-                    const int c = dk * 2 + hh;
-                    const u32x4 raw = *reinterpret_cast<const u32x4*>(kb + krow * C::ROWB + swz_k<D>(c, krow) * 16);
-                    const v8 a = __builtin_bit_cast(v8, raw);
-#pragma unroll
-                    for (int rb = 0; rb < RB; rb++)
-                        if (!skip[rb]) s_acc[rb][nb] = Elem<T>::mfma32(a, qf[rb][dk], s_acc[rb][nb]);
-                }
-            }
+            product_rows<T, D, C::NB, C::KS, 4>(s_acc[0], kb, lo.r, qf[0]);
 
             // ---- mask, online softmax, pack P
             v8 pf[RB][C::PT];
@@ -282,22 +267,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
             }
 
             // ---- O^T += V^T P^T
-#pragma unroll
-            for (int t16 = 0; t16 < C::PT; t16++) {
-                const int vrow = t16 * 16 + 4 * hh + tj;   // second read: +8 rows (same row & 3)
-#pragma unroll
-                for (int db = 0; db < C::DB; db++) {
-                    const int c = db * 4 + dhalf * 2 + (tq >> 1);
-                    const int off = swz_v<D>(c, vrow) * 16 + (tq & 1) * 8;
-                    const u32x2 lo = lds_read_tr16(vb + vrow * C::ROWB + off);
-                    const u32x2 hi = lds_read_tr16(vb + (vrow + 8) * C::ROWB + off);
-                    u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
-                    const v8 a = __builtin_bit_cast(v8, raw);
-#pragma unroll
-                    for (int rb = 0; rb < RB; rb++)
-                        if (!skip[rb]) o_acc[rb][db] = Elem<T>::mfma32(a, pf[rb][t16], o_acc[rb][db]);
-                }
-            }
+            product_cols<T, D, C::PT, C::DB, 4>(o_acc[0], vb, lo.c, pf[0]);
         }
 
         if (has_next) store_tile(buf ^ 1, t - 1);
