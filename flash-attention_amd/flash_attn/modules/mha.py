@@ -1,20 +1,74 @@
 """Self-attention layer with a KV cache: the caller of `flash_attn_with_kvcache` during generation.
 
-Covers the decoding glue of the reference's flash_attn/modules/mha.py: `_update_kv_cache` (:296-322),
+Covers the flash-attention wrappers `FlashSelfAttention` (:36-94) and `FlashCrossAttention` (:97-174)
+and the decoding glue of the reference's flash_attn/modules/mha.py: `_update_kv_cache` (:296-322),
 `MHA.allocate_inference_cache` (:422-434), `MHA._apply_rotary_update_kvcache_attention` (:442-479),
 `MHA._update_kvcache_attention` (:481-507) and the self-attention branches of `MHA.forward`
-(:515-653): packed QKV projection, rotary, MHA / GQA / MQA, causal mask.  Not carried over (the
-reference's options outside the attention path): cross-attention, depthwise convolution, dropout,
-ALiBi, fused dense layers, the non-flash attention fallbacks, activation checkpointing and the
-tensor-parallel variant.
+(:515-653): packed QKV projection, rotary, MHA / GQA / MQA, causal mask, attention dropout, packed
+variable-length input.  Not carried over (the reference's options outside the attention path):
+the cross-attention projections, depthwise convolution, fused dense layers, the non-flash attention
+fallbacks, activation checkpointing and the tensor-parallel variant.
 """
 import math
 
 import torch
 import torch.nn as nn
 
-from flash_attn import flash_attn_kvpacked_func, flash_attn_qkvpacked_func, flash_attn_with_kvcache
+from flash_attn import (flash_attn_kvpacked_func, flash_attn_qkvpacked_func, flash_attn_varlen_kvpacked_func,
+                        flash_attn_varlen_qkvpacked_func, flash_attn_with_kvcache)
 from flash_attn.layers.rotary import RotaryEmbedding
+
+
+class FlashSelfAttention(nn.Module):
+    """Softmax attention over a packed qkv tensor.  qkv (B, S, 3, H, D), or (total, 3, H, D) with
+    cu_seqlens (int32, batch + 1) and max_seqlen; dropout applies in training mode only."""
+
+    def __init__(self, causal=False, softmax_scale=None, attention_dropout=0.0, window_size=(-1, -1)):
+        super().__init__()
+        self.causal = causal
+        self.softmax_scale = softmax_scale
+        self.window_size = window_size
+        self.drop = nn.Dropout(attention_dropout)
+
+    def forward(self, qkv, causal=None, cu_seqlens=None, max_seqlen=None):
+        assert qkv.dtype in [torch.float16, torch.bfloat16]
+        assert qkv.is_cuda
+        causal = self.causal if causal is None else causal
+        p = self.drop.p if self.training else 0.0
+        if cu_seqlens is not None:
+            assert cu_seqlens.dtype == torch.int32
+            assert isinstance(max_seqlen, int)
+            return flash_attn_varlen_qkvpacked_func(qkv, cu_seqlens, max_seqlen, p, softmax_scale=self.softmax_scale,
+                                                    causal=causal, window_size=self.window_size)
+        return flash_attn_qkvpacked_func(qkv, p, softmax_scale=self.softmax_scale, causal=causal,
+                                         window_size=self.window_size)
+
+
+class FlashCrossAttention(nn.Module):
+    """Softmax attention of q (B, Sq, H, D) over kv (B, Sk, 2, H_k, D), or the packed forms
+    (total_q, H, D) / (total_k, 2, H_k, D) with cu_seqlens / max_seqlen for q and for k."""
+
+    def __init__(self, causal=False, softmax_scale=None, attention_dropout=0.0, window_size=(-1, -1)):
+        super().__init__()
+        self.causal = causal
+        self.softmax_scale = softmax_scale
+        self.window_size = window_size
+        self.drop = nn.Dropout(attention_dropout)
+
+    def forward(self, q, kv, causal=None, cu_seqlens=None, max_seqlen=None, cu_seqlens_k=None, max_seqlen_k=None):
+        assert q.dtype in [torch.float16, torch.bfloat16]
+        assert q.is_cuda and kv.is_cuda
+        causal = self.causal if causal is None else causal
+        p = self.drop.p if self.training else 0.0
+        if cu_seqlens is not None:
+            assert cu_seqlens.dtype == torch.int32 and isinstance(max_seqlen, int)
+            assert cu_seqlens_k is not None and cu_seqlens_k.dtype == torch.int32 and isinstance(max_seqlen_k, int)
+            return flash_attn_varlen_kvpacked_func(q, kv, cu_seqlens, cu_seqlens_k, max_seqlen, max_seqlen_k, p,
+                                                   softmax_scale=self.softmax_scale, causal=causal,
+                                                   window_size=self.window_size)
+        assert kv.shape[0] == q.shape[0] and kv.shape[4] == q.shape[3]
+        return flash_attn_kvpacked_func(q, kv, p, softmax_scale=self.softmax_scale, causal=causal,
+                                        window_size=self.window_size)
 
 
 def _update_kv_cache(kv, inference_params, layer_idx):
@@ -40,7 +94,7 @@ class MHA(nn.Module):
     """Multi-head self-attention on the flash attention kernels, with the reference's constructor
     arguments for the options that are supported."""
 
-    def __init__(self, embed_dim, num_heads, num_heads_kv=None, qkv_proj_bias=True, out_proj_bias=True,
+    def __init__(self, embed_dim, num_heads, num_heads_kv=None, qkv_proj_bias=True, out_proj_bias=True, dropout=0.0,
                  softmax_scale=None, causal=False, layer_idx=None, rotary_emb_dim=0, rotary_emb_base=10000.0,
                  rotary_emb_scale_base=None, rotary_emb_interleaved=False, window_size=(-1, -1), device=None,
                  dtype=None):
@@ -62,6 +116,10 @@ class MHA(nn.Module):
         if self.rotary_emb_dim > 0:
             self.rotary_emb = RotaryEmbedding(self.rotary_emb_dim, base=rotary_emb_base, scale_base=rotary_emb_scale_base,
                                               interleaved=rotary_emb_interleaved, device=device)
+        self.inner_attn = FlashSelfAttention(causal=causal, softmax_scale=softmax_scale, attention_dropout=dropout,
+                                             window_size=window_size)
+        self.inner_cross_attn = FlashCrossAttention(causal=causal, softmax_scale=softmax_scale,
+                                                    attention_dropout=dropout, window_size=window_size)
         self.Wqkv = nn.Linear(embed_dim, qkv_dim, bias=qkv_proj_bias, **factory_kwargs)
         self.out_proj = nn.Linear(embed_dim, embed_dim, bias=out_proj_bias, **factory_kwargs)
 
@@ -69,6 +127,24 @@ class MHA(nn.Module):
         dtype = self.out_proj.weight.dtype if dtype is None else dtype
         return torch.empty(batch_size, max_seqlen, 2, self.num_heads_kv, self.head_dim, dtype=dtype,
                            device=self.out_proj.weight.device)
+
+    def _rotate_packed(self, q, k_part, nk, cu_seqlens, max_seqlen, ret):
+        """Rotary on packed (total, ...) q and k: every sequence starts at position 0."""
+        from flash_attn.layers.rotary import apply_rotary_emb
+        assert self.rotary_emb.scale is None, "packed input does not support xPos"
+        self.rotary_emb._update_cos_sin_cache(max_seqlen, device=q.device, dtype=q.dtype)
+        cos, sin = self.rotary_emb._cos_cached, self.rotary_emb._sin_cached
+        total = q.shape[0]
+        if ret is not None:      # qkv packed: q and k heads are one run of 2h heads per token
+            qk = ret.view(total, 3 * self.num_heads, self.head_dim)[:, : 2 * self.num_heads]
+            apply_rotary_emb(qk, cos, sin, interleaved=self.rotary_emb.interleaved, inplace=True, cu_seqlens=cu_seqlens,
+                             max_seqlen=max_seqlen)
+            return ret
+        apply_rotary_emb(q, cos, sin, interleaved=self.rotary_emb.interleaved, inplace=True, cu_seqlens=cu_seqlens,
+                         max_seqlen=max_seqlen)
+        apply_rotary_emb(k_part[:, 0], cos, sin, interleaved=self.rotary_emb.interleaved, inplace=True,
+                         cu_seqlens=cu_seqlens, max_seqlen=max_seqlen)
+        return None
 
     def _update_kv_cache(self, kv, inference_params):
         assert self.layer_idx is not None, "Generation requires layer_idx in the constructor"
@@ -101,15 +177,33 @@ class MHA(nn.Module):
         cache and attends within the prompt; later steps append and attend to the cache."""
         if inference_params.seqlen_offset == 0:
             kv = self._update_kv_cache(kv, inference_params)
-            return flash_attn_kvpacked_func(q, kv, softmax_scale=self.softmax_scale, causal=self.causal,
-                                            window_size=self.window_size)
+            return self.inner_cross_attn(q, kv)
         kv_cache, cache_seqlens = self._cache_and_lengths(q.shape[0], inference_params)
         return flash_attn_with_kvcache(q, kv_cache[:, :, 0], kv_cache[:, :, 1], kv[:, :, 0], kv[:, :, 1],
                                        cache_seqlens=cache_seqlens, softmax_scale=self.softmax_scale, causal=self.causal,
                                        window_size=self.window_size)
 
-    def forward(self, x, inference_params=None):
-        """x (batch, seqlen, embed_dim) -> (batch, seqlen, embed_dim)."""
+    def forward(self, x, cu_seqlens=None, max_seqlen=None, inference_params=None):
+        """x (batch, seqlen, embed_dim) -> (batch, seqlen, embed_dim); or packed (total, embed_dim) with
+        cu_seqlens / max_seqlen (not together with inference_params)."""
+        if cu_seqlens is not None:
+            assert max_seqlen is not None and inference_params is None and x.dim() == 2
+            total = x.shape[0]
+            qkv = self.Wqkv(x)
+            kw = dict(cu_seqlens=cu_seqlens, max_seqlen=max_seqlen)
+            if self.num_heads_kv == self.num_heads:
+                qkv = qkv.view(total, 3, self.num_heads, self.head_dim)
+                if self.rotary_emb_dim > 0:
+                    qkv = self._rotate_packed(qkv[:, 0], qkv[:, :2], 2, cu_seqlens, max_seqlen, qkv)
+                context = self.inner_attn(qkv, **kw)
+            else:
+                nq = self.num_heads * self.head_dim
+                q = qkv[..., :nq].reshape(total, self.num_heads, self.head_dim)
+                kv = qkv[..., nq:].reshape(total, 2, self.num_heads_kv, self.head_dim)
+                if self.rotary_emb_dim > 0:
+                    self._rotate_packed(q, kv[:, :1], 1, cu_seqlens, max_seqlen, None)
+                context = self.inner_cross_attn(q, kv, cu_seqlens_k=cu_seqlens, max_seqlen_k=max_seqlen, **kw)
+            return self.out_proj(context.reshape(total, self.embed_dim))
         if inference_params is None:
             seqlen_offset, rotary_max_seqlen = 0, None
         else:
@@ -129,8 +223,7 @@ class MHA(nn.Module):
                 if self.rotary_emb_dim > 0:
                     qkv = self.rotary_emb(qkv, seqlen_offset=seqlen_offset, max_seqlen=rotary_max_seqlen)
                 if inference_params is None:
-                    context = flash_attn_qkvpacked_func(qkv, softmax_scale=self.softmax_scale, causal=self.causal,
-                                                        window_size=self.window_size)
+                    context = self.inner_attn(qkv)
                 else:
                     context = self._update_kvcache_attention(qkv[:, :, 0], qkv[:, :, 1:], inference_params)
         else:
@@ -143,8 +236,7 @@ class MHA(nn.Module):
                 if self.rotary_emb_dim > 0:
                     q, kv = self.rotary_emb(q, kv, seqlen_offset=seqlen_offset, max_seqlen=rotary_max_seqlen)
                 if inference_params is None:
-                    context = flash_attn_kvpacked_func(q, kv, softmax_scale=self.softmax_scale, causal=self.causal,
-                                                       window_size=self.window_size)
+                    context = self.inner_cross_attn(q, kv)
                 else:
                     context = self._update_kvcache_attention(q, kv, inference_params)
         return self.out_proj(context.reshape(batch, seqlen, self.embed_dim))

@@ -145,3 +145,73 @@ def test_sampling_helpers():
     torch.manual_seed(0)
     picks = torch.stack([sample(logits, top_k=2, top_p=0.0, temperature=0.7) for _ in range(50)])
     assert set(picks[:, 0].tolist()) <= {2, 3} and set(picks[:, 1].tolist()) <= {0, 1}
+
+
+@pytest.mark.parametrize("heads_kv", [4, 2])
+@pytest.mark.parametrize("rotary_dim", [0, 32])
+def test_mha_packed_varlen_equals_per_sequence(heads_kv, rotary_dim):
+    """Packed (total, dim) input with cu_seqlens: every sequence must come out as if it went through the
+    layer alone (rotary positions restart at 0 for each sequence)."""
+    from flash_attn.modules.mha import MHA
+    _say("mha varlen", heads_kv, rotary_dim)
+    torch.manual_seed(5)
+    dtype, dim, h = torch.bfloat16, 256, 4
+    layer = MHA(dim, h, num_heads_kv=heads_kv, causal=True, layer_idx=0, rotary_emb_dim=rotary_dim, device=DEV, dtype=dtype).eval()
+    lens = [70, 1, 200, 33]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    x = torch.randn(sum(lens), dim, device=DEV, dtype=dtype)
+    with torch.no_grad():
+        packed = layer(x, cu_seqlens=cu, max_seqlen=max(lens))
+        for i, L in enumerate(lens):
+            a, e = int(cu[i]), int(cu[i + 1])
+            alone = layer(x[a:e][None])[0]
+            err = (packed[a:e].float() - alone.float()).abs().max().item()
+            assert err < 2e-2, (i, err)
+
+
+def test_flash_attention_wrappers_train_and_eval():
+    """FlashSelfAttention / FlashCrossAttention: dropout only in training mode, gradients flow, the
+    eval output equals the functional call."""
+    import flash_attn
+    from flash_attn.modules.mha import FlashCrossAttention, FlashSelfAttention
+    _say("wrappers")
+    torch.manual_seed(6)
+    qkv = torch.randn(2, 130, 3, 4, 64, device=DEV, dtype=torch.float16, requires_grad=True)
+    sa = FlashSelfAttention(causal=True, attention_dropout=0.3)
+    sa.eval()
+    assert torch.equal(sa(qkv), flash_attn.flash_attn_qkvpacked_func(qkv, causal=True))
+    sa.train()
+    torch.cuda.manual_seed(1)
+    out_a = sa(qkv)
+    torch.cuda.manual_seed(1)
+    out_b = sa(qkv)
+    assert torch.equal(out_a, out_b) and not torch.equal(out_a, sa.eval()(qkv))
+    out_a.float().sum().backward()
+    assert qkv.grad is not None and torch.isfinite(qkv.grad).all()
+    q = torch.randn(2, 50, 4, 64, device=DEV, dtype=torch.float16)
+    kv = torch.randn(2, 90, 2, 2, 64, device=DEV, dtype=torch.float16)
+    ca = FlashCrossAttention().eval()
+    assert torch.equal(ca(q, kv), flash_attn.flash_attn_kvpacked_func(q, kv))
+    cu_q = torch.tensor([0, 50, 100], dtype=torch.int32, device=DEV)
+    cu_k = torch.tensor([0, 90, 180], dtype=torch.int32, device=DEV)
+    packed = ca(q.reshape(100, 4, 64), kv.reshape(180, 2, 2, 64), cu_seqlens=cu_q, max_seqlen=50, cu_seqlens_k=cu_k,
+                max_seqlen_k=90)
+    assert (packed.reshape(2, 50, 4, 64).float() - ca(q, kv).float()).abs().max().item() < 2e-3
+
+
+def test_mha_trains_with_dropout():
+    """Forward + backward through the layer in training mode (attention dropout on): finite gradients for
+    every parameter, and the same seed reproduces them."""
+    from flash_attn.modules.mha import MHA
+    _say("mha train")
+    torch.manual_seed(7)
+    layer = MHA(256, 4, num_heads_kv=2, dropout=0.1, causal=True, rotary_emb_dim=32, device=DEV, dtype=torch.bfloat16).train()
+    x = torch.randn(2, 300, 256, device=DEV, dtype=torch.bfloat16)
+    grads = []
+    for _ in range(2):
+        layer.zero_grad()
+        torch.cuda.manual_seed(11)
+        layer(x).float().square().mean().backward()
+        grads.append([p.grad.clone() for p in layer.parameters()])
+    for a, b in zip(*grads):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
