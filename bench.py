@@ -10,6 +10,8 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
   * decode   -- flash_attn_with_kvcache, bf16, batch 64, 1 new token appended with rotary, caches
                 (64, 32768, 8, 128), 64 query heads, cache_seqlens uniform in [1024, 32767];
                 reported as achieved HBM GB/s over the algorithmic bytes.
+  * rotary   -- apply_rotary_emb in place on (8, 8192, 32, 128) bf16 (the standalone rotary kernel), GB/s
+                over 2 x the tensor's bytes;
   * backward -- gradients of the prefill workload (rowsum(dO o O), dQ pass, dK/dV pass); reported under
                 "backward" at the conventional 2.5 x forward FLOP count.
 Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
@@ -72,6 +74,26 @@ def bench_prefill(steps, warmup):
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"),
                      "kernel": "fa::prefill_pp_kernel<bf16,128,64>", "flops_per_launch": flops},
+    }
+
+
+def bench_rotary(steps, warmup):
+    import torch
+    from flash_attn.layers.rotary import apply_rotary
+    b, s, h, d = 8, 8192, 32, 128
+    torch.manual_seed(0)
+    x = torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16)
+    ang = torch.rand(s, d // 2, device="cuda") * 6.28
+    cos, sin = torch.cos(ang).to(torch.bfloat16), torch.sin(ang).to(torch.bfloat16)
+    fn = lambda: apply_rotary(x, cos, sin, inplace=True)
+    ms, wall_ms = time_steps(fn, steps, warmup)
+    algo_bytes = 2 * x.numel() * x.element_size()
+    gbs = algo_bytes / (ms * 1e-3) / 1e9
+    return {
+        "ms": ms, "wall_ms": wall_ms, "gb_per_s": gbs,
+        "workload": "apply_rotary_emb bf16 (8, 8192, 32, 128) rotary_dim 128 in place",
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                     "traffic": None, "kernel": "fa::rotary_kernel<bf16,bf16,u32>", "bytes_per_launch": algo_bytes},
     }
 
 
@@ -195,6 +217,7 @@ def main():
         dec = bench_decode(a.steps, a.warmup)
         out["decode"] = dec
     if not a.no_backward:
+        out["rotary"] = bench_rotary(a.steps, a.warmup)
         out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
