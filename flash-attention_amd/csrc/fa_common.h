@@ -294,24 +294,25 @@ template <typename T, int D, int NBLK, int KS, int GRP>
 FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const typename Elem<T>::v8* bfrag) {
     typedef typename Elem<T>::v8 v8;
     constexpr int TOTAL = NBLK * KS, NG = TOTAL / GRP;
-    static_assert(TOTAL % GRP == 0 && KS % GRP == 0, "group shape");
+    static_assert(TOTAL % GRP == 0, "group shape");
+    // step st -> (k-step st / NBLK, row block st % NBLK): consecutive MFMAs go to different accumulators
     v8 a[2][GRP];
 #pragma unroll
-    for (int j = 0; j < GRP; j++) a[0][j] = lds_rows_at<T, D>(tile, offr[j % KS], j / KS);
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_rows_at<T, D>(tile, offr[j / NBLK], j % NBLK);
 #pragma unroll
     for (int g = 0; g < NG; g++) {
         if (g + 1 < NG) {
 #pragma unroll
             for (int j = 0; j < GRP; j++) {
                 const int st = (g + 1) * GRP + j;
-                a[(g + 1) & 1][j] = lds_rows_at<T, D>(tile, offr[st % KS], st / KS);
+                a[(g + 1) & 1][j] = lds_rows_at<T, D>(tile, offr[st / NBLK], st % NBLK);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < GRP; j++) {
             const int st = g * GRP + j;
-            mfma_step<T>(acc[st / KS], a[g & 1][j], bfrag[st % KS], st % KS);
+            mfma_step<T>(acc[st % NBLK], a[g & 1][j], bfrag[st / NBLK], st / NBLK);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
