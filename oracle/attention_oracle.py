@@ -25,8 +25,10 @@ It restates, in plain PyTorch on the CPU, the semantics that the reference pins 
 How each function is pinned (none is "parity unpinned"): see tests/test_oracle.py -- library
 routine `scaled_dot_product_attention`, brute-force scalar loops on tiny shapes, the docstring
 mask matrices (`flash_attn/flash_attn_interface.py:611-621`), closed forms (uniform attention
-for zero scores, rotation norm preservation / composition), and the heuristic's own worked
-example (`flash_api.cpp:206-211`).
+for zero scores, rotation norm preservation / composition), the heuristic's own worked
+example (`flash_api.cpp:206-211`), and for the gradients and dropout: central differences of a
+scalar-loop forward in fp64, torch autograd through the forward restatement, one-key and equal-value
+closed forms, an all-kept mask (output scales by 1 / (1 - p), log-sum-exp unchanged).
 
 The score tensor of the reference form is (b, h, sq, sk) fp32, tens of GB at benchmark sizes, so
 every routine here walks (batch, head-block) chunks, which are independent.
