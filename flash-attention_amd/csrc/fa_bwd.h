@@ -6,8 +6,7 @@
 //   D_i   = sum_d dO[i,d] O[i,d]                                   (bwd_dot_kernel)
 //   P     = exp(scale * Q K^T - lse),   dP = dO V^T,   dS = P o (dP - D)
 //   dQ    = scale * dS K                                           (bwd_dq_kernel: per query tile)
-//   dV    = P^T dO,   dK = scale * dS^T Q                          (per key tile: bwd_dkv3_kernel for
-//                                                                    head dim <= 128, bwd_dkv_kernel above)
+//   dV    = P^T dO,   dK = scale * dS^T Q                          (bwd_dkv3_kernel: per key tile)
 //
 // Both kernels keep the forward kernels' register geometry: every product is computed TRANSPOSED with
 // v_mfma_f32_32x32x16 so that the accumulator gives each lane ONE row of the resident operand (a
@@ -266,226 +265,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 }
 
 // ------------------------------------------------------------------------------------------------
-// dK, dV: a workgroup owns 128 keys of one (batch, kv head) and streams the Q / dO tiles (BM query
-// rows) of every query head of the group.  With DPARTS = 2 a workgroup accumulates only half of the
-// head dimension (the scores are computed in full by both halves): head dim 256 would otherwise
-// need more than 512 registers per lane.
-// ------------------------------------------------------------------------------------------------
-template <typename T, int D, int BM, int DPARTS>
-struct BwdDkvCfg {
-    static constexpr int kThreads = 256, kWaves = 4, BNW = 128;
-    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32 / DPARTS, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
-    static constexpr int TILE_BYTES = BM * ROWB;
-    static constexpr int LOADS = BM * CPR / kThreads;
-    static constexpr int STAGE = 2 * TILE_BYTES + 2 * BM * 4;   // Q, dO, lse (log2 units), D
-    static constexpr int SMEM = 2 * STAGE;
-    static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
-};
-
-template <typename T, int D, int BM, int DPARTS, int MINW, bool DROPOUT>
-__global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp) {
-    typedef BwdDkvCfg<T, D, BM, DPARTS> C;
-    typedef typename Elem<T>::v8 v8;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    const fa_bwd_params& p = kp.p;
-    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
-
-    const int G = p.h / p.h_k;
-    const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
-    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b * DPARTS;
-    const int per_xcd = gridDim.x >> 3;
-    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (w >= total) return;
-    const int dpart = (int)(w % DPARTS); w /= DPARTS;
-    const int nblk = (int)(w % num_n_blocks); w /= num_n_blocks;
-    const int hk = (int)(w % p.h_k);
-    const int b = (int)(w / p.h_k);
-
-    const BwdSeq si = bwd_seq(p, b);
-    const int n0 = nblk * C::BNW;
-    if (n0 >= si.sk) return;
-    const int shift = si.sk - si.sq;
-    const int wl = p.window_left, wr = p.window_right;
-    const bool has_left = kp.has_left, has_right = kp.has_right;
-    // query rows that see at least one of this workgroup's keys
-    int i_lo = 0, i_hi = si.sq;
-    if (has_right) i_lo = max(0, n0 - shift - wr);
-    if (has_left) i_hi = min(si.sq, min(n0 + C::BNW, si.sk) - shift + wl);
-    const int t_lo = i_lo / BM;
-    const int t_hi = i_hi > i_lo ? (i_hi + BM - 1) / BM : t_lo;
-    const int nt = t_hi - t_lo;
-    const int iters = nt * G;
-
-    // resident operands: this lane's key row of K and V
-    const int j0w = n0 + wave * 32;
-    const int key = j0w + l32;
-    const bool key_ok = key < si.sk;
-    v8 kf[C::KS], vf[C::KS];
-    {
-        const T* krow = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)key * p.k_row_stride + (int64_t)hk * p.k_head_stride;
-        const T* vrow = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)key * p.v_row_stride + (int64_t)hk * p.v_head_stride;
-#pragma unroll
-        for (int dk = 0; dk < C::KS; dk++) {
-            const int d0 = dk * 16 + 8 * hh;
-            u32x4 a = {0, 0, 0, 0}, c = {0, 0, 0, 0};
-            if (key_ok && d0 < p.d) { a = ld_global16(krow + d0); c = ld_global16(vrow + d0); }
-            kf[dk] = __builtin_bit_cast(v8, a);
-            vf[dk] = __builtin_bit_cast(v8, c);
-        }
-    }
-    wait_resident_loads();
-
-    f32x16 dk_acc[C::DB], dv_acc[C::DB];
-#pragma unroll
-    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) { dk_acc[db][r] = 0.f; dv_acc[db][r] = 0.f; }
-
-    u32x4 qr[C::LOADS], gr[C::LOADS];
-    float aux = 0.f;
-    const int d_last_chunk = p.d / 8 - 1;
-    auto load_tile = [&](int g, int t) {
-        const int head = hk * G + g;
-        const int i0 = t * BM;
-        const T* qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
-        const T* gg = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride;
-#pragma unroll
-        for (int i = 0; i < C::LOADS; i++) {
-            const int f = tid + i * C::kThreads;
-            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
-            const int n = min(i0 + r, si.sq - 1);
-            qr[i] = ld_global16(qg + (int64_t)n * p.q_row_stride + c * 8);
-            gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
-        }
-        if (tid < 2 * BM) {
-            // raw value only: anything computed from it here would make the wave wait for the load
-            // (and, loads completing in order, for the whole tile) before the current tile's products
-            const int r = min(i0 + (tid < BM ? tid : tid - BM), si.sq - 1);
-            const float* src = tid < BM ? p.softmax_lse + ((int64_t)b * p.h + head) * p.seqlen_q
-                                        : p.softmax_d + ((int64_t)b * p.h + head) * p.seqlen_q_rounded;
-            aux = src[r];
-        }
-    };
-    auto store_tile = [&](int buf, int t) {
-        char* qb = smem + buf * C::STAGE;
-        char* gb = qb + C::TILE_BYTES;
-        const int i0 = t * BM;
-#pragma unroll
-        for (int i = 0; i < C::LOADS; i++) {
-            const int f = tid + i * C::kThreads;
-            const int r = f / C::CPR, c = f % C::CPR;
-            const bool ok = (i0 + r < si.sq) && (c <= d_last_chunk);
-            const u32x4 z = {0, 0, 0, 0};
-            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
-            *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
-            *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
-        }
-        if (tid < 2 * BM) {
-            const bool in_range = i0 + (tid < BM ? tid : tid - BM) < si.sq;   // rows past the end: lse = +inf => P = 0
-            reinterpret_cast<float*>(gb + C::TILE_BYTES)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? aux : 0.f);
-        }
-    };
-
-    const float sl2 = kp.scale_log2;
-    const int rel_hi = has_right ? shift + wr : 0x3fffffff;
-    const int rel_lo = has_left ? shift - wl : -0x3fffffff;
-    LdsOffs<D, C::KS, D / 32> lo;
-    lo.init(lane);
-    if (iters > 0) { load_tile(0, t_lo); store_tile(0, t_lo); }
-    __syncthreads();
-    int buf = 0;
-    int cur_t = t_lo, cur_g = 0, nxt_g = 0, nxt_t = t_lo;   // (head of group, query tile) walked without divisions
-    Drop drop = {0, 0, 256, 1.f};
-    for (int it = 0; it < iters; ++it) {
-        const bool has_next = it + 1 < iters;
-        if (has_next) {
-            if (++nxt_t == t_hi) { nxt_t = t_lo; ++nxt_g; }
-            load_tile(nxt_g, nxt_t);
-        }
-        const int i0 = cur_t * BM;
-        if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, hk * G + cur_g, p.h);
-        const char* qb = smem + buf * C::STAGE;
-        const char* gb = qb + C::TILE_BYTES;
-        const float* lse_s = reinterpret_cast<const float*>(gb + C::TILE_BYTES);
-        const float* dsum_s = lse_s + BM;
-
-        // keys of this wave against the rows of the tile: nothing visible -> nothing to add
-        const bool wave_skip = (has_right && j0w > i0 + BM - 1 + shift + wr) || (has_left && j0w + 31 < i0 + shift - wl) ||
-                               (j0w >= si.sk);
-        if (!wave_skip) {
-            f32x16 s_acc[C::MBK], dp_acc[C::MBK];
-            product_rows<T, D, C::MBK, C::KS, 4>(s_acc, qb, lo.r, kf);
-            product_rows<T, D, C::MBK, C::KS, 4>(dp_acc, gb, lo.r, vf);
-            v8 pf[C::PT], dsf[C::PT];
-#pragma unroll
-            for (int mb = 0; mb < C::MBK; mb++) {
-                const int ib = i0 + mb * 32;
-                const bool need_mask = (has_right && j0w + 31 > ib + shift + wr) || (has_left && j0w < ib + 31 + shift - wl);
-                if (need_mask) {
-                    // key - row must lie in [rel_lo, rel_hi]; the row of register r is ib + 4 hh + c_r
-                    const int rel = key - ib - 4 * hh;
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int c_r = 8 * (r >> 2) + (r & 3);
-                        s_acc[mb][r] = (rel > rel_hi + c_r || rel < rel_lo + c_r) ? -INFINITY : s_acc[mb][r];
-                    }
-                }
-                uint32_t keep = 0xffffu;
-                if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);
-#pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) {
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int r = 4 * q4 + e;
-                        const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
-                        const bool kept = (keep >> r) & 1u;
-                        float dpv = dp_acc[mb][r];
-                        if constexpr (DROPOUT) dpv = kept ? dpv * drop.rp : 0.f;
-                        s_acc[mb][r] = (!DROPOUT || kept) ? pv : 0.f;
-                        dp_acc[mb][r] = pv * (dpv - d4[e]);
-                    }
-                }
-                pf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
-                pf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
-                dsf[2 * mb] = pack_acc8<T>(dp_acc[mb], 0);
-                dsf[2 * mb + 1] = pack_acc8<T>(dp_acc[mb], 8);
-            }
-            // dV^T += dO^T P,  dK^T += Q^T dS   (columns of this workgroup's part of the head dim)
-            product_cols<T, D, C::PT, C::DB, 4>(dv_acc, gb, lo.c, pf, dpart * C::DB);
-            product_cols<T, D, C::PT, C::DB, 4>(dk_acc, qb, lo.c, dsf, dpart * C::DB);
-        }
-        if (has_next) store_tile(buf ^ 1, nxt_t);
-        __syncthreads();
-        buf ^= 1;
-        cur_t = nxt_t;
-        cur_g = nxt_g;
-    }
-
-    if (!key_ok) return;
-    T* dkrow = reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride;
-    T* dvrow = reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
-    const float sc = p.softmax_scale;
-    const float rp = DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f;
-#pragma unroll
-    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-            const int d0 = (dpart * C::DB + db) * 32 + 8 * q4 + 4 * hh;
-            if (d0 < p.d) {
-                u32x2 a = {pack2<T>(dk_acc[db][4 * q4] * sc, dk_acc[db][4 * q4 + 1] * sc),
-                           pack2<T>(dk_acc[db][4 * q4 + 2] * sc, dk_acc[db][4 * q4 + 3] * sc)};
-                u32x2 c = {pack2<T>(dv_acc[db][4 * q4] * rp, dv_acc[db][4 * q4 + 1] * rp),
-                           pack2<T>(dv_acc[db][4 * q4 + 2] * rp, dv_acc[db][4 * q4 + 3] * rp)};
-                st_global8(dkrow + d0, a);
-                st_global8(dvrow + d0, c);
-            }
-        }
-}
-
-// ------------------------------------------------------------------------------------------------
-// dK, dV without repeating any product (head dim <= 128).  8 waves; wave w < 4 ("P wave") owns key
+// dK, dV: a workgroup owns 128 keys of one (batch, kv head) and streams the Q / dO tiles (BM query rows)
+// of every query head of the group; no product is repeated.  8 waves; wave w < 4 ("P wave") owns key
 // block w for S = Q K^T, P = exp(S - lse) and dV^T += dO^T P; wave w + 4 ("dS wave") owns the same keys
 // for dP = dO V^T, dS = P o (dP - D) and dK^T += Q^T dS.  P goes from the first to the second through
 // LDS in accumulator layout (both waves map lanes to keys and registers to query rows identically,
@@ -494,11 +275,14 @@ __global__ void __launch_bounds__(256, MINW) bwd_dkv_kernel(const BwdKParams kp)
 // t - 1 (P of that tile was published before the barrier that ended step t - 1), so no barrier is
 // added and its exp-free vector work overlaps its own products.  The Q ring therefore has three
 // stages (tile t + 1 arriving, t read by the P wave, t - 1 read transposed by the dS wave); dO has two.
+// With DPARTS = 2 (head dim 256) two workgroups share a key block and each accumulates half of the
+// head dimension of dK / dV (both form S and dP in full): the accumulators of all 256 columns would
+// not fit next to the resident K / V row in 256 registers.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int D, int BM>
+template <typename T, int D, int BM, int DPARTS>
 struct BwdDkv3Cfg {
     static constexpr int kThreads = 512, kWaves = 8, BNW = 128;
-    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32 / DPARTS, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
     static constexpr int TILE_BYTES = BM * ROWB;
     static constexpr int LOADS = BM * CPR / kThreads;
     static constexpr int Q_OFF = 0;                                  // 3 stages
@@ -507,13 +291,13 @@ struct BwdDkv3Cfg {
     static constexpr int X_OFF = AUX_OFF + 3 * 2 * BM * 4;           // P hand-over: 2 buffers x 4 key blocks
     static constexpr int XBLK = BM * 32 * 4;                         // one key block's P tile, fp32
     static constexpr int SMEM = X_OFF + 2 * 4 * XBLK;
-    static_assert(BM % 32 == 0 && D % 32 == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
+    static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
     static_assert(SMEM <= 160 * 1024, "LDS budget");
 };
 
-template <typename T, int D, int BM, bool DROPOUT>
+template <typename T, int D, int BM, int DPARTS, bool DROPOUT>
 __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
-    typedef BwdDkv3Cfg<T, D, BM> C;
+    typedef BwdDkv3Cfg<T, D, BM, DPARTS> C;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_bwd_params& p = kp.p;
@@ -523,10 +307,11 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
 
     const int G = p.h / p.h_k;
     const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
-    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b;
+    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b * DPARTS;
     const int per_xcd = gridDim.x >> 3;
     int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (w >= total) return;
+    const int dpart = (int)(w % DPARTS); w /= DPARTS;      // with DPARTS = 2 a workgroup accumulates half of the head dim
     const int nblk = (int)(w % num_n_blocks); w /= num_n_blocks;
     const int hk = (int)(w % p.h_k);
     const int b = (int)(w / p.h_k);
@@ -622,7 +407,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     const int rel_hi = has_right ? shift + wr : 0x3fffffff;
     const int rel_lo = has_left ? shift - wl : -0x3fffffff;
     LdsOffs<D, C::KS, C::DB> lo;
-    lo.init(lane);
+    lo.init(lane, dpart * C::DB);
 
     // The tile walk shared by both kinds of wave; `body(it, i0, g, live, prev_live, q3, q3_prev)` is the
     // wave's own work of one step.  iters + 1 steps: the last one drains the dS wave's final tile.
@@ -746,7 +531,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
-            const int d0 = db * 32 + 8 * q4 + 4 * hh;
+            const int d0 = (dpart * C::DB + db) * 32 + 8 * q4 + 4 * hh;
             if (d0 < p.d) {
                 u32x2 a = {pack2<T>(acc[db][4 * q4] * sc, acc[db][4 * q4 + 1] * sc),
                            pack2<T>(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc)};
@@ -775,27 +560,14 @@ int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-template <typename T, int D, int BM, int DPARTS, int MINW, bool DROPOUT>
-int launch_bwd_dkv(const BwdKParams& kp, hipStream_t stream) {
-    typedef BwdDkvCfg<T, D, BM, DPARTS> C;
+template <typename T, int D, int BM, int DPARTS, bool DROPOUT>
+int launch_bwd_dkv3(const BwdKParams& kp, hipStream_t stream) {
+    typedef BwdDkv3Cfg<T, D, BM, DPARTS> C;
     const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b * DPARTS;
     if (total <= 0) return 0;
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    auto kern = bwd_dkv_kernel<T, D, BM, DPARTS, MINW, DROPOUT>;
-    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
-    return (int)hipGetLastError();
-}
-
-template <typename T, int D, int BM, bool DROPOUT>
-int launch_bwd_dkv3(const BwdKParams& kp, hipStream_t stream) {
-    typedef BwdDkv3Cfg<T, D, BM> C;
-    const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b;
-    if (total <= 0) return 0;
-    const int64_t per_xcd = (total + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    auto kern = bwd_dkv3_kernel<T, D, BM, DROPOUT>;
+    auto kern = bwd_dkv3_kernel<T, D, BM, DPARTS, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();

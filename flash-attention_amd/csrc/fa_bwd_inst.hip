@@ -20,10 +20,10 @@ static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers
     if (int e = launch_bwd_dq<InstT, FA_D, (FA_D > 64 ? 32 : 64), 2, DROPOUT>(kp, stream)) return e;
-    return launch_bwd_dkv3<InstT, FA_D, 64, DROPOUT>(kp, stream);
+    return launch_bwd_dkv3<InstT, FA_D, 64, 1, DROPOUT>(kp, stream);
 #else
     if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
-    return launch_bwd_dkv<InstT, FA_D, 32, 2, 1, DROPOUT>(kp, stream);
+    return launch_bwd_dkv3<InstT, FA_D, 32, 2, DROPOUT>(kp, stream);
 #endif
 }
 

@@ -259,7 +259,7 @@ template <int D, int KS, int DB>
 struct LdsOffs {
     int r[KS];       // row-wise: row l32, k-step dk
     int c[DB][2];    // transposed: column block db, rows 4hh + tj and 8 more
-    FA_DEV void init(int lane) {
+    FA_DEV void init(int lane, int db0 = 0) {      // db0: first 32-column block of the DB blocks this wave reads
         const int l32 = lane & 31, hh = lane >> 5;
 #pragma unroll
         for (int dk = 0; dk < KS; dk++) r[dk] = l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16;
@@ -267,7 +267,7 @@ struct LdsOffs {
         const int row = 4 * hh + tj;
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-            const int cc = db * 4 + dhalf * 2 + (tq >> 1);
+            const int cc = (db0 + db) * 4 + dhalf * 2 + (tq >> 1);
             c[db][0] = row * (D * 2) + swz_u<D>(cc, row) * 16 + (tq & 1) * 8;
             c[db][1] = (row + 8) * (D * 2) + swz_u<D>(cc, row + 8) * 16 + (tq & 1) * 8;
         }
@@ -319,20 +319,20 @@ FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const t
 }
 // acc[db] += columns [32 db, 32 db + 32) of tile rows [16 t16, 16 t16 + 16), transposed  x  bfrag[t16]
 template <typename T, int D, int PT, int DB, int GRP>
-FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], const typename Elem<T>::v8* bfrag, int db0 = 0) {
+FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], const typename Elem<T>::v8* bfrag) {
     typedef typename Elem<T>::v8 v8;
     constexpr int TOTAL = PT * DB, NG = TOTAL / GRP;
     static_assert(TOTAL % GRP == 0, "group shape");
     v8 a[2][GRP];
 #pragma unroll
-    for (int j = 0; j < GRP; j++) a[0][j] = lds_cols_at<T, D>(tile, offc[db0 + j % DB][0], offc[db0 + j % DB][1], j / DB);
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_cols_at<T, D>(tile, offc[j % DB][0], offc[j % DB][1], j / DB);
 #pragma unroll
     for (int g = 0; g < NG; g++) {
         if (g + 1 < NG) {
 #pragma unroll
             for (int j = 0; j < GRP; j++) {
                 const int st = (g + 1) * GRP + j;
-                a[(g + 1) & 1][j] = lds_cols_at<T, D>(tile, offc[db0 + st % DB][0], offc[db0 + st % DB][1], st / DB);
+                a[(g + 1) & 1][j] = lds_cols_at<T, D>(tile, offc[st % DB][0], offc[st % DB][1], st / DB);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
