@@ -208,6 +208,10 @@ static int run_bwd(const fa_bwd_params* p, bool varlen, hipStream_t stream) {
                                   p->q_batch_stride, p->k_batch_stride, p->v_batch_stride, p->o_batch_stride, p->do_batch_stride};
     for (int64_t st : in_strides) if (st % 8 != 0) return fail("input strides must be multiples of 8 elements (16-byte rows)");
 
+    // the tile movers add a 32-bit lane byte offset (up to 128 rows) to a 64-bit tile base
+    const int64_t row_strides[] = {p->q_row_stride, p->k_row_stride, p->v_row_stride, p->do_row_stride};
+    for (int64_t st : row_strides) if (st < 0 || st >= ((int64_t)1 << 23)) return fail("row strides must be below 2^23 elements");
+
     BwdKParams kp;
     kp.p = *p;
     if (kp.p.is_causal) kp.p.window_right = 0;     // flash_api.cpp:627

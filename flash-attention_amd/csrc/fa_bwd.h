@@ -95,6 +95,7 @@ struct BwdDqCfg {
     static constexpr int LOADS = BN * CPR / kThreads;
     static constexpr int SMEM = 4 * TILE_BYTES;   // {K, V} x 2 stages
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
+    static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
 };
 
 template <typename T, int D, int BN, int MINW, bool DROPOUT>
@@ -162,32 +163,42 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 #pragma unroll
         for (int r = 0; r < 16; r++) dq_acc[db][r] = 0.f;
 
-    u32x4 kr[C::LOADS], vr[C::LOADS];
+    // Tile movers: K and V go from global memory straight into LDS (global_load_lds, 1 KB per wave
+    // instruction); the swizzle is applied on the global side.  No zero fill: keys past the sequence
+    // repeat its last key and are masked, columns past d repeat the last chunk and meet the zero
+    // columns of the resident Q / dO rows or land in dQ columns that are never written.
     const int d_last_chunk = p.d / 8 - 1;
-    auto load_tile = [&](int t) {
-        const int n0 = t * BN;
+    const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
+    const uint32_t fill0 = __builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(wave * C::LOADS * 1024)));
+    int f_row[C::LOADS], f_col[C::LOADS];
+    uint32_t f_koff[C::LOADS], f_voff[C::LOADS];
 #pragma unroll
-        for (int i = 0; i < C::LOADS; i++) {
-            const int f = tid + i * C::kThreads;
-            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
-            const int n = min(n0 + r, si.sk - 1);
-            kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
-            vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
-        }
-    };
-    auto store_tile = [&](int buf, int t) {
-        char* kb = smem + buf * 2 * C::TILE_BYTES;
-        char* vb = kb + C::TILE_BYTES;
+    for (int j = 0; j < C::LOADS; j++) {
+        const int pos = (wave * C::LOADS + j) * 1024 + lane * 16;
+        f_row[j] = pos / C::ROWB;
+        f_col[j] = min(swz_u<D>((pos % C::ROWB) / 16, f_row[j]), d_last_chunk);
+        f_koff[j] = (uint32_t)((f_row[j] * (int)p.k_row_stride + f_col[j] * 8) * 2);
+        f_voff[j] = (uint32_t)((f_row[j] * (int)p.v_row_stride + f_col[j] * 8) * 2);
+    }
+    auto load_tile = [&](int buf, int t) {
         const int n0 = t * BN;
+        const T* kt = kg + (int64_t)n0 * p.k_row_stride;
+        const T* vt = vg + (int64_t)n0 * p.v_row_stride;
+        const uint32_t dk_ = fill0 + (uint32_t)(buf * 2 * C::TILE_BYTES);
+        const uint32_t dv_ = dk_ + (uint32_t)C::TILE_BYTES;
+        if (n0 + BN <= si.sk) {
 #pragma unroll
-        for (int i = 0; i < C::LOADS; i++) {
-            const int f = tid + i * C::kThreads;
-            const int r = f / C::CPR, c = f % C::CPR;
-            const bool ok = (n0 + r < si.sk) && (c <= d_last_chunk);
-            const u32x4 z = {0, 0, 0, 0};
-            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
-            *reinterpret_cast<u32x4*>(kb + off) = ok ? kr[i] : z;
-            *reinterpret_cast<u32x4*>(vb + off) = ok ? vr[i] : z;
+            for (int j = 0; j < C::LOADS; j++) {
+                async_fill16(kt, f_koff[j], dk_ + j * 1024);
+                async_fill16(vt, f_voff[j], dv_ + j * 1024);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) {
+                const int r = min(f_row[j], si.sk - 1 - n0);
+                async_fill16(kt, (uint32_t)((r * (int)p.k_row_stride + f_col[j] * 8) * 2), dk_ + j * 1024);
+                async_fill16(vt, (uint32_t)((r * (int)p.v_row_stride + f_col[j] * 8) * 2), dv_ + j * 1024);
+            }
         }
     };
 
@@ -196,12 +207,12 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
     LdsOffs<D, C::KS, C::DB> lo;
     lo.init(lane);
-    if (t_hi > t_lo) { load_tile(t_lo); store_tile(0, t_lo); }
+    if (t_hi > t_lo) { load_tile(0, t_lo); wait_vmcnt<0>(); }
     __syncthreads();
     int buf = 0;
     for (int t = t_lo; t < t_hi; ++t) {
         const bool has_next = t + 1 < t_hi;
-        if (has_next) load_tile(t + 1);
+        if (has_next) load_tile(buf ^ 1, t + 1);     // the other stage was last read before the previous barrier
         const int n0 = t * BN;
         const char* kb = smem + buf * 2 * C::TILE_BYTES;
         const char* vb = kb + C::TILE_BYTES;
@@ -243,7 +254,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
             // dQ^T += K^T dS^T
             product_cols<T, D, C::PT, C::DB, 4>(dq_acc, kb, lo.c, dsf);
         }
-        if (has_next) store_tile(buf ^ 1, t + 1);
+        wait_vmcnt<0>();       // this wave's fills of the next tile have landed; the barrier publishes them
         __syncthreads();
         buf ^= 1;
     }
@@ -293,6 +304,7 @@ struct BwdDkv3Cfg {
     static constexpr int SMEM = X_OFF + 2 * 4 * XBLK;
     static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
     static_assert(SMEM <= 160 * 1024, "LDS budget");
+    static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
 };
 
 template <typename T, int D, int BM, int DPARTS, bool DROPOUT>
@@ -355,47 +367,61 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
 
-    u32x4 qr[C::LOADS], gr[C::LOADS];
+    // Tile movers.  Q and dO go from global memory straight into their ring slots (global_load_lds,
+    // 1 KB per wave instruction, no staging registers and no LDS store pass): LDS bytes are laid down
+    // in lane order, so the swizzle is applied on the global side -- the lane that fills physical chunk
+    // pc of row r fetches logical chunk swz_u(pc, r).  There is no zero fill on this path: rows past
+    // the sequence repeat its last row and are neutralised by lse = +inf (P = 0), columns past d repeat
+    // the last chunk and meet the zero columns of the resident K / V rows, or land in gradient
+    // columns that are never written.  lse and D take the register path (one float per lane).
     float aux = 0.f;
     const int d_last_chunk = p.d / 8 - 1;
-    auto load_tile = [&](int g, int t) {
+    const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
+    const uint32_t fill0 = __builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(wave * C::LOADS * 1024)));
+    int f_row[C::LOADS], f_col[C::LOADS];
+    uint32_t f_qoff[C::LOADS], f_goff[C::LOADS];
+#pragma unroll
+    for (int j = 0; j < C::LOADS; j++) {
+        const int pos = (wave * C::LOADS + j) * 1024 + lane * 16;
+        f_row[j] = pos / C::ROWB;
+        f_col[j] = min(swz_u<D>((pos % C::ROWB) / 16, f_row[j]), d_last_chunk);
+        f_qoff[j] = (uint32_t)((f_row[j] * (int)p.q_row_stride + f_col[j] * 8) * 2);
+        f_goff[j] = (uint32_t)((f_row[j] * (int)p.do_row_stride + f_col[j] * 8) * 2);
+    }
+    const int aux_row = tid < BM ? tid : tid - BM;
+    auto load_tile = [&](int g, int t, int q3, int g2) {
         const int head = hk * G + g;
         const int i0 = t * BM;
-        const T* qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
-        const T* gg = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride;
+        const T* qt = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride + (int64_t)i0 * p.q_row_stride;
+        const T* gt = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride + (int64_t)i0 * p.do_row_stride;
+        const uint32_t dq_ = fill0 + (uint32_t)(C::Q_OFF + q3 * C::TILE_BYTES);
+        const uint32_t dg_ = fill0 + (uint32_t)(C::G_OFF + g2 * C::TILE_BYTES);
+        if (i0 + BM <= si.sq) {
 #pragma unroll
-        for (int i = 0; i < C::LOADS; i++) {
-            const int f = tid + i * C::kThreads;
-            const int r = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
-            const int n = min(i0 + r, si.sq - 1);
-            qr[i] = ld_global16(qg + (int64_t)n * p.q_row_stride + c * 8);
-            gr[i] = ld_global16(gg + (int64_t)n * p.do_row_stride + c * 8);
+            for (int j = 0; j < C::LOADS; j++) {
+                async_fill16(qt, f_qoff[j], dq_ + j * 1024);
+                async_fill16(gt, f_goff[j], dg_ + j * 1024);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < C::LOADS; j++) {
+                const int r = min(f_row[j], si.sq - 1 - i0);
+                async_fill16(qt, (uint32_t)((r * (int)p.q_row_stride + f_col[j] * 8) * 2), dq_ + j * 1024);
+                async_fill16(gt, (uint32_t)((r * (int)p.do_row_stride + f_col[j] * 8) * 2), dg_ + j * 1024);
+            }
         }
         if (tid < 2 * BM) {
             // raw value only: anything computed from it here would make the wave wait for the load
-            // (and, loads completing in order, for the whole tile) before the current tile's products
-            const int r = min(i0 + (tid < BM ? tid : tid - BM), si.sq - 1);
             const float* src = tid < BM ? p.softmax_lse + ((int64_t)b * p.h + head) * p.seqlen_q
                                         : p.softmax_d + ((int64_t)b * p.h + head) * p.seqlen_q_rounded;
-            aux = src[r];
+            aux = src[min(i0 + aux_row, si.sq - 1)];
         }
     };
-    auto store_tile = [&](int q3, int g2, int t) {
-        char* qb = smem + C::Q_OFF + q3 * C::TILE_BYTES;
-        char* gb = smem + C::G_OFF + g2 * C::TILE_BYTES;
-        const int i0 = t * BM;
-#pragma unroll
-        for (int i = 0; i < C::LOADS; i++) {
-            const int f = tid + i * C::kThreads;
-            const int r = f / C::CPR, c = f % C::CPR;
-            const bool ok = (i0 + r < si.sq) && (c <= d_last_chunk);
-            const u32x4 z = {0, 0, 0, 0};
-            const int off = r * C::ROWB + swz_u<D>(c, r) * 16;
-            *reinterpret_cast<u32x4*>(qb + off) = ok ? qr[i] : z;
-            *reinterpret_cast<u32x4*>(gb + off) = ok ? gr[i] : z;
-        }
+    // end of a step: the wave's own fills have landed (the barrier that follows publishes them), lse / D go to LDS
+    auto finish_tile = [&](int q3, int t) {
+        wait_vmcnt<0>();
         if (tid < 2 * BM) {
-            const bool in_range = i0 + (tid < BM ? tid : tid - BM) < si.sq;   // rows past the end: lse = +inf => P = 0
+            const bool in_range = t * BM + aux_row < si.sq;   // rows past the end: lse = +inf => P = 0
             reinterpret_cast<float*>(smem + C::AUX_OFF + q3 * 2 * BM * 4)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? aux : 0.f);
         }
     };
@@ -412,23 +438,25 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     // The tile walk shared by both kinds of wave; `body(it, i0, g, live, prev_live, q3, q3_prev)` is the
     // wave's own work of one step.  iters + 1 steps: the last one drains the dS wave's final tile.
     auto walk = [&](auto&& body) {
-        if (iters > 0) { load_tile(0, t_lo); store_tile(0, 0, t_lo); }
+        if (iters > 0) { load_tile(0, t_lo, 0, 0); finish_tile(0, t_lo); }
         __syncthreads();
         int q3 = 0, q3_prev = 0;                     // Q / aux ring slots of the current and the previous tile
         int cur_t = t_lo, cur_g = 0, nxt_g = 0, nxt_t = t_lo;
         bool prev_live = false;                      // the previous tile was not skipped (its P is in the hand-over)
         for (int it = 0; it <= iters; ++it) {
             const bool has_next = it + 1 < iters;
+            const int q3_next = q3 == 2 ? 0 : q3 + 1;
             if (has_next) {
                 if (++nxt_t == t_hi) { nxt_t = t_lo; ++nxt_g; }
-                load_tile(nxt_g, nxt_t);
+                // slots free since the barrier that ended the previous step: Q[q3_next] held tile it - 2
+                // (last read transposed by the dS wave in step it - 1), dO[(it + 1) & 1] held tile it - 1
+                load_tile(nxt_g, nxt_t, q3_next, (it + 1) & 1);
             }
             const int i0 = cur_t * BM;
             const bool live = it < iters && !skip_tile(i0);
             body(it, i0, cur_g, live, prev_live, q3, q3_prev);
             prev_live = live;
-            const int q3_next = q3 == 2 ? 0 : q3 + 1;
-            if (has_next) store_tile(q3_next, (it + 1) & 1, nxt_t);
+            if (has_next) finish_tile(q3_next, nxt_t);
             __syncthreads();
             q3_prev = q3;
             q3 = q3_next;

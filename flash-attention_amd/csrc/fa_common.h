@@ -345,6 +345,21 @@ FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], co
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// 16 B per lane from global memory (uniform base + per-lane byte offset) to LDS address
+// m0_base + lane * 16, bypassing registers.  The base is uniform by construction; reading it through
+// readfirstlane tells the compiler so (the instruction takes it in scalar registers).
+FA_DEV void async_fill16(const void* base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
+    const uint64_t a = (uint64_t)base_uniform;
+    const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                           ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base_uniform), "v"(lane_offset), "s"(sbase) : "memory", "m0");
+}
+// wait until at most N of this wave's vector-memory operations are outstanding (N < 16)
+template <int N> FA_DEV void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));
+}
+
 // Resolved per-(batch) sequence bookkeeping.  Mirrors the reference's BlockInfo
 // (csrc/flash_attn/src/block_info.h:11-42) with 64-bit offsets.
 struct SeqInfo {

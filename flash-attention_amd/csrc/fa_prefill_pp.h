@@ -53,21 +53,6 @@ struct PPCfg {
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
-// 16 B per lane from global memory (uniform base + per-lane byte offset) to LDS address
-// m0_base + lane * 16, bypassing registers.  The base is uniform by construction; reading it through
-// readfirstlane tells the compiler so (the instruction takes it in scalar registers).
-FA_DEV void async_fill16(const void* base_uniform, uint32_t lane_offset, uint32_t lds_base_uniform) {
-    const uint64_t a = (uint64_t)base_uniform;
-    const uint64_t sbase = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
-                           ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_base_uniform), "v"(lane_offset), "s"(sbase) : "memory", "m0");
-}
-// wait until at most N of this wave's vector-memory operations are outstanding (N < 16)
-template <int N> FA_DEV void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));
-}
-
 template <typename T, int D, int BN>
 __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     typedef PPCfg<T, D, BN> C;
