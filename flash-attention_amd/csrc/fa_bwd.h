@@ -377,12 +377,16 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     float aux = 0.f;
     const int d_last_chunk = p.d / 8 - 1;
     const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
-    const uint32_t fill0 = __builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(wave * C::LOADS * 1024)));
-    int f_row[C::LOADS], f_col[C::LOADS];
-    uint32_t f_qoff[C::LOADS], f_goff[C::LOADS];
+    // Only the P waves request tiles (FL fills each per tensor): a CU accepts 64 bytes of vector loads
+    // per cycle, so a tile keeps the requesting waves at the top of the step for several hundred
+    // cycles; meanwhile the dS waves, which request nothing, have the matrix pipe to themselves.
+    constexpr int FL = 2 * C::LOADS;
+    const uint32_t fill0 = __builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(kblk * FL * 1024)));
+    int f_row[FL], f_col[FL];
+    uint32_t f_qoff[FL], f_goff[FL];
 #pragma unroll
-    for (int j = 0; j < C::LOADS; j++) {
-        const int pos = (wave * C::LOADS + j) * 1024 + lane * 16;
+    for (int j = 0; j < FL; j++) {
+        const int pos = (kblk * FL + j) * 1024 + lane * 16;
         f_row[j] = pos / C::ROWB;
         f_col[j] = min(swz_u<D>((pos % C::ROWB) / 16, f_row[j]), d_last_chunk);
         f_qoff[j] = (uint32_t)((f_row[j] * (int)p.q_row_stride + f_col[j] * 8) * 2);
@@ -396,15 +400,17 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
         const T* gt = reinterpret_cast<const T*>(p.dout) + si.do_off + (int64_t)head * p.do_head_stride + (int64_t)i0 * p.do_row_stride;
         const uint32_t dq_ = fill0 + (uint32_t)(C::Q_OFF + q3 * C::TILE_BYTES);
         const uint32_t dg_ = fill0 + (uint32_t)(C::G_OFF + g2 * C::TILE_BYTES);
-        if (i0 + BM <= si.sq) {
+        if (role_ds) {
+            // nothing to request
+        } else if (i0 + BM <= si.sq) {
 #pragma unroll
-            for (int j = 0; j < C::LOADS; j++) {
+            for (int j = 0; j < FL; j++) {
                 async_fill16(qt, f_qoff[j], dq_ + j * 1024);
                 async_fill16(gt, f_goff[j], dg_ + j * 1024);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < C::LOADS; j++) {
+            for (int j = 0; j < FL; j++) {
                 const int r = min(f_row[j], si.sq - 1 - i0);
                 async_fill16(qt, (uint32_t)((r * (int)p.q_row_stride + f_col[j] * 8) * 2), dq_ + j * 1024);
                 async_fill16(gt, (uint32_t)((r * (int)p.do_row_stride + f_col[j] * 8) * 2), dg_ + j * 1024);
