@@ -51,6 +51,14 @@ static int check_common(const fa_fwd_params* p) {
     if (p->h <= 0 || p->h_k <= 0 || p->h % p->h_k != 0) return fail("Number of heads in key/value must divide number of heads in query");
     if (p->seqlen_q < 0 || p->seqlen_k < 0) return fail("sequence lengths must be non-negative");
     if (p->num_splits < 0 || p->num_splits > FA_MAX_SPLITS) return fail("num_splits > 128 not supported");
+    // every global access is a 16-byte piece of a row
+    const void* ptrs[] = {p->q, p->k, p->v, p->o, p->k_new, p->v_new};
+    for (const void* q : ptrs) if ((uintptr_t)q % 16 != 0) return fail("q, k, v, o, k_new and v_new must be 16-byte aligned");
+    const int64_t strides[] = {p->q_batch_stride, p->q_row_stride, p->q_head_stride, p->k_batch_stride, p->k_row_stride,
+                               p->k_head_stride, p->v_batch_stride, p->v_row_stride, p->v_head_stride, p->o_batch_stride,
+                               p->o_row_stride, p->o_head_stride, p->knew_batch_stride, p->knew_row_stride,
+                               p->knew_head_stride, p->vnew_batch_stride, p->vnew_row_stride, p->vnew_head_stride};
+    for (int64_t st : strides) if (st % 8 != 0) return fail("strides must be multiples of 8 elements (16-byte rows)");
     if (!(p->p_dropout >= 0.f && p->p_dropout < 1.f)) return fail("p_dropout must be in [0, 1)");
     if (p->p_dropout > 0.f && !p->rng_state) return fail("rng_state is required when p_dropout > 0");
     if (p->s_dmask && (p->sdm_rows < p->seqlen_q || p->sdm_cols < p->seqlen_k)) return fail("s_dmask is smaller than (seqlen_q, seqlen_k)");
@@ -208,6 +216,10 @@ static int run_bwd(const fa_bwd_params* p, bool varlen, hipStream_t stream) {
                                   p->q_batch_stride, p->k_batch_stride, p->v_batch_stride, p->o_batch_stride, p->do_batch_stride};
     for (int64_t st : in_strides) if (st % 8 != 0) return fail("input strides must be multiples of 8 elements (16-byte rows)");
 
+    const void* in_ptrs[] = {p->dout, p->q, p->k, p->v, p->out};
+    for (const void* q : in_ptrs) if ((uintptr_t)q % 16 != 0) return fail("dout, q, k, v and out must be 16-byte aligned");
+    const void* out_ptrs[] = {p->dq, p->dk, p->dv};
+    for (const void* q : out_ptrs) if ((uintptr_t)q % 8 != 0) return fail("dq, dk and dv must be 8-byte aligned");
     // the tile movers add a 32-bit lane byte offset (up to 128 rows) to a 64-bit tile base
     const int64_t row_strides[] = {p->q_row_stride, p->k_row_stride, p->v_row_stride, p->do_row_stride};
     for (int64_t st : row_strides) if (st < 0 || st >= ((int64_t)1 << 23)) return fail("row strides must be below 2^23 elements");
