@@ -219,37 +219,36 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
         const bool skip = (has_right && n0 > r0w + 31 + shift + wr) || (has_left && n0 + BN - 1 < r0w + shift - wl) ||
                           (r0w >= si.sq);
         if (!skip) {
-            f32x16 s_acc[C::NB], dp_acc[C::NB];
-            product_rows<T, D, C::NB, C::KS, 4>(s_acc, kb, lo.r, qf);
-            product_rows<T, D, C::NB, C::KS, 4>(dp_acc, vb, lo.r, gf);
+            // one 32-key block at a time, so that only one block's S and dP are live
             const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0w + shift + wr) ||
                                    (has_left && n0 < r0w + 31 + shift - wl);
-            if (need_mask) {
-                int lim_hi = si.sk - 1;
-                if (has_right) lim_hi = min(lim_hi, row + shift + wr);
-                const int lim_lo = has_left ? row + shift - wl : 0;
-#pragma unroll
-                for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-                        if (n > lim_hi || n < lim_lo) s_acc[nb][r] = -INFINITY;
-                    }
-            }
+            int lim_hi = si.sk - 1;
+            if (has_right) lim_hi = min(lim_hi, row + shift + wr);
+            const int lim_lo = has_left ? row + shift - wl : 0;
             v8 dsf[C::PT];
 #pragma unroll
             for (int nb = 0; nb < C::NB; nb++) {
+                f32x16 s_acc[1], dp_acc[1];
+                product_rows<T, D, 1, C::KS, 4>(s_acc, kb + nb * 32 * C::ROWB, lo.r, qf);
+                product_rows<T, D, 1, C::KS, 4>(dp_acc, vb + nb * 32 * C::ROWB, lo.r, gf);
+                if (need_mask) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                        if (n > lim_hi || n < lim_lo) s_acc[0][r] = -INFINITY;
+                    }
+                }
                 uint32_t keep = 0xffffu;
                 if constexpr (DROPOUT) keep = drop_keep16_row(drop, row, n0 + nb * 32, hh);
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const float pv = fast_exp2(s_acc[nb][r] * sl2 - lse2);
-                    float dpv = dp_acc[nb][r];
+                    const float pv = fast_exp2(s_acc[0][r] * sl2 - lse2);
+                    float dpv = dp_acc[0][r];
                     if constexpr (DROPOUT) dpv = (keep >> r) & 1u ? dpv * drop.rp : 0.f;   // gradient through the dropped P
-                    s_acc[nb][r] = pv * (dpv - dsum);
+                    s_acc[0][r] = pv * (dpv - dsum);
                 }
-                dsf[2 * nb] = pack_acc8<T>(s_acc[nb], 0);
-                dsf[2 * nb + 1] = pack_acc8<T>(s_acc[nb], 8);
+                dsf[2 * nb] = pack_acc8<T>(s_acc[0], 0);
+                dsf[2 * nb + 1] = pack_acc8<T>(s_acc[0], 8);
             }
             // dQ^T += K^T dS^T
             product_cols<T, D, C::PT, C::DB, 4>(dq_acc, kb, lo.c, dsf);

@@ -15,11 +15,14 @@ typedef _Float16 InstT;
 
 // dQ pass then dK/dV pass on the same stream; both read softmax_d, which the caller's stream has
 // already filled (launch_bwd_dot).
+#ifndef FA_DQ_BN
+#define FA_DQ_BN (FA_D > 64 ? 32 : 64)
+#endif
 template <bool DROPOUT>
 static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers
-    if (int e = launch_bwd_dq<InstT, FA_D, (FA_D > 64 ? 32 : 64), 2, DROPOUT>(kp, stream)) return e;
+    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, 2, DROPOUT>(kp, stream)) return e;
     return launch_bwd_dkv3<InstT, FA_D, 64, 1, DROPOUT>(kp, stream);
 #else
     if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
