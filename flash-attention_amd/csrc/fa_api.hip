@@ -59,6 +59,9 @@ static int check_common(const fa_fwd_params* p) {
                                p->o_row_stride, p->o_head_stride, p->knew_batch_stride, p->knew_row_stride,
                                p->knew_head_stride, p->vnew_batch_stride, p->vnew_row_stride, p->vnew_head_stride};
     for (int64_t st : strides) if (st % 8 != 0) return fail("strides must be multiples of 8 elements (16-byte rows)");
+    // the long-sequence kernels add a 32-bit lane byte offset (up to 64 rows) to a 64-bit tile base
+    if (p->k_row_stride < 0 || p->k_row_stride >= ((int64_t)1 << 23) || p->v_row_stride < 0 || p->v_row_stride >= ((int64_t)1 << 23))
+        return fail("k and v row strides must be below 2^23 elements");
     if (!(p->p_dropout >= 0.f && p->p_dropout < 1.f)) return fail("p_dropout must be in [0, 1)");
     if (p->p_dropout > 0.f && !p->rng_state) return fail("rng_state is required when p_dropout > 0");
     if (p->s_dmask && (p->sdm_rows < p->seqlen_q || p->sdm_cols < p->seqlen_k)) return fail("s_dmask is smaller than (seqlen_q, seqlen_k)");
