@@ -69,11 +69,12 @@ def test_pipelined_kernel_square(d, s, mode):
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
-@pytest.mark.parametrize("sq,sk", [(600, 1500), (1500, 600), (513, 4000), (1100, 1101)])
+@pytest.mark.parametrize("sq,sk,dtype", [(600, 1500, torch.float16), (600, 1500, torch.bfloat16), (1500, 600, torch.float16),
+                                         (1500, 600, torch.bfloat16), (513, 4000, torch.bfloat16), (1100, 1101, torch.bfloat16)])
 @pytest.mark.parametrize("mode", ["causal", "local"])
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_pipelined_kernel_rectangular(sq, sk, mode, dtype):
-    """seqlen_q != seqlen_k: bottom-right alignment, rows without any visible key (sq > sk)."""
+def test_pipelined_kernel_rectangular(sq, sk, dtype, mode):
+    """seqlen_q != seqlen_k: bottom-right alignment, rows without any visible key (sq > sk).  (fp16 only on
+    the smaller shapes: the low-precision CPU oracle is slow in fp16.)"""
     _say("pipelined rect", sq, sk, mode, dtype)
     d, b, h = 128, 2, 32
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, 1, d), dtype, 2); v = _gen((b, sk, 1, d), dtype, 3)   # MQA
@@ -111,7 +112,7 @@ def test_pingpong_kernel(case):
                                          (1500, 600, "local"), (1024, 1024, "local")])
 def test_pair_kernel_head_dims_above_128(d, sq, sk, mode):
     _say("pair kernel", d, sq, sk, mode)
-    dtype = torch.float16 if d in (160, 224) else torch.bfloat16
+    dtype = torch.float16 if d == 160 and sq <= 777 else torch.bfloat16
     b, h, hk = 4, 16, 2
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
     window = _window(mode, sk, d * 31 + sq)
@@ -124,7 +125,7 @@ def test_pair_kernel_head_dims_above_128(d, sq, sk, mode):
 def test_long_kernels_take_strided_packed_input(s, d):
     """q, k, v as strided views of one (b, s, 3, h, d) tensor: row stride 3*h*d."""
     _say("packed long", s, d)
-    dtype = torch.float16
+    dtype = torch.bfloat16
     b, h = 2, 16
     qkv = _gen((b, s, 3, h, d), dtype, 5)
     out, lse, _ = _fa().flash_attn_qkvpacked_func(qkv.to(DEV), causal=True, return_attn_probs=True)
