@@ -14,6 +14,9 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
                 over 2 x the tensor's bytes;
   * backward -- gradients of the prefill workload (rowsum(dO o O), dQ pass, dK/dV pass); reported under
                 "backward" at the conventional 2.5 x forward FLOP count.
+  * fwd_bwd  -- the one kernel metric the reference publishes (forward + backward together, fp16, causal,
+                head dim 128, seqlen 8k, batch 2, 16 heads: 182 TFLOP/s on A100, 308 on H100), FLOPs
+                counted as 3.5 x forward like the reference's benchmark script;
 Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
 attention_ref) timed on the host cores on a bounded sample of the same workload.
 """
@@ -120,6 +123,30 @@ def bench_backward(steps, warmup):
     }
 
 
+def bench_fwd_bwd(steps, warmup):
+    import torch
+    from flash_attn import _native as nat
+    b, s, h, d = 2, 8192, 16, 128
+    torch.manual_seed(0)
+    q, k, v, dout = (torch.randn(b, s, h, d, device="cuda", dtype=torch.float16) for _ in range(4))
+    scale = d ** -0.5
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+    def fn():
+        out, _, _, _, _, lse, _, _ = nat.fwd(q, k, v, None, 0.0, scale, True, -1, -1, False, None)
+        nat.bwd(dout, q, k, v, out, lse, dq, dk, dv, 0.0, scale, True, -1, -1, None, None)
+
+    ms, wall_ms = time_steps(fn, steps, warmup)
+    flops = 3.5 * 4.0 * b * s * s * h * d / 2
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {
+        "ms": ms, "wall_ms": wall_ms, "tflops": tflops,
+        "workload": "flash_attn_func fwd+bwd fp16 batch=2 seqlen=8192 nheads=16 headdim=128 causal",
+        "published": {"a100_tflops": 182.0, "h100_tflops": 308.0, "vs_a100": tflops / 182.0, "vs_h100": tflops / 308.0,
+                      "source": "reference assets/flash2_a100_fwd_bwd_benchmark.png, flash2_h100_fwd_bwd_benchmark.png, panel (d)"},
+    }
+
+
 def bench_decode(steps, warmup):
     import torch
     import flash_attn
@@ -219,6 +246,7 @@ def main():
     if not a.no_backward:
         out["rotary"] = bench_rotary(a.steps, a.warmup)
         out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))
+        out["fwd_bwd"] = bench_fwd_bwd(a.steps, a.warmup)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
