@@ -199,3 +199,41 @@ def test_backward_rejects_missing_rng_state_and_bad_shapes():
         nat.bwd(q, q, q, q, q, lse, q[:, :4], None, None, 0.0, 0.125, False, -1, -1, None, None)
     with pytest.raises(RuntimeError, match="same dtype"):
         nat.bwd(q, q, q.to(torch.bfloat16), q, q, lse, None, None, None, 0.0, 0.125, False, -1, -1, None, None)
+
+
+def test_forward_and_backward_replay_from_a_hip_graph():
+    """A training step's attention (forward + backward, no dropout) captured once and replayed with new
+    inputs copied into the static tensors: every replay must equal the eager result.  Nothing in the
+    two entry points synchronises, allocates outside torch's graph pool or depends on device values
+    on the host."""
+    _say("bwd graph")
+    dtype, b, s, h, hk, d = torch.bfloat16, 2, 384, 4, 2, 128
+    fa = _fa()
+    q = torch.zeros(b, s, h, d, device=DEV, dtype=dtype, requires_grad=True)
+    k = torch.zeros(b, s, hk, d, device=DEV, dtype=dtype, requires_grad=True)
+    v = torch.zeros(b, s, hk, d, device=DEV, dtype=dtype, requires_grad=True)
+    dout = torch.zeros(b, s, h, d, device=DEV, dtype=dtype)
+
+    def step():
+        out = fa.flash_attn_func(q, k, v, causal=True)
+        return (out,) + torch.autograd.grad(out, (q, k, v), dout)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static = step()
+    for seed in (1, 2, 3):
+        with torch.no_grad():
+            q.copy_(_gen((b, s, h, d), dtype, seed)); k.copy_(_gen((b, s, hk, d), dtype, seed + 10))
+            v.copy_(_gen((b, s, hk, d), dtype, seed + 20)); dout.copy_(_gen((b, s, h, d), dtype, seed + 30))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = step()
+        torch.cuda.synchronize()
+        for a, c in zip(static, eager):
+            assert torch.equal(a, c)
