@@ -280,7 +280,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 // block w for S = Q K^T, P = exp(S - lse) and dV^T += dO^T P; wave w + 4 ("dS wave") owns the same keys
 // for dP = dO V^T, dS = P o (dP - D) and dK^T += Q^T dS.  P goes from the first to the second through
 // LDS in accumulator layout (both waves map lanes to keys and registers to query rows identically,
-// so the hand-over is lane to same lane, 16 bytes at a time, sign bit = dropped by dropout).
+// so the hand-over is lane to same lane, 16 bytes at a time, sign bit = dropped by dropout).  P is
+// handed over in fp16 whatever the tensor type: it lies in [0, 1], and its rounding (2^-11 relative)
+// is no coarser than the rounding dS = P o (dP - D) gets anyway as an operand of the dK product.
 // The dS wave runs ONE TILE BEHIND: in step t it forms dP of tile t (matrix pipe) and dS, dK of tile
 // t - 1 (P of that tile was published before the barrier that ended step t - 1), so no barrier is
 // added and its exp-free vector work overlaps its own products.  The Q ring therefore has three
@@ -299,7 +301,7 @@ struct BwdDkv3Cfg {
     static constexpr int G_OFF = 3 * TILE_BYTES;                     // dO: 2 stages
     static constexpr int AUX_OFF = 5 * TILE_BYTES;                   // 3 stages x {lse (log2 units), D} x BM floats
     static constexpr int X_OFF = AUX_OFF + 3 * 2 * BM * 4;           // P hand-over: 2 buffers x 4 key blocks
-    static constexpr int XBLK = BM * 32 * 4;                         // one key block's P tile, fp32
+    static constexpr int XBLK = BM * 32 * 2;                         // one key block's P tile, fp16
     static constexpr int SMEM = X_OFF + 2 * 4 * XBLK;
     static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
     static_assert(SMEM <= 160 * 1024, "LDS budget");
@@ -496,20 +498,21 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                 }
                 uint32_t keep = 0xffffu;
                 if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);
+                f32x16 xo;
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
                     const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
-                    f32x4 out4;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int r = 4 * q4 + e;
                         const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
                         const bool kept = !DROPOUT || ((keep >> r) & 1u);
-                        out4[e] = kept ? pv : -pv;             // sign bit = dropped
+                        xo[r] = kept ? pv : -pv;               // sign bit = dropped
                         s_acc[mb][r] = kept ? pv : 0.f;
                     }
-                    *reinterpret_cast<f32x4*>(xw + ((mb * 4 + q4) * 64 + lane) * 16) = out4;
                 }
+                *reinterpret_cast<f16x8*>(xw + ((mb * 2) * 64 + lane) * 16) = pack_acc8<_Float16>(xo, 0);
+                *reinterpret_cast<f16x8*>(xw + ((mb * 2 + 1) * 64 + lane) * 16) = pack_acc8<_Float16>(xo, 8);
                 pf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
                 pf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
             }
@@ -532,16 +535,18 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                 v8 dsf[C::PT];
 #pragma unroll
                 for (int mb = 0; mb < C::MBK; mb++) {
+                    const f16x8 ph[2] = {*reinterpret_cast<const f16x8*>(xr + ((mb * 2) * 64 + lane) * 16),
+                                         *reinterpret_cast<const f16x8*>(xr + ((mb * 2 + 1) * 64 + lane) * 16)};
 #pragma unroll
                     for (int q4 = 0; q4 < 4; q4++) {
-                        const f32x4 p4 = *reinterpret_cast<const f32x4*>(xr + ((mb * 4 + q4) * 64 + lane) * 16);
                         const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const int r = 4 * q4 + e;
+                            const float pv = (float)ph[r >> 3][r & 7];
                             float dpv = dp[mb][r];
-                            if constexpr (DROPOUT) dpv = __builtin_signbit(p4[e]) ? 0.f : dpv * rp;
-                            dp[mb][r] = fabsf(p4[e]) * (dpv - d4[e]);
+                            if constexpr (DROPOUT) dpv = __builtin_signbit(pv) ? 0.f : dpv * rp;
+                            dp[mb][r] = fabsf(pv) * (dpv - d4[e]);
                         }
                     }
                     dsf[2 * mb] = pack_acc8<T>(dp[mb], 0);

@@ -18,12 +18,17 @@ typedef _Float16 InstT;
 #ifndef FA_DQ_BN
 #define FA_DQ_BN (FA_D > 64 ? 32 : 64)
 #endif
+// query rows per dK/dV step: with head dim 64 a 64-row step holds too few products to cover its fixed
+// cost (tile requests, barrier), and the fp16 hand-over leaves room for 128 rows
+#ifndef FA_BWD_BM
+#define FA_BWD_BM (FA_D == 64 ? 128 : 64)
+#endif
 template <bool DROPOUT>
 static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers
     if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, 2, DROPOUT>(kp, stream)) return e;
-    return launch_bwd_dkv3<InstT, FA_D, 64, 1, DROPOUT>(kp, stream);
+    return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 1, DROPOUT>(kp, stream);
 #else
     if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
     return launch_bwd_dkv3<InstT, FA_D, 32, 2, DROPOUT>(kp, stream);
