@@ -213,16 +213,10 @@ static int run_bwd(const fa_bwd_params* p, bool varlen, hipStream_t stream) {
                                p->dq_row_stride, p->dq_head_stride, p->dk_row_stride, p->dk_head_stride,
                                p->dv_row_stride, p->dv_head_stride, p->q_batch_stride, p->k_batch_stride, p->v_batch_stride,
                                p->o_batch_stride, p->do_batch_stride, p->dq_batch_stride, p->dk_batch_stride, p->dv_batch_stride};
-    for (int64_t st : strides) if (st % 4 != 0) return fail("strides must be multiples of 4 elements");
-    const int64_t in_strides[] = {p->q_row_stride, p->q_head_stride, p->k_row_stride, p->k_head_stride, p->v_row_stride,
-                                  p->v_head_stride, p->o_row_stride, p->o_head_stride, p->do_row_stride, p->do_head_stride,
-                                  p->q_batch_stride, p->k_batch_stride, p->v_batch_stride, p->o_batch_stride, p->do_batch_stride};
-    for (int64_t st : in_strides) if (st % 8 != 0) return fail("input strides must be multiples of 8 elements (16-byte rows)");
+    for (int64_t st : strides) if (st % 8 != 0) return fail("strides must be multiples of 8 elements (16-byte rows)");
 
-    const void* in_ptrs[] = {p->dout, p->q, p->k, p->v, p->out};
-    for (const void* q : in_ptrs) if ((uintptr_t)q % 16 != 0) return fail("dout, q, k, v and out must be 16-byte aligned");
-    const void* out_ptrs[] = {p->dq, p->dk, p->dv};
-    for (const void* q : out_ptrs) if ((uintptr_t)q % 8 != 0) return fail("dq, dk and dv must be 8-byte aligned");
+    const void* ptrs[] = {p->dout, p->q, p->k, p->v, p->out, p->dq, p->dk, p->dv};
+    for (const void* q : ptrs) if ((uintptr_t)q % 16 != 0) return fail("dout, q, k, v, out, dq, dk and dv must be 16-byte aligned");
     // the tile movers add a 32-bit lane byte offset (up to 128 rows) to a 64-bit tile base
     const int64_t row_strides[] = {p->q_row_stride, p->k_row_stride, p->v_row_stride, p->do_row_stride};
     for (int64_t st : row_strides) if (st < 0 || st >= ((int64_t)1 << 23)) return fail("row strides must be below 2^23 elements");

@@ -93,7 +93,8 @@ struct BwdDqCfg {
     static constexpr int NB = BN / 32, KS = D / 16, DB = D / 32, PT = BN / 16, CPR = D / 8, ROWB = D * 2;
     static constexpr int TILE_BYTES = BN * ROWB;
     static constexpr int LOADS = BN * CPR / kThreads;
-    static constexpr int SMEM = 4 * TILE_BYTES;   // {K, V} x 2 stages
+    static constexpr int STAGE_BYTES = 32 * (DB * 64 + 16);      // a wave's dQ rows on their way out
+    static constexpr int SMEM = 4 * TILE_BYTES > kWaves * STAGE_BYTES ? 4 * TILE_BYTES : kWaves * STAGE_BYTES;   // {K, V} x 2 stages
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
     static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
 };
@@ -258,20 +259,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
         buf ^= 1;
     }
 
-    if (!row_ok) return;
-    T* orow = reinterpret_cast<T*>(p.dq) + si.dq_off + (int64_t)row * p.dq_row_stride + (int64_t)head * p.dq_head_stride;
-    const float sc = p.softmax_scale;
-#pragma unroll
-    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-            const int d0 = db * 32 + 8 * q4 + 4 * hh;
-            if (d0 < p.d) {
-                u32x2 v = {pack2<T>(dq_acc[db][4 * q4] * sc, dq_acc[db][4 * q4 + 1] * sc),
-                           pack2<T>(dq_acc[db][4 * q4 + 2] * sc, dq_acc[db][4 * q4 + 3] * sc)};
-                st_global8(orow + d0, v);
-            }
-        }
+    // every tile read is behind the loop's last barrier: the ring is free to stage the gradient rows
+    T* obase = reinterpret_cast<T*>(p.dq) + si.dq_off + (int64_t)r0w * p.dq_row_stride + (int64_t)head * p.dq_head_stride;
+    store_tile_rows<T, C::DB>(dq_acc, p.softmax_scale, smem + wave * C::STAGE_BYTES, lane, obase, p.dq_row_stride, si.sq - r0w, p.d);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -303,6 +293,9 @@ struct BwdDkv3Cfg {
     static constexpr int X_OFF = AUX_OFF + 3 * 2 * BM * 4;           // P hand-over: 2 buffers x 4 key blocks
     static constexpr int XBLK = BM * 32 * 2;                         // one key block's P tile, fp16
     static constexpr int SMEM = X_OFF + 2 * 4 * XBLK;
+    // the resident K / V rows come in through LDS where the idle ring stages and the hand-over hold them
+    static constexpr bool STAGED_ROWS = 4 * 32 * ROWB <= 2 * TILE_BYTES && 4 * 32 * ROWB <= 2 * 4 * XBLK;
+    static_assert(kWaves * 32 * (DB * 64 + 16) <= SMEM, "gradient rows are staged in the ring");
     static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
     static_assert(SMEM <= 160 * 1024, "LDS budget");
     static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
@@ -343,24 +336,9 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     const int nt = t_hi - t_lo;
     const int iters = nt * G;
 
-    // resident operand: this lane's key row of K (P wave) or of V (dS wave)
     const int j0w = n0 + kblk * 32;
     const int key = j0w + l32;
     const bool key_ok = key < si.sk;
-    v8 rf[C::KS];
-    {
-        const T* row = role_ds
-            ? reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)key * p.v_row_stride + (int64_t)hk * p.v_head_stride
-            : reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)key * p.k_row_stride + (int64_t)hk * p.k_head_stride;
-#pragma unroll
-        for (int dk = 0; dk < C::KS; dk++) {
-            const int d0 = dk * 16 + 8 * hh;
-            u32x4 a = {0, 0, 0, 0};
-            if (key_ok && d0 < p.d) a = ld_global16(row + d0);
-            rf[dk] = __builtin_bit_cast(v8, a);
-        }
-    }
-    wait_resident_loads();
 
     f32x16 acc[C::DB];      // dV^T (P wave) or dK^T (dS wave) of this wave's keys
 #pragma unroll
@@ -436,6 +414,40 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
         return (has_right && j0w > i0 + BM - 1 + shift + wr) || (has_left && j0w + 31 < i0 + shift - wl) || (j0w >= si.sk);
     };
 
+    // Prologue: the first tile's requests go out first, then the resident operand -- this lane's key
+    // row of K (P wave) or of V (dS wave) -- so that the two latencies overlap.
+    if (iters > 0) load_tile(0, t_lo, 0, 0);
+    v8 rf[C::KS];
+    {
+        const T* blk = role_ds
+            ? reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)n0 * p.v_row_stride + (int64_t)hk * p.v_head_stride
+            : reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)n0 * p.k_row_stride + (int64_t)hk * p.k_head_stride;
+        const int rs = (int)(role_ds ? p.v_row_stride : p.k_row_stride);
+        if constexpr (C::STAGED_ROWS) {
+            // through a wave-private piece of LDS that the ring does not use before the first barrier
+            // (K rows: Q stages 1 and 2, V rows: the P hand-over); keys past the sequence repeat its
+            // last key: whatever a lane computes for such a key stays in that lane and is never written
+            const int region = (role_ds ? C::X_OFF : C::Q_OFF + C::TILE_BYTES) + kblk * 32 * C::ROWB;
+            const int last = si.sk - 1 - n0;
+            stage_rows_issue<T, D>(blk, [&](int r) { return min(kblk * 32 + r, last) * rs; }, p.d,
+                                   (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)region)), lane);
+            wait_vmcnt<0>();
+            stage_rows_read<T, D>(rf, smem + region, p.d, lane);
+        } else {
+            const T* row = blk + (int64_t)(kblk * 32 + l32) * rs;
+#pragma unroll
+            for (int dk = 0; dk < C::KS; dk++) {
+                const int d0 = dk * 16 + 8 * hh;
+                u32x4 a = {0, 0, 0, 0};
+                if (key_ok && d0 < p.d) a = ld_global16(row + d0);
+                rf[dk] = __builtin_bit_cast(v8, a);
+            }
+        }
+    }
+    wait_resident_loads();
+    if (iters > 0) finish_tile(0, t_lo);
+    __syncthreads();
+
     const float sl2 = kp.scale_log2;
     const int rel_hi = has_right ? shift + wr : 0x3fffffff;
     const int rel_lo = has_left ? shift - wl : -0x3fffffff;
@@ -445,8 +457,6 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     // The tile walk shared by both kinds of wave; `body(it, i0, g, live, prev_live, q3, q3_prev)` is the
     // wave's own work of one step.  iters + 1 steps: the last one drains the dS wave's final tile.
     auto walk = [&](auto&& body) {
-        if (iters > 0) { load_tile(0, t_lo, 0, 0); finish_tile(0, t_lo); }
-        __syncthreads();
         int q3 = 0, q3_prev = 0;                     // Q / aux ring slots of the current and the previous tile
         int cur_t = t_lo, cur_g = 0, nxt_g = 0, nxt_t = t_lo;
         bool prev_live = false;                      // the previous tile was not skipped (its P is in the hand-over)
@@ -560,22 +570,13 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
             }
         });
     }
-
-    if (!key_ok) return;
-    T* orow = role_ds ? reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)key * p.dk_row_stride + (int64_t)hk * p.dk_head_stride
-                      : reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)key * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
+    // every tile read is behind the loop's last barrier: the ring is free to stage the gradient rows
+    T* obase = role_ds ? reinterpret_cast<T*>(p.dk) + si.dk_off + (int64_t)j0w * p.dk_row_stride + (int64_t)hk * p.dk_head_stride
+                       : reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)j0w * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
     const float sc = role_ds ? p.softmax_scale : (DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f);
-#pragma unroll
-    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-            const int d0 = (dpart * C::DB + db) * 32 + 8 * q4 + 4 * hh;
-            if (d0 < p.d) {
-                u32x2 a = {pack2<T>(acc[db][4 * q4] * sc, acc[db][4 * q4 + 1] * sc),
-                           pack2<T>(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc)};
-                st_global8(orow + d0, a);
-            }
-        }
+    const int col0 = dpart * C::DB * 32;
+    store_tile_rows<T, C::DB>(acc, sc, smem + wave * (32 * (C::DB * 64 + 16)), lane, obase + col0,
+                              role_ds ? p.dk_row_stride : p.dv_row_stride, si.sk - j0w, p.d - col0);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -360,6 +360,64 @@ template <int N> FA_DEV void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));
 }
 
+// A wave's 32 resident rows (each lane keeps one row in registers as MFMA operand) fetched through a
+// wave-private LDS region of 32 * D * 2 bytes instead of 16 B per lane from 32 different rows: the
+// fills are whole 1 KB runs, so the memory system sees 64-byte requests instead of 32 row pieces per
+// instruction.  `base` is uniform; row r of the wave is at element offset row_off(r) from it (the
+// caller clamps rows past the sequence).  stage_rows_issue only requests; after the wave's vmcnt has
+// drained, stage_rows_read hands every lane its row with columns >= d zeroed.
+template <typename T, int D, typename RowOff>
+FA_DEV void stage_rows_issue(const T* base, RowOff row_off, int d, uint32_t lds_region, int lane) {
+    constexpr int ROWB = D * 2;
+    const int d_last_chunk = d / 8 - 1;
+#pragma unroll
+    for (int j = 0; j < ROWB / 32; j++) {
+        const int pos = j * 1024 + lane * 16;
+        const int r = pos / ROWB;
+        const int c = min(swz_u<D>((pos % ROWB) / 16, r), d_last_chunk);
+        async_fill16(base, ((uint32_t)row_off(r) + (uint32_t)(c * 8)) * 2u, lds_region + j * 1024);
+    }
+}
+template <typename T, int D>
+FA_DEV void stage_rows_read(typename Elem<T>::v8 (&rf)[D / 16], const char* region, int d, int lane) {
+    typedef typename Elem<T>::v8 v8;
+    const int l32 = lane & 31, hh = lane >> 5;
+    asm volatile("" ::: "memory");     // the region was written by the fills, not by anything the compiler saw
+#pragma unroll
+    for (int dk = 0; dk < D / 16; dk++) {
+        u32x4 a = *reinterpret_cast<const u32x4*>(region + l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16);
+        if (dk * 16 + 8 * hh >= d) a = u32x4{0, 0, 0, 0};
+        rf[dk] = __builtin_bit_cast(v8, a);
+    }
+}
+
+// A wave's 32 x (32 DB) accumulator tile (lane l32 = row, registers = columns) to global memory
+// through a wave-private LDS region of 32 * (64 DB + 16) bytes, so that every store instruction
+// writes whole rows, 16 B per lane, instead of 8-byte pieces of 32 rows.  `base` points at row 0,
+// column 0 of the tile; rows >= rows_ok and columns >= cols_ok are not written.
+template <typename T, int DB>
+FA_DEV void store_tile_rows(const f32x16 (&acc)[DB], float sc, char* stage, int lane, T* base, int64_t row_stride,
+                            int rows_ok, int cols_ok) {
+    constexpr int PITCH = DB * 64 + 16, CPR = DB * 4, RPP = 64 / CPR;
+    const int l32 = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const int d0 = db * 32 + 8 * q4 + 4 * hh;
+            const u32x2 v = {pack2<T>(acc[db][4 * q4] * sc, acc[db][4 * q4 + 1] * sc),
+                             pack2<T>(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc)};
+            *reinterpret_cast<u32x2*>(stage + l32 * PITCH + d0 * 2) = v;
+        }
+    const int srow = lane / CPR, sch = lane % CPR;
+#pragma unroll
+    for (int j = 0; j < 32 / RPP; j++) {
+        const int rr = j * RPP + srow;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
+        if (rr < rows_ok && sch * 8 < cols_ok) st_global16(base + (int64_t)rr * row_stride + sch * 8, v);
+    }
+}
+
 // Resolved per-(batch) sequence bookkeeping.  Mirrors the reference's BlockInfo
 // (csrc/flash_attn/src/block_info.h:11-42) with 64-bit offsets.
 struct SeqInfo {
