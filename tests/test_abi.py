@@ -64,7 +64,11 @@ def test_backward_argument_errors_do_not_abort(lib):
     assert lib.fa_varlen_bwd(ctypes.byref(p), None) != 0 and b"cu_seqlens" in lib.fa_last_error()
     p.q_row_stride = 4
     assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"strides" in lib.fa_last_error()
-    p.q_row_stride, p.p_dropout = 0, 0.1
+    p.q_row_stride, p.dk_row_stride = 0, 4     # gradients leave 16 bytes per lane as well
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"strides" in lib.fa_last_error()
+    p.dk_row_stride, p.dv = 0, 24
+    assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"16-byte aligned" in lib.fa_last_error()
+    p.dv, p.p_dropout = 16, 0.1
     assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"rng_state" in lib.fa_last_error()
     p.p_dropout = 1.0
     assert lib.fa_bwd(ctypes.byref(p), None) != 0 and b"p_dropout" in lib.fa_last_error()
