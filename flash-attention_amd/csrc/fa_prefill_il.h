@@ -87,7 +87,7 @@ struct ILCfgPair {
     static_assert((BN * CPR) % kThreads == 0, "tile shape");
 };
 
-template <typename T, typename C>
+template <typename T, typename C, bool DROPOUT = false>
 __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParams kp) {
     constexpr int D = C::D, BN = C::BN;
     typedef typename Elem<T>::v8 v8;
@@ -152,6 +152,10 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
 #pragma unroll
         for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
+    // dropout: the row sums are of the undropped probabilities; dropped entries leave the second
+    // product only, and 1 / (1 - p) is applied once in the epilogue
+    Drop drop = {0, 0, 256, 1.f};
+    if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
     const float sl2 = kp.scale_log2;
 
     // visit i of the key loop handles key tile t_hi - 1 - i and uses ring slot i % NS
@@ -307,7 +311,10 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
                 }
         }
     };
-    auto probs = [&](const f32x16 (&s)[C::NB], v8 (&pf)[C::PT], float& corr_out, bool& move_out, float sl2) __attribute__((always_inline)) {
+    auto probs = [&](int i, const f32x16 (&s)[C::NB], v8 (&pf)[C::PT], float& corr_out, bool& move_out, float sl2) __attribute__((always_inline)) {
+        uint32_t keep[C::NB];
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++) keep[nb] = DROPOUT ? drop_keep16_row(drop, row, tile_of(i) * C::BN + nb * 32, hh) : 0xffffu;
         float mx = -INFINITY;
 #pragma unroll
         for (int nb = 0; nb < C::NB; nb++)
@@ -331,7 +338,10 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
                 const float e1 = fast_exp2(s[nb][r8 + 2 * e + 1] * sl2 - msc);
                 suma += e0;
                 sumb += e1;
-                pk[e] = pack2<T>(e0, e1);
+                if constexpr (DROPOUT)
+                    pk[e] = pack2<T>((keep[nb] >> (r8 + 2 * e)) & 1u ? e0 : 0.f, (keep[nb] >> (r8 + 2 * e + 1)) & 1u ? e1 : 0.f);
+                else
+                    pk[e] = pack2<T>(e0, e1);
             }
             pf[t16] = __builtin_bit_cast(v8, pk);
         }
@@ -443,6 +453,9 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
         float mx = -INFINITY, msc = 0.f, corr = 1.f, suma = 0.f, sumb = 0.f;
         bool move = false;
         uint32_t pk[NP];
+        uint32_t keep[C::NB];
+#pragma unroll
+        for (int nb = 0; nb < C::NB; nb++) keep[nb] = DROPOUT ? drop_keep16_row(drop, row, tile_of(i) * C::BN + nb * 32, hh) : 0xffffu;
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             // ---- matrix instruction f and the read for f + LA
@@ -482,7 +495,11 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
                         const float e1 = fast_exp2(s_cur[(2 * pr + 1) / 16][(2 * pr + 1) % 16] * sc - msc);
                         suma += e0;
                         sumb += e1;
-                        pk[pr] = pack2<T>(e0, e1);
+                        if constexpr (DROPOUT)
+                            pk[pr] = pack2<T>((keep[(2 * pr) / 16] >> ((2 * pr) % 16)) & 1u ? e0 : 0.f,
+                                              (keep[(2 * pr + 1) / 16] >> ((2 * pr + 1) % 16)) & 1u ? e1 : 0.f);
+                        else
+                            pk[pr] = pack2<T>(e0, e1);
                     }
                 }
             }
@@ -514,7 +531,7 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
         }
         mask_tile(i, sA);
         float corr; bool move;
-        probs(sA, pA, corr, move, sl2);
+        probs(i, sA, pA, corr, move, sl2);
         rescale(corr, move);
 #pragma unroll
         for (int nb = 0; nb < C::NB; nb++) sA[nb] = sB[nb];
@@ -549,7 +566,7 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
     // ---- epilogue
     const float l_tot = xhalf_sum(l_run);
     const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
-    const float inv = dead ? 1.f : 1.f / l_tot;
+    const float inv = dead ? 1.f : drop.rp / l_tot;
     const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
     if (hh == 0 && dcol0 == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
     // output tile of the wave (32 rows x DH columns) through LDS (whole rows per store instruction); all ring reads are
@@ -580,21 +597,25 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
     }
 }
 
-template <typename T, typename C>
-int launch_prefill_il_cfg(KParams kp, hipStream_t stream) {
+template <typename T, typename C, bool DROPOUT>
+int launch_prefill_il_one(KParams kp, hipStream_t stream) {
     kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
     if (total <= 0) return 0;
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
     dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
-    auto kern = prefill_il_kernel<T, C>;
+    auto kern = prefill_il_kernel<T, C, DROPOUT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
 
+template <typename T, typename C>
+int launch_prefill_il_cfg(const KParams& kp, hipStream_t stream) {
+    return kp.p.p_dropout > 0.f ? launch_prefill_il_one<T, C, true>(kp, stream) : launch_prefill_il_one<T, C, false>(kp, stream);
+}
 template <typename T, int D, int BN>
 int launch_prefill_il(const KParams& kp, hipStream_t stream) { return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream); }
 template <typename T>

@@ -23,8 +23,7 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     //  * otherwise from 512 query rows on: the software-pipelined kernel, two independent
     //    128-row workgroups per CU, whose start-up and output phases overlap.
     // Shorter sequences, split key ranges and q rotary take the general 4-wave kernel.
-    // Dropout runs on the general kernel.
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512 && kp.p.p_dropout == 0.f) {
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) {
         const bool masked = kp.has_right || kp.has_left;
         const bool long_keys = kp.p.seqlen_k > (masked ? 4096 : 2048);
         if (FA_D >= 128 && long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
@@ -32,7 +31,7 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     }
 #else
     // head dim 129..256: pairs of waves split the head dimension (fa_prefill_il.h)
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512 && kp.p.p_dropout == 0.f) return launch_prefill_il_pair<InstT>(kp, stream);
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) return launch_prefill_il_pair<InstT>(kp, stream);
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }

@@ -53,7 +53,7 @@ struct PPCfg {
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
-template <typename T, int D, int BN>
+template <typename T, int D, int BN, bool DROPOUT = false>
 __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     typedef PPCfg<T, D, BN> C;
     typedef typename Elem<T>::v8 v8;
@@ -120,6 +120,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     const float sl2 = kp.scale_log2;
+    Drop drop = {0, 0, 256, 1.f};
+    if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
 
     // visit i of the key loop handles key tile tile_of(i) and uses ring slot i % NS
 #ifdef FA_PP_ASCENDING
@@ -314,6 +316,16 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
                 sumb += e1;
             }
         l_run += suma + sumb;
+        if constexpr (DROPOUT) {
+            // the row sum is of the undropped probabilities; dropped entries leave the second product
+            // only, and 1 / (1 - p) is applied once in the epilogue
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++) {
+                const uint32_t keep = drop_keep16_row(drop, row, tt * BN + nb * 32, hh);
+#pragma unroll
+                for (int r = 0; r < 16; r++) s_acc[nb][r] = (keep >> r) & 1u ? s_acc[nb][r] : 0.f;
+            }
+        }
 #pragma unroll
         for (int t16 = 0; t16 < C::PT; t16++) {
             const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
@@ -358,7 +370,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     // ---- epilogue
     const float l_tot = xhalf_sum(l_run);
     const bool dead = (l_tot == 0.f) || (l_tot != l_tot);
-    const float inv = dead ? 1.f : 1.f / l_tot;
+    const float inv = dead ? 1.f : drop.rp / l_tot;
     const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
     if (hh == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
     // The output tile of the wave (32 rows x D) goes through LDS so that every store instruction
@@ -389,8 +401,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     }
 }
 
-template <typename T, int D, int BN>
-int launch_prefill_pp(KParams kp, hipStream_t stream) {
+template <typename T, int D, int BN, bool DROPOUT>
+int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     typedef PPCfg<T, D, BN> C;
     kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
@@ -398,11 +410,15 @@ int launch_prefill_pp(KParams kp, hipStream_t stream) {
     const int64_t per_xcd = (total + 7) / 8;
     if (per_xcd * 8 > 0x7fffffffLL) return -2;
     dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
-    auto kern = prefill_pp_kernel<T, D, BN>;
+    auto kern = prefill_pp_kernel<T, D, BN, DROPOUT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     return (int)hipGetLastError();
+}
+template <typename T, int D, int BN>
+int launch_prefill_pp(const KParams& kp, hipStream_t stream) {
+    return kp.p.p_dropout > 0.f ? launch_prefill_pp_one<T, D, BN, true>(kp, stream) : launch_prefill_pp_one<T, D, BN, false>(kp, stream);
 }
 
 }  // namespace fa

@@ -87,10 +87,11 @@ def test_dropout_forward_backward(sq, sk, d, mode, dtype):
     _check_all(out, lse, S, grads, q, k, v, dout, p, mode == "causal", window)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 256])
 @pytest.mark.parametrize("p", [0.1, 0.5])
-def test_dropout_long_sequences_use_general_kernel(d, p):
-    """Lengths that without dropout take the long-sequence kernels."""
+def test_dropout_on_the_long_sequence_kernels(d, p):
+    """From 512 query rows on the forward runs on the software-pipelined kernels (pairs of waves at
+    head dim 256), which walk the score matrix in steps of their own."""
     _say("dropout long", d, p)
     dtype, b, h, s = torch.bfloat16, 1, 4, 1100
     q = _gen((b, s, h, d), dtype, 1); k = _gen((b, s, h, d), dtype, 2); v = _gen((b, s, h, d), dtype, 3)
@@ -99,6 +100,23 @@ def test_dropout_long_sequences_use_general_kernel(d, p):
     out, lse, S = _fa().flash_attn_func(qd, kd, vd, dropout_p=p, causal=True, return_attn_probs=True)
     grads = torch.autograd.grad(out, (qd, kd, vd), dout.to(DEV))
     _check_all(out, lse, S, grads, q, k, v, dout, p, True, (-1, -1))
+
+
+@pytest.mark.parametrize("sq,sk,d,mode,dtype", [(640, 2300, 128, "full", torch.bfloat16), (600, 4200, 96, "causal", torch.float16),
+                                                  (1030, 4300, 128, "local", torch.bfloat16)])
+def test_dropout_on_the_long_key_kernel(sq, sk, d, mode, dtype):
+    """Key lengths past 2048 (full) / 4096 (masked) at head dim 65..128 take the 8-wave kernel, which
+    applies the mask in its own register geometry (one query row per lane)."""
+    _say("dropout long keys", sq, sk, d, mode, dtype)
+    b, h, hk, p = 1, 4, 2, 0.17
+    q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
+    dout = _gen((b, sq, h, d), dtype, 4)
+    window = (1500, 300) if mode == "local" else (-1, -1)
+    qd, kd, vd = [t.to(DEV).requires_grad_() for t in (q, k, v)]
+    out, lse, S = _fa().flash_attn_func(qd, kd, vd, dropout_p=p, causal=(mode == "causal"), window_size=window,
+                                        return_attn_probs=True)
+    grads = torch.autograd.grad(out, (qd, kd, vd), dout.to(DEV))
+    _check_all(out, lse, S, grads, q, k, v, dout, p, mode == "causal", window)
 
 
 def test_dropout_qkvpacked_and_varlen():
