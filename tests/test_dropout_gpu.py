@@ -105,7 +105,7 @@ def test_dropout_on_the_long_sequence_kernels(d, p):
 @pytest.mark.parametrize("sq,sk,d,mode,dtype", [(640, 2300, 128, "full", torch.bfloat16), (600, 4200, 96, "causal", torch.float16),
                                                   (1030, 4300, 128, "local", torch.bfloat16)])
 def test_dropout_on_the_long_key_kernel(sq, sk, d, mode, dtype):
-    """Key lengths past 2048 (full) / 4096 (masked) at head dim 65..128 take the 8-wave kernel, which
+    """Key lengths past 768 (full) / 2048 (masked) at head dim 65..128 take the 8-wave kernel, which
     applies the mask in its own register geometry (one query row per lane)."""
     _say("dropout long keys", sq, sk, d, mode, dtype)
     b, h, hk, p = 1, 4, 2, 0.17
