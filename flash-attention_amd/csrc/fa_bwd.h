@@ -232,13 +232,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
                 f32x16 s_acc[1], dp_acc[1];
                 product_rows<T, D, 1, C::KS, 4>(s_acc, kb + nb * 32 * C::ROWB, lo.r, qf);
                 product_rows<T, D, 1, C::KS, 4>(dp_acc, vb + nb * 32 * C::ROWB, lo.r, gf);
-                if (need_mask) {
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-                        if (n > lim_hi || n < lim_lo) s_acc[0][r] = -INFINITY;
-                    }
-                }
+                if (need_mask) mask_acc16(s_acc[0], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
                 uint32_t keep = 0xffffu;
                 if constexpr (DROPOUT) keep = drop_keep16_row(drop, row, n0 + nb * 32, hh);
 #pragma unroll
@@ -499,12 +493,9 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                 const int ib = i0 + mb * 32;
                 const bool need_mask = (has_right && j0w + 31 > ib + shift + wr) || (has_left && j0w < ib + 31 + shift - wl);
                 if (need_mask) {
+                    // entry r is query row ib + 4 hh + c_r, visible iff rel_lo + c_r <= key - ib - 4 hh <= rel_hi + c_r
                     const int rel = key - ib - 4 * hh;
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int c_r = 8 * (r >> 2) + (r & 3);
-                        s_acc[mb][r] = (rel > rel_hi + c_r || rel < rel_lo + c_r) ? -INFINITY : s_acc[mb][r];
-                    }
+                    mask_acc16(s_acc[mb], 0, rel - rel_hi, rel - rel_lo);
                 }
                 uint32_t keep = 0xffffu;
                 if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);

@@ -245,6 +245,17 @@ template <typename T> FA_DEV void mfma_step(f32x16& acc, typename Elem<T>::v8 a,
     acc = Elem<T>::mfma32(a, b, dk == 0 ? zero : acc);
 }
 
+// Mask of one 32-wide accumulator block: entry r of the lane stands at position
+// pos0 + 8 * (r >> 2) + (r & 3) (pos0 includes the lane's 4 * hh) and is visible iff lo <= position <= hi.
+// One add, one unsigned compare and one select per entry; hi < lo masks everything.
+FA_DEV void mask_acc16(f32x16& s, int pos0, int lo, int hi) {
+    const bool any = hi >= lo;
+    const uint32_t span = any ? (uint32_t)(hi - lo) : 0u;
+    const int z = any ? pos0 - lo : -64;
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[r] = (uint32_t)(z + (8 * (r >> 2) + (r & 3))) > span ? -INFINITY : s[r];
+}
+
 // accumulator registers [r8, r8+8) -> B operand of the next product
 template <typename T> FA_DEV typename Elem<T>::v8 pack_acc8(const f32x16& a, int r8) {
     u32x4 pk;

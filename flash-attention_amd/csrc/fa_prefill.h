@@ -210,12 +210,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                     if (has_right) lim_hi = min(lim_hi, row + shift + wr);
                     const int lim_lo = has_left ? row + shift - wl : 0;
 #pragma unroll
-                    for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-                            if (n > lim_hi || n < lim_lo) s_acc[rb][nb][r] = -INFINITY;
-                        }
+                    for (int nb = 0; nb < C::NB; nb++) mask_acc16(s_acc[rb][nb], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
                 }
                 float mx = -INFINITY;
 #pragma unroll

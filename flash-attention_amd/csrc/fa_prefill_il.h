@@ -303,12 +303,7 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
             if (has_right) lim_hi = min(lim_hi, row + shift + wr);
             const int lim_lo = has_left ? row + shift - wl : 0;
 #pragma unroll
-            for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int n = n0 + nb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
-                    if (n > lim_hi || n < lim_lo) s[nb][r] = -INFINITY;
-                }
+            for (int nb = 0; nb < C::NB; nb++) mask_acc16(s[nb], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
         }
     };
     auto probs = [&](int i, const f32x16 (&s)[C::NB], v8 (&pf)[C::PT], float& corr_out, bool& move_out, float sl2) __attribute__((always_inline)) {
@@ -561,6 +556,7 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
         }
         for (; i < nt; i++) plain_step(i);
         mma(std::true_type(), std::false_type(), nt - 1, 0, pA, sB);
+        __syncthreads();      // the output staging below reuses the ring this product has just read
     }
 
     // ---- epilogue
@@ -570,7 +566,7 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
     const float lse = dead ? INFINITY : m_run * p.softmax_scale + __logf(l_tot);
     if (hh == 0 && dcol0 == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
     // output tile of the wave (32 rows x DH columns) through LDS (whole rows per store instruction); all ring reads are
-    // behind the last barrier and each wave uses its own region
+    // behind the barrier that follows the last product and each wave uses its own region
     {
         constexpr int PITCH = C::DH * 2 + 16;
         constexpr int OCPR = C::DH / 8;                 // 16 B chunks per output row of the wave
