@@ -419,6 +419,7 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
         static_assert(NF > CE + 1, "tile too small for the chunked step");
         open_step(i);
         xch_read_add(i, s_cur);
+        if constexpr (!C::kPair) mask_tile(i, s_cur);
         // an opaque copy of the scale keeps the vector work in this block (behind the barrier)
         float sc = sl2;
         asm volatile("" : "+v"(sc));
@@ -543,9 +544,12 @@ __global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParam
         xch_write(0, sA);
         __syncthreads();      // K(0)'s ring slot is refilled when step 0 opens
 
-        // steps [i_fb, i_fe) visit tiles that need no masking for this wave, an even number of them
-        int i_fb = max(1, t_hi - 1 - tf_hi);
-        int i_fe = min(nt - 1, t_hi - tf_lo);
+        // Steps [i_fb, i_fe), an even number of them, take the chunked form.  With the whole head
+        // dimension in one wave that is every step but the first and the last (the mask is applied on
+        // the way in); in pair mode only the tiles that need no masking for this wave (measured: the
+        // masked tiles are faster there as plain steps).
+        int i_fb = C::kPair ? max(1, t_hi - 1 - tf_hi) : 1;
+        int i_fe = C::kPair ? min(nt - 1, t_hi - tf_lo) : nt - 1;
         i_fb = __builtin_amdgcn_readfirstlane(min(i_fb, nt));
         i_fe = __builtin_amdgcn_readfirstlane(i_fe <= i_fb ? i_fb : i_fb + ((i_fe - i_fb) & ~1));
         int i = 0;
