@@ -55,7 +55,7 @@ def test_dense_basic(dtype, d, causal):
 
 
 def test_config1_fp16_dense():
-    """BASELINE config 1: fp16, batch 2, seqlen 512, 8 heads, headdim 64, non-causal."""
+    """The smallest benchmark configuration: fp16, batch 2, seqlen 512, 8 heads, headdim 64, non-causal."""
     _say("config1")
     torch.manual_seed(0)
     q, k, v = (_gen((2, 512, 8, 64), torch.float16, i) for i in (1, 2, 3))
