@@ -87,8 +87,11 @@ struct ILCfgPair {
     static_assert((BN * CPR) % kThreads == 0, "tile shape");
 };
 
+// Occupancy: two workgroups per CU at head dim 128 (about 250 registers); at head dim 64, where the
+// vector work per matrix instruction doubles and a third wave per SIMD adds the issue slots it needs,
+// three workgroups in 168 registers each (measured +3..10 %).
 template <typename T, typename C, bool DROPOUT = false>
-__global__ void __launch_bounds__(C::kThreads, 2) prefill_il_kernel(const KParams kp) {
+__global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2) prefill_il_kernel(const KParams kp) {
     constexpr int D = C::D, BN = C::BN;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
