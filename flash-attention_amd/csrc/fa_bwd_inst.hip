@@ -26,8 +26,9 @@ typedef _Float16 InstT;
 template <bool DROPOUT>
 static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
-    // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers
-    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, 2, DROPOUT>(kp, stream)) return e;
+    // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers;
+    // three at head dim 64 (168 registers), where the vector work per matrix instruction doubles
+    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, (FA_D == 64 ? 3 : 2), DROPOUT>(kp, stream)) return e;
     return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 1, DROPOUT>(kp, stream);
 #else
     if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
