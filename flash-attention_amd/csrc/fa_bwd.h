@@ -401,7 +401,9 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
         wait_vmcnt<0>();
         if (tid < 2 * BM) {
             const bool in_range = t * BM + aux_row < si.sq;   // rows past the end: lse = +inf => P = 0
-            reinterpret_cast<float*>(smem + C::AUX_OFF + q3 * 2 * BM * 4)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? aux : 0.f);
+            // D goes in negated where the dS wave starts dP from it (dS = P o (dP - D) without a subtraction)
+            const float dval = DROPOUT ? aux : -aux;
+            reinterpret_cast<float*>(smem + C::AUX_OFF + q3 * 2 * BM * 4)[tid] = tid < BM ? (in_range ? aux * kLog2e : INFINITY) : (in_range ? dval : 0.f);
         }
     };
     auto skip_tile = [&](int i0) {   // keys of this wave against the rows of a tile: nothing visible
@@ -526,7 +528,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
         for (int mb = 0; mb < C::MBK; mb++)
 #pragma unroll
             for (int r = 0; r < 16; r++) dp[mb][r] = 0.f;
-        walk([&](int it, int, int, bool live, bool prev_live, int, int q3_prev) {
+        walk([&](int it, int, int, bool live, bool prev_live, int q3, int q3_prev) {
             // first the previous tile (consumes dp), then dP of this tile into the same registers
             if (prev_live) {
                 const char* qp = smem + C::Q_OFF + q3_prev * C::TILE_BYTES;
@@ -538,17 +540,22 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                 for (int mb = 0; mb < C::MBK; mb++) {
                     const f16x8 ph[2] = {*reinterpret_cast<const f16x8*>(xr + ((mb * 2) * 64 + lane) * 16),
                                          *reinterpret_cast<const f16x8*>(xr + ((mb * 2 + 1) * 64 + lane) * 16)};
+                    if constexpr (DROPOUT) {
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
+                        for (int q4 = 0; q4 < 4; q4++) {
+                            const f32x4 d4 = *reinterpret_cast<const f32x4*>(dsum_s + mb * 32 + 8 * q4 + 4 * hh);
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const int r = 4 * q4 + e;
-                            const float pv = (float)ph[r >> 3][r & 7];
-                            float dpv = dp[mb][r];
-                            if constexpr (DROPOUT) dpv = __builtin_signbit(pv) ? 0.f : dpv * rp;
-                            dp[mb][r] = fabsf(pv) * (dpv - d4[e]);
+                            for (int e = 0; e < 4; e++) {
+                                const int r = 4 * q4 + e;
+                                const float pv = (float)ph[r >> 3][r & 7];
+                                const float dpv = __builtin_signbit(pv) ? 0.f : dp[mb][r] * rp;
+                                dp[mb][r] = fabsf(pv) * (dpv - d4[e]);
+                            }
                         }
+                    } else {
+                        // dp already holds dP - D: the product below started from -D
+#pragma unroll
+                        for (int r = 0; r < 16; r++) dp[mb][r] *= (float)ph[r >> 3][r & 7];
                     }
                     dsf[2 * mb] = pack_acc8<T>(dp[mb], 0);
                     dsf[2 * mb + 1] = pack_acc8<T>(dp[mb], 8);
@@ -557,7 +564,21 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
             }
             if (live) {
                 const char* gb = smem + C::G_OFF + (it & 1) * C::TILE_BYTES;
-                product_rows<T, D, C::MBK, C::KS, 4>(dp, gb, lo.r, rf);
+                if constexpr (DROPOUT) {
+                    product_rows<T, D, C::MBK, C::KS, 4>(dp, gb, lo.r, rf);
+                } else {
+                    // dP - D in one go: the accumulators start from -D of their rows (entry r of a lane
+                    // is row 8 (r >> 2) + 4 hh + (r & 3) of its block)
+                    const float* nd = reinterpret_cast<const float*>(smem + C::AUX_OFF + q3 * 2 * BM * 4) + BM;
+#pragma unroll
+                    for (int mb = 0; mb < C::MBK; mb++)
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; q4++) {
+                            const f32x4 d4 = *reinterpret_cast<const f32x4*>(nd + mb * 32 + 8 * q4 + 4 * hh);
+                            dp[mb][4 * q4] = d4[0]; dp[mb][4 * q4 + 1] = d4[1]; dp[mb][4 * q4 + 2] = d4[2]; dp[mb][4 * q4 + 3] = d4[3];
+                        }
+                    product_rows<T, D, C::MBK, C::KS, 4, false>(dp, gb, lo.r, rf);
+                }
             }
         });
     }

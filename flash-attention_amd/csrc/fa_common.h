@@ -301,7 +301,8 @@ template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_cols_at(const char*
 // MFMA, read, wait, MFMA ... with one operand register set, and every MFMA pays an LDS round trip.)
 //
 // acc[blk] (+)= rows [32 blk, 32 blk + 32) of `tile`  x  bfrag[dk]   for blk < NBLK, dk < KS
-template <typename T, int D, int NBLK, int KS, int GRP>
+// (ZERO0 = false: the accumulators already hold the value the product is added to.)
+template <typename T, int D, int NBLK, int KS, int GRP, bool ZERO0 = true>
 FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const typename Elem<T>::v8* bfrag) {
     typedef typename Elem<T>::v8 v8;
     constexpr int TOTAL = NBLK * KS, NG = TOTAL / GRP;
@@ -323,7 +324,7 @@ FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const t
 #pragma unroll
         for (int j = 0; j < GRP; j++) {
             const int st = g * GRP + j;
-            mfma_step<T>(acc[st % NBLK], a[g & 1][j], bfrag[st / NBLK], st / NBLK);
+            mfma_step<T>(acc[st % NBLK], a[g & 1][j], bfrag[st / NBLK], ZERO0 ? st / NBLK : 1);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
