@@ -79,7 +79,7 @@ __global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp) {
     const int hk = (int)((idx / cpr) % p.h_k);
     const int t = (int)((idx / ((int64_t)cpr * p.h_k)) % p.seqlen_knew);
     const int b = (int)(idx / ((int64_t)cpr * p.h_k * p.seqlen_knew));
-    const int len = p.cu_seqlens_k ? p.cu_seqlens_k[b] : p.seqlen_k;
+    const int len = p.cu_seqlens_k ? min(max(p.cu_seqlens_k[b], 0), p.seqlen_k) : p.seqlen_k;
     const int pos = len + t;
     if (pos >= p.seqlen_k) return;     // never write past the cache capacity
     const int bk = p.cache_batch_idx ? p.cache_batch_idx[b] : b;

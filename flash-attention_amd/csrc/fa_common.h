@@ -457,8 +457,10 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
         s.v_off = (int64_t)r0 * p.v_row_stride;
     } else {
         const int bk = p.cache_batch_idx ? p.cache_batch_idx[b] : b;
-        s.sk_cache = p.cu_seqlens_k ? p.cu_seqlens_k[b] : p.seqlen_k;
-        s.sk = s.sk_cache + p.seqlen_knew;
+        // a cache length outside [0, capacity] is a caller error; clamped so that no key, rotary
+        // table row or appended row beyond the cache is ever touched
+        s.sk_cache = p.cu_seqlens_k ? min(max(p.cu_seqlens_k[b], 0), p.seqlen_k) : p.seqlen_k;
+        s.sk = min(s.sk_cache + p.seqlen_knew, p.seqlen_k);
         s.k_off = (int64_t)bk * p.k_batch_stride;
         s.v_off = (int64_t)bk * p.v_batch_stride;
     }

@@ -266,6 +266,30 @@ def test_kvcache_int_seqlens_and_no_seqlens():
     assert orc.tolerance_ok(out.cpu(), o_ref, o_pt, 3.0, 1e-5)[0]
 
 
+@pytest.mark.parametrize("seqlen_q", [1, 40])
+def test_kvcache_lengths_outside_the_cache_are_clamped(seqlen_q):
+    """cache_seqlens beyond the capacity or negative are a caller error the reference does not check
+    (flash_attn_interface.py:944-946).  Here they are clamped to [0, capacity]: no key, table row or
+    appended row outside the cache is touched, and the result is that of the clamped lengths."""
+    _say("kvcache_clamped", seqlen_q)
+    dtype, d, cap = torch.float16, 64, 300
+    q = _gen((2, seqlen_q, 4, d), dtype, 1); kc = _gen((2, cap, 2, d), dtype, 2); vc = _gen((2, cap, 2, d), dtype, 3)
+    fa = _fa()
+    bad = torch.tensor([cap + 100, -5], dtype=torch.int32)
+    good = torch.tensor([cap, 0], dtype=torch.int32)
+    out_bad = fa.flash_attn_with_kvcache(q.to(DEV), kc.to(DEV), vc.to(DEV), cache_seqlens=bad.to(DEV))
+    out_good = fa.flash_attn_with_kvcache(q.to(DEV), kc.to(DEV), vc.to(DEV), cache_seqlens=good.to(DEV))
+    assert torch.equal(out_bad, out_good)
+    assert torch.equal(out_bad[1], torch.zeros_like(out_bad[1]))          # no visible key
+    # with one new token: nothing is appended past the capacity, row 0 of the empty sequence is
+    kn = _gen((2, 1, 2, d), dtype, 4); vn = _gen((2, 1, 2, d), dtype, 5)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    out = fa.flash_attn_with_kvcache(q[:, :1].to(DEV), kc_d, vc_d, k=kn.to(DEV), v=vn.to(DEV), cache_seqlens=bad.to(DEV))
+    assert torch.equal(kc_d[0].cpu(), kc[0]) and torch.equal(vc_d[0].cpu(), vc[0])
+    assert torch.equal(vc_d[1, 0].cpu(), vn[1, 0]) and torch.equal(vc_d[1, 1:].cpu(), vc[1, 1:])
+    assert torch.allclose(out[1, 0].float().cpu(), vn[1, 0].float().repeat_interleave(2, dim=0), atol=1e-3)
+
+
 def test_kvcache_strided_cache_views():
     """K and V caches as strided views of one (b, s, 2, h_k, d) tensor, as the reference's MHA module
     passes them (flash_attn/modules/mha.py:459-477)."""
