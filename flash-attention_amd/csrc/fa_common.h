@@ -468,4 +468,42 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
     return s;
 }
 
+// Work item of a workgroup of the long-sequence forward kernels.  Block ids are dealt round-robin
+// over the 8 XCDs by hardware, each XCD has its own L2, and all row blocks of a (batch, kv head)
+// stream should meet in one L2 (heavy, late row blocks first; grouped q heads adjacent).
+//  * Dense batches: every stream costs the same, so XCD x takes the x-th contiguous eighth of the
+//    (batch, kv head, row block, group) order, which balances the XCDs to within one item.
+//  * Packed variable-length batches: streams cost as their sequence length squared, and a contiguous
+//    eighth is a handful of whole sequences (64 sequences x 16 heads: 8 sequences per XCD, whose
+//    summed cost varies by tens of percent).  There XCD x takes every 8th stream of the order in which
+//    kv heads vary fastest, so the heads of each sequence are spread over the XCDs.
+FA_DEV bool xcd_strided(const fa_fwd_params& p) { return p.cu_seqlens_q != nullptr && (uint32_t)(p.b * p.h_k) >= 8u; }
+FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, int& g, int& mb, int& hk, int& b) {
+    const uint32_t G = (uint32_t)(p.h / p.h_k), x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    if (xcd_strided(p)) {
+        const uint32_t r = j / G, s = (r / nmb) * 8u + x;
+        if (s >= (uint32_t)(p.b * p.h_k)) return false;
+        g = (int)(j % G);
+        mb = (int)(nmb - 1u - r % nmb);
+        hk = (int)(s % (uint32_t)p.h_k);
+        b = (int)(s / (uint32_t)p.h_k);
+        return true;
+    }
+    const uint32_t total = nmb * (uint32_t)p.h * (uint32_t)p.b;
+    uint32_t w = x * (gridDim.x >> 3) + j;
+    if (w >= total) return false;
+    g = (int)(w % G); w /= G;
+    mb = (int)(nmb - 1u - w % nmb); w /= nmb;
+    hk = (int)(w % (uint32_t)p.h_k);
+    b = (int)(w / (uint32_t)p.h_k);
+    return true;
+}
+// grid size that goes with xcd_work_item (host side); 0 when it does not fit 31 bits
+inline int64_t xcd_grid(const fa_fwd_params& p, int64_t nmb) {
+    int64_t per_xcd;
+    if (p.cu_seqlens_q != nullptr && (int64_t)p.b * p.h_k >= 8) per_xcd = ((int64_t)p.b * p.h_k + 7) / 8 * (p.h / p.h_k) * nmb;
+    else per_xcd = (nmb * p.h * p.b + 7) / 8;
+    return per_xcd * 8 > 0x7fffffffLL ? 0 : per_xcd * 8;
+}
+
 }  // namespace fa

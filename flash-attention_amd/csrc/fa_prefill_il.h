@@ -102,14 +102,8 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2
     const int l32 = lane & 31, hh = lane >> 5;
 
     const int G = p.h / p.h_k;
-    const int64_t total = (int64_t)kp.num_m_blocks * p.h * p.b;
-    const int per_xcd = gridDim.x >> 3;
-    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (w >= total) return;
-    const int g = (int)(w % G); w /= G;
-    const int mb = kp.num_m_blocks - 1 - (int)(w % kp.num_m_blocks); w /= kp.num_m_blocks;
-    const int hk = (int)(w % p.h_k);
-    const int b = (int)(w / p.h_k);
+    int g, mb, hk, b;
+    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, g, mb, hk, b)) return;
     const int head = hk * G + g;
 
     const SeqInfo si = seq_info(p, b);
@@ -605,9 +599,9 @@ int launch_prefill_il_one(KParams kp, hipStream_t stream) {
     kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
     if (total <= 0) return 0;
-    const int64_t per_xcd = (total + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
+    const int64_t nblocks = xcd_grid(kp.p, kp.num_m_blocks);
+    if (nblocks == 0) return -2;
+    dim3 grid((unsigned)nblocks), block(C::kThreads);
     auto kern = prefill_il_kernel<T, C, DROPOUT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
     if (e != hipSuccess) return (int)e;

@@ -67,15 +67,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 
     // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
     const uint32_t G = (uint32_t)(p.h / p.h_k);
-    const uint32_t nmb = (uint32_t)kp.num_m_blocks;
-    const uint32_t total = nmb * (uint32_t)p.h * (uint32_t)p.b;
-    const uint32_t per_xcd = gridDim.x >> 3;
-    uint32_t w = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-    if (w >= total) return;
-    const int g = (int)(w % G); w /= G;
-    const int mb = (int)(nmb - 1 - w % nmb); w /= nmb;
-    const int hk = (int)(w % (uint32_t)p.h_k);
-    const int b = (int)(w / (uint32_t)p.h_k);
+    int g, mb, hk, b;
+    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, g, mb, hk, b)) return;
     const int head = hk * (int)G + g;
 
     const SeqInfo si = seq_info(p, b);
@@ -402,9 +395,9 @@ int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
     if (total <= 0) return 0;
-    const int64_t per_xcd = (total + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
+    const int64_t nblocks = xcd_grid(kp.p, kp.num_m_blocks);
+    if (nblocks == 0) return -2;
+    dim3 grid((unsigned)nblocks), block(C::kThreads);
     auto kern = prefill_pp_kernel<T, D, BN, DROPOUT>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
     if (e != hipSuccess) return (int)e;
