@@ -107,18 +107,17 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     const fa_bwd_params& p = kp.p;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, hh = lane >> 5;
 
-    // logical order: heads of one group adjacent, then query tiles, then kv heads, then batch; runs of
-    // the order go to one XCD so that workgroups streaming the same K / V share an L2
+    // logical order: heads of one group adjacent, then query tiles, then kv heads, then batch; whole
+    // (batch, kv head) streams go to one XCD so that workgroups streaming the same K / V share an L2
+    // (xcd_stream_unit: contiguous eighths for dense batches, every 8th stream for packed ones)
     const int G = p.h / p.h_k;
     const int num_m_blocks = (p.seqlen_q + C::BM - 1) / C::BM;
-    const int64_t total = (int64_t)num_m_blocks * p.h * p.b;
-    const int per_xcd = gridDim.x >> 3;
-    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (w >= total) return;
-    const int g = (int)(w % G); w /= G;
-    const int mb = num_m_blocks - 1 - (int)(w % num_m_blocks); w /= num_m_blocks;
-    const int hk = (int)(w % p.h_k);
-    const int b = (int)(w / p.h_k);
+    uint32_t unit;
+    int hk, b;
+    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
+                         (uint32_t)(G * num_m_blocks), unit, hk, b)) return;
+    const int g = (int)(unit % (uint32_t)G);
+    const int mb = num_m_blocks - 1 - (int)(unit / (uint32_t)G);
     const int head = hk * G + g;
 
     const BwdSeq si = bwd_seq(p, b);
@@ -307,14 +306,12 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
 
     const int G = p.h / p.h_k;
     const int num_n_blocks = (p.seqlen_k + C::BNW - 1) / C::BNW;
-    const int64_t total = (int64_t)num_n_blocks * p.h_k * p.b * DPARTS;
-    const int per_xcd = gridDim.x >> 3;
-    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (w >= total) return;
-    const int dpart = (int)(w % DPARTS); w /= DPARTS;      // with DPARTS = 2 a workgroup accumulates half of the head dim
-    const int nblk = (int)(w % num_n_blocks); w /= num_n_blocks;
-    const int hk = (int)(w % p.h_k);
-    const int b = (int)(w / p.h_k);
+    uint32_t unit;
+    int hk, b;
+    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
+                         (uint32_t)(num_n_blocks * DPARTS), unit, hk, b)) return;
+    const int dpart = (int)(unit % DPARTS);      // with DPARTS = 2 a workgroup accumulates half of the head dim
+    const int nblk = (int)(unit / DPARTS);
 
     const BwdSeq si = bwd_seq(p, b);
     const int n0 = nblk * C::BNW;
@@ -601,26 +598,26 @@ template <typename K> static int bwd_set_smem(K kern, int bytes) {
 template <typename T, int D, int BN, int MINW, bool DROPOUT>
 int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDqCfg<T, D, BN> C;
-    const int64_t total = (int64_t)((kp.p.seqlen_q + C::BM - 1) / C::BM) * kp.p.h * kp.p.b;
-    if (total <= 0) return 0;
-    const int64_t per_xcd = (total + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    const int64_t per_stream = (int64_t)((kp.p.seqlen_q + C::BM - 1) / C::BM) * (kp.p.h / kp.p.h_k);
+    if (per_stream * kp.p.h_k * kp.p.b <= 0) return 0;
+    const int64_t nblocks = xcd_grid(xcd_strided(kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k), kp.p.b, kp.p.h_k, per_stream);
+    if (nblocks == 0) return -2;
     auto kern = bwd_dq_kernel<T, D, BN, MINW, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
 
 template <typename T, int D, int BM, int DPARTS, bool DROPOUT>
 int launch_bwd_dkv3(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDkv3Cfg<T, D, BM, DPARTS> C;
-    const int64_t total = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * kp.p.h_k * kp.p.b * DPARTS;
-    if (total <= 0) return 0;
-    const int64_t per_xcd = (total + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return -2;
+    const int64_t per_stream = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * DPARTS;
+    if (per_stream * kp.p.h_k * kp.p.b <= 0) return 0;
+    const int64_t nblocks = xcd_grid(xcd_strided(kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k), kp.p.b, kp.p.h_k, per_stream);
+    if (nblocks == 0) return -2;
     auto kern = bwd_dkv3_kernel<T, D, BM, DPARTS, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(per_xcd * 8)), dim3(C::kThreads), C::SMEM, stream, kp);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
 

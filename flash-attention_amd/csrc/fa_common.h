@@ -477,33 +477,40 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
 //    eighth is a handful of whole sequences (64 sequences x 16 heads: 8 sequences per XCD, whose
 //    summed cost varies by tens of percent).  There XCD x takes every 8th stream of the order in which
 //    kv heads vary fastest, so the heads of each sequence are spread over the XCDs.
-FA_DEV bool xcd_strided(const fa_fwd_params& p) { return p.cu_seqlens_q != nullptr && (uint32_t)(p.b * p.h_k) >= 8u; }
-FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, int& g, int& mb, int& hk, int& b) {
-    const uint32_t G = (uint32_t)(p.h / p.h_k), x = blockIdx.x & 7u, j = blockIdx.x >> 3;
-    if (xcd_strided(p)) {
-        const uint32_t r = j / G, s = (r / nmb) * 8u + x;
-        if (s >= (uint32_t)(p.b * p.h_k)) return false;
-        g = (int)(j % G);
-        mb = (int)(nmb - 1u - r % nmb);
-        hk = (int)(s % (uint32_t)p.h_k);
-        b = (int)(s / (uint32_t)p.h_k);
-        return true;
+__host__ __device__ inline bool xcd_strided(bool varlen, int64_t batch, int64_t h_k) { return varlen && batch * h_k >= 8; }
+// Every (batch, kv head) stream has per_stream work units; yields this workgroup's unit and stream.
+FA_DEV bool xcd_stream_unit(bool strided, uint32_t batch, uint32_t h_k, uint32_t per_stream, uint32_t& unit, int& hk, int& b) {
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    uint32_t s;
+    if (strided) {
+        unit = j % per_stream;
+        s = (j / per_stream) * 8u + x;
+    } else {
+        const uint32_t w = x * (gridDim.x >> 3) + j;
+        unit = w % per_stream;
+        s = w / per_stream;
     }
-    const uint32_t total = nmb * (uint32_t)p.h * (uint32_t)p.b;
-    uint32_t w = x * (gridDim.x >> 3) + j;
-    if (w >= total) return false;
-    g = (int)(w % G); w /= G;
-    mb = (int)(nmb - 1u - w % nmb); w /= nmb;
-    hk = (int)(w % (uint32_t)p.h_k);
-    b = (int)(w / (uint32_t)p.h_k);
+    if (s >= batch * h_k) return false;
+    hk = (int)(s % h_k);
+    b = (int)(s / h_k);
     return true;
 }
-// grid size that goes with xcd_work_item (host side); 0 when it does not fit 31 bits
-inline int64_t xcd_grid(const fa_fwd_params& p, int64_t nmb) {
-    int64_t per_xcd;
-    if (p.cu_seqlens_q != nullptr && (int64_t)p.b * p.h_k >= 8) per_xcd = ((int64_t)p.b * p.h_k + 7) / 8 * (p.h / p.h_k) * nmb;
-    else per_xcd = (nmb * p.h * p.b + 7) / 8;
+// grid size that goes with xcd_stream_unit (host side); 0 when it does not fit 31 bits
+inline int64_t xcd_grid(bool strided, int64_t batch, int64_t h_k, int64_t per_stream) {
+    const int64_t per_xcd = strided ? (batch * h_k + 7) / 8 * per_stream : (batch * h_k * per_stream + 7) / 8;
     return per_xcd * 8 > 0x7fffffffLL ? 0 : per_xcd * 8;
+}
+// Forward kernels: a stream's units are its row blocks (heavy, late ones first) x grouped q heads.
+FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, int& g, int& mb, int& hk, int& b) {
+    const uint32_t G = (uint32_t)(p.h / p.h_k);
+    uint32_t unit;
+    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k, G * nmb, unit, hk, b)) return false;
+    g = (int)(unit % G);
+    mb = (int)(nmb - 1u - unit / G);
+    return true;
+}
+inline int64_t xcd_grid(const fa_fwd_params& p, int64_t nmb) {
+    return xcd_grid(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), p.b, p.h_k, (int64_t)(p.h / p.h_k) * nmb);
 }
 
 }  // namespace fa

@@ -50,19 +50,17 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int l32 = lane & 31, hh = lane >> 5;
 
-    // ---- work decode: contiguous ranges of the logical order go to one XCD (block ids are
-    // dealt round-robin over the 8 XCDs), so that workgroups sharing a K/V stream share an L2.
+    // ---- work decode: whole (batch, kv head) streams go to one XCD (block ids are dealt round-robin
+    // over the 8 XCDs), so that workgroups sharing a K/V stream share an L2; see xcd_stream_unit.
     const int G = p.h / p.h_k;
     const int S = SPLIT ? kp.num_splits : 1;
-    const int64_t total = (int64_t)kp.num_m_blocks * p.h * p.b * S;
-    const int per_xcd = gridDim.x >> 3;
-    int64_t w = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (w >= total) return;
-    const int split = (int)(w % S); w /= S;
-    const int g = (int)(w % G); w /= G;
-    const int mb = kp.num_m_blocks - 1 - (int)(w % kp.num_m_blocks); w /= kp.num_m_blocks;
-    const int hk = (int)(w % p.h_k);
-    const int b = (int)(w / p.h_k);
+    uint32_t unit;
+    int hk, b;
+    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
+                         (uint32_t)(S * G * kp.num_m_blocks), unit, hk, b)) return;
+    const int split = (int)(unit % (uint32_t)S); unit /= (uint32_t)S;
+    const int g = (int)(unit % (uint32_t)G);
+    const int mb = kp.num_m_blocks - 1 - (int)(unit / (uint32_t)G);
     const int head = hk * G + g;
 
     const SeqInfo si = seq_info(p, b);
@@ -320,9 +318,10 @@ int launch_prefill(KParams kp, hipStream_t stream) {
     const bool split = kp.num_splits > 1;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b * (split ? kp.num_splits : 1);
     if (total <= 0) return 0;
-    const int64_t per_xcd = (total + 7) / 8;
-    if (per_xcd * 8 > 0x7fffffffLL) return -2;
-    dim3 grid((unsigned)(per_xcd * 8)), block(C::kThreads);
+    const int64_t nblocks = xcd_grid(xcd_strided(kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k), kp.p.b, kp.p.h_k,
+                                     (int64_t)kp.num_m_blocks * (kp.p.h / kp.p.h_k) * (split ? kp.num_splits : 1));
+    if (nblocks == 0) return -2;
+    dim3 grid((unsigned)nblocks), block(C::kThreads);
     hipError_t e;
     if (split) {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, true>;
