@@ -478,19 +478,38 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
 //    summed cost varies by tens of percent).  There XCD x takes every 8th stream of the order in which
 //    kv heads vary fastest, so the heads of each sequence are spread over the XCDs.
 __host__ __device__ inline bool xcd_strided(bool varlen, int64_t batch, int64_t h_k) { return varlen && batch * h_k >= 8; }
-// Every (batch, kv head) stream has per_stream work units; yields this workgroup's unit and stream.
-FA_DEV bool xcd_stream_unit(bool strided, uint32_t batch, uint32_t h_k, uint32_t per_stream, uint32_t& unit, int& hk, int& b) {
-    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+// Every (batch, kv head) stream has per_stream work units, heavy ones first; yields this workgroup's
+// unit and stream.  `slots` is the number of workgroups an XCD holds at once (32 CUs x workgroups
+// per CU).  A stream with fewer units than slots cannot keep an XCD busy by itself, and handing the
+// streams out one after the other leaves the CUs that drew a stream's light units idle while its
+// heavy ones finish (causal row blocks cost as their index; 16 blocks on 32 slots: 9 % lost, 8 on
+// 64: 20-35 %).  So the streams of an XCD are taken k at a time, k * per_stream >= slots, and inside
+// such a group the order is unit-major: the heaviest unit of each of the k streams, then the next.
+// The k streams then share the L2 (k x K/V of a short sequence is no more than one long one).
+// Callers pass slots = 0 (k = 1, one stream after the other) when no mask is active: all units of
+// a stream then cost the same and sharing the L2 only costs (measured -1..2 %).
+FA_DEV bool xcd_stream_unit(bool strided, uint32_t batch, uint32_t h_k, uint32_t per_stream, uint32_t slots,
+                            uint32_t& unit, int& hk, int& b) {
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3, S = batch * h_k;
     uint32_t s;
-    if (strided) {
-        unit = j % per_stream;
-        s = (j / per_stream) * 8u + x;
-    } else {
+    if (!strided && (S & 7u) != 0u) {
+        // dense batch whose streams do not divide over the XCDs: contiguous eighths of the unit order
         const uint32_t w = x * (gridDim.x >> 3) + j;
         unit = w % per_stream;
         s = w / per_stream;
+    } else {
+        const uint32_t n_local = strided ? (S + 7u - x) >> 3 : S >> 3;       // streams of this XCD
+        const uint32_t k = max(1u, min((slots + per_stream - 1u) / per_stream, n_local));
+        const uint32_t grp = j / (k * per_stream), first = grp * k;
+        if (first >= n_local) return false;
+        const uint32_t kk = min(k, n_local - first);                          // the last group may be short
+        const uint32_t r = j - grp * k * per_stream;
+        if (r >= kk * per_stream) return false;
+        unit = r / kk;
+        const uint32_t ls = first + r % kk;
+        s = strided ? ls * 8u + x : x * n_local + ls;
     }
-    if (s >= batch * h_k) return false;
+    if (s >= S) return false;
     hk = (int)(s % h_k);
     b = (int)(s / h_k);
     return true;
@@ -501,10 +520,10 @@ inline int64_t xcd_grid(bool strided, int64_t batch, int64_t h_k, int64_t per_st
     return per_xcd * 8 > 0x7fffffffLL ? 0 : per_xcd * 8;
 }
 // Forward kernels: a stream's units are its row blocks (heavy, late ones first) x grouped q heads.
-FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, int& g, int& mb, int& hk, int& b) {
+FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, uint32_t slots, int& g, int& mb, int& hk, int& b) {
     const uint32_t G = (uint32_t)(p.h / p.h_k);
     uint32_t unit;
-    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k, G * nmb, unit, hk, b)) return false;
+    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k, G * nmb, slots, unit, hk, b)) return false;
     g = (int)(unit % G);
     mb = (int)(nmb - 1u - unit / G);
     return true;

@@ -103,7 +103,8 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2
 
     const int G = p.h / p.h_k;
     int g, mb, hk, b;
-    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, g, mb, hk, b)) return;
+    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks,
+                       !(kp.has_left || kp.has_right) ? 0u : C::kPair ? 32u : (C::D == 64 ? 96u : 64u), g, mb, hk, b)) return;
     const int head = hk * G + g;
 
     const SeqInfo si = seq_info(p, b);

@@ -68,7 +68,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
     const uint32_t G = (uint32_t)(p.h / p.h_k);
     int g, mb, hk, b;
-    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, g, mb, hk, b)) return;
+    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, (kp.has_left || kp.has_right) ? 32u : 0u, g, mb, hk, b)) return;
     const int head = hk * (int)G + g;
 
     const SeqInfo si = seq_info(p, b);
