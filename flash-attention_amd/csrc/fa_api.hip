@@ -35,6 +35,9 @@ static const int kNumCU = 256;   // MI355X
 #ifndef FA_DEC_SB
 #define FA_DEC_SB 8
 #endif
+#ifndef FA_DEC_MINLEN
+#define FA_DEC_MINLEN 512       // shortest chunk of the decode kernel (keys) once the launch fills the CUs
+#endif
 
 // The small-q streaming kernel packs seqlen_q x (h / h_k) rows into 16 MFMA columns.
 static bool use_decode_kernel(const fa_fwd_params& p) {
@@ -93,12 +96,15 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
             automatic = true;
             if (dec) {
                 // ~8k chunk slots over the whole launch (16 per resident workgroup), chunks of at
-                // least 256 keys: measured best trade between per-workgroup start-up cost and
+                // least 256 to 512 keys: measured best trade between per-workgroup start-up cost and
                 // the tail left by ragged cache lengths on 256 CUs x 2 resident groups.
                 // With the caller's scratch word the kernel is persistent and takes longer chunks
                 // (4096 keys at batch 64 x 8 kv heads x 32k), their ragged remainders in eighths.
                 const int64_t streams = (int64_t)p.b * p.h_k;
-                int64_t len = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS), 128);
+                // Chunks shorter than 512 keys are mostly start-up and merge (batch 4 x 32k: +22 % with
+                // 512 over 256); 256 only while 512-key chunks would leave resident slots empty.
+                const int64_t minlen = streams * ((sk + FA_DEC_MINLEN - 1) / FA_DEC_MINLEN) < 2 * kNumCU ? 256 : FA_DEC_MINLEN;
+                int64_t len = rup(std::max<int64_t>(minlen, (int64_t)sk * streams / FA_DEC_SLOTS), 128);
                 if (p.work_counter) {
                     const int64_t lp = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS_P), 128);
                     if (lp >= 1024) len = lp;
