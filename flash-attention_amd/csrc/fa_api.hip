@@ -156,11 +156,11 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.work_counter = q.work_counter;
 }
 
-static int run_attention(KParams& kp, hipStream_t stream) {
+static int run_attention(KParams& kp, hipStream_t stream, bool counter_is_reset = false) {
     const fa_fwd_params& p = kp.p;
     int e;
     if (use_decode_kernel(p)) {
-        if (kp.dec_persistent) {
+        if (kp.dec_persistent && !counter_is_reset) {
             e = launch_zero_counter(kp.work_counter, stream);
             if (e) return fail_hip(e, "ticket reset launch");
         }
@@ -341,10 +341,12 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
     kp.rotary_q = kp.p.rotary_dim > 0;
     if (int r = resolve_splits(kp, kp.p, true)) return r;
     hipStream_t stream = (hipStream_t)hip_stream;
+    // the append launch also resets the ticket counter of a persistent decode launch (one launch less)
+    const bool reset_in_append = has_new && kp.dec_persistent && use_decode_kernel(kp.p);
     if (has_new) {
-        if (int e = launch_append_kv(kp, stream)) return fail_hip(e, "append_kv kernel launch");
+        if (int e = launch_append_kv(kp, reset_in_append ? kp.work_counter : nullptr, stream)) return fail_hip(e, "append_kv kernel launch");
     }
-    return run_attention(kp, stream);
+    return run_attention(kp, stream, reset_in_append);
 }
 
 int32_t fa_sizeof_rotary_params(void) { return (int32_t)sizeof(fa_rotary_params); }

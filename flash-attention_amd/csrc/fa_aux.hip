@@ -69,8 +69,9 @@ int launch_combine(const KParams& kp, hipStream_t stream) {
 
 // One thread per 16-byte chunk of one new (token, kv-head) row.
 template <typename T>
-__global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp) {
+__global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp, int32_t* zero) {
     const fa_fwd_params& p = kp.p;
+    if (zero && blockIdx.x == 0 && threadIdx.x == 0) *zero = 0;     // ticket counter of the decode launch that follows
     const int cpr = p.d / 8;
     const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * cpr;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -103,13 +104,13 @@ __global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp) {
     st_global16(kdst + d0, raw);
 }
 
-int launch_append_kv(const KParams& kp, hipStream_t stream) {
+int launch_append_kv(const KParams& kp, int32_t* zero, hipStream_t stream) {
     const fa_fwd_params& p = kp.p;
     const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * (p.d / 8);
-    if (total == 0) return 0;
+    if (total == 0) return zero ? launch_zero_counter(zero, stream) : 0;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
-    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(append_kv_kernel<__bf16>, grid, block, 0, stream, kp);
-    else hipLaunchKernelGGL(append_kv_kernel<_Float16>, grid, block, 0, stream, kp);
+    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(append_kv_kernel<__bf16>, grid, block, 0, stream, kp, zero);
+    else hipLaunchKernelGGL(append_kv_kernel<_Float16>, grid, block, 0, stream, kp, zero);
     return (int)hipGetLastError();
 }
 
