@@ -18,14 +18,14 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     typedef PrefillTile<FA_D> Tile;
 #if FA_D <= 128
     // Long query sequences (measured cross-overs on MI355X):
-    //  * head dim 128, keys beyond 2048 (causal / windowed) or 768 (full): the 8-wave ping-pong
+    //  * head dim 128, from 2048 keys on (causal / windowed) or beyond 768 (full): the 8-wave ping-pong
     //    kernel, 256 rows per workgroup, each K/V tile fetched once per 256 rows;
     //  * otherwise from 512 query rows on: the software-pipelined kernel, two independent
     //    128-row workgroups per CU, whose start-up and output phases overlap.
     // Shorter sequences, split key ranges and q rotary take the general 4-wave kernel.
     if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) {
         const bool masked = kp.has_right || kp.has_left;
-        const bool long_keys = kp.p.seqlen_k > (masked ? 2048 : 768);
+        const bool long_keys = kp.p.seqlen_k >= (masked ? 2048 : 769);
         if (FA_D >= 128 && long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
         return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }
