@@ -468,9 +468,9 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
     return s;
 }
 
-// Work item of a workgroup of the long-sequence forward kernels.  Block ids are dealt round-robin
+// Which work item a workgroup of the tiled forward and backward kernels takes.  Block ids are dealt round-robin
 // over the 8 XCDs by hardware, each XCD has its own L2, and all row blocks of a (batch, kv head)
-// stream should meet in one L2 (heavy, late row blocks first; grouped q heads adjacent).
+// stream should meet in one L2 (heavy blocks first; grouped q heads adjacent).
 //  * Dense batches: every stream costs the same, so XCD x takes the x-th contiguous eighth of the
 //    (batch, kv head, row block, group) order, which balances the XCDs to within one item.
 //  * Packed variable-length batches: streams cost as their sequence length squared, and a contiguous
