@@ -17,6 +17,8 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
   * fwd_bwd  -- the one kernel metric the reference publishes (forward + backward together, fp16, causal,
                 head dim 128, seqlen 8k, batch 2, 16 heads: 182 TFLOP/s on A100, 308 on H100), FLOPs
                 counted as 3.5 x forward like the reference's benchmark script;
+  * varlen   -- flash_attn_varlen_func, bf16, 64 packed sequences with lengths uniform in [128, 4096]
+                (seed 0), 16 heads, head dim 128 and 256, causal; FLOPs over the visible (row, key) pairs;
 Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
 attention_ref) timed on the host cores on a bounded sample of the same workload.
 """
@@ -121,6 +123,30 @@ def bench_backward(steps, warmup):
                      "kernel": "fa::bwd_dkv3_kernel<bf16,128,64> + fa::bwd_dq_kernel<bf16,128,32> (7 tile products executed for 5 counted)",
                      "flops_per_launch": flops},
     }
+
+
+def bench_varlen(steps, warmup):
+    import torch
+    import flash_attn
+    torch.manual_seed(0)
+    lens = torch.randint(128, 4097, (64,))
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(torch.int32)
+    total, mx, h = int(cu[-1]), int(lens.max()), 16
+    cu_d = cu.cuda()
+    res = {"workload": "flash_attn_varlen_func fwd bf16 64 sequences U[128,4096] (%d tokens) nheads=16 causal" % total}
+    for d in (128, 256):
+        q, k, v = (torch.randn(total, h, d, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+        fn = lambda: flash_attn.flash_attn_varlen_func(q, k, v, cu_d, cu_d, mx, mx, causal=True)
+        ms, wall_ms = time_steps(fn, steps, warmup)
+        flops = sum(4.0 * h * d * (int(l) * (int(l) + 1) / 2) for l in lens)
+        tflops = flops / (ms * 1e-3) / 1e12
+        res["d%d" % d] = {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": total / (ms * 1e-3),
+                          "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                       "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                                       "kernel": "fa::prefill_pp_kernel<bf16,128,64>" if d == 128 else "fa::prefill_il_kernel<bf16,pair 256>",
+                                       "flops_per_launch": flops}}
+        del q, k, v
+    return res
 
 
 def bench_fwd_bwd(steps, warmup):
@@ -247,6 +273,7 @@ def main():
         out["rotary"] = bench_rotary(a.steps, a.warmup)
         out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))
         out["fwd_bwd"] = bench_fwd_bwd(a.steps, a.warmup)
+        out["varlen"] = bench_varlen(a.steps, a.warmup)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
