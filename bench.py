@@ -19,6 +19,8 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
                 counted as 3.5 x forward like the reference's benchmark script;
   * varlen   -- flash_attn_varlen_func, bf16, 64 packed sequences with lengths uniform in [128, 4096]
                 (seed 0), 16 heads, head dim 128 and 256, causal; FLOPs over the visible (row, key) pairs;
+  * gqa_window -- flash_attn_func, bf16, batch 2, seqlen 16384, 32 query / 8 kv heads, head dim 128, causal
+                with window (4096, 0); FLOPs over the visible pairs (sum_i min(i + 1, 4097) per head);
 Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
 attention_ref) timed on the host cores on a bounded sample of the same workload.
 """
@@ -149,6 +151,27 @@ def bench_varlen(steps, warmup):
     return res
 
 
+def bench_gqa_window(steps, warmup):
+    import torch
+    import flash_attn
+    b, s, h, hk, d, wl = 2, 16384, 32, 8, 128, 4096
+    torch.manual_seed(0)
+    q = torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16)
+    k, v = (torch.randn(b, s, hk, d, device="cuda", dtype=torch.bfloat16) for _ in range(2))
+    fn = lambda: flash_attn.flash_attn_func(q, k, v, causal=True, window_size=(wl, 0))
+    ms, wall_ms = time_steps(fn, steps, warmup)
+    pairs = (wl + 1) * (wl + 2) // 2 + (s - wl - 1) * (wl + 1)       # sum_i min(i + 1, wl + 1)
+    flops = 4.0 * d * pairs * b * h
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {
+        "ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
+        "workload": "flash_attn_func fwd bf16 batch=2 seqlen=16384 nheads=32 nheads_kv=8 headdim=128 causal window=(4096,0)",
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "fa::prefill_pp_kernel<bf16,128,64>", "flops_per_launch": flops},
+    }
+
+
 def bench_fwd_bwd(steps, warmup):
     import torch
     from flash_attn import _native as nat
@@ -274,6 +297,7 @@ def main():
         out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))
         out["fwd_bwd"] = bench_fwd_bwd(a.steps, a.warmup)
         out["varlen"] = bench_varlen(a.steps, a.warmup)
+        out["gqa_window"] = bench_gqa_window(a.steps, a.warmup)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
