@@ -112,12 +112,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     // (xcd_stream_unit: contiguous eighths for dense batches, every 8th stream for packed ones)
     const int G = p.h / p.h_k;
     const int num_m_blocks = (p.seqlen_q + C::BM - 1) / C::BM;
-    uint32_t unit;
-    int hk, b;
-    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
-                         (uint32_t)(G * num_m_blocks), (kp.has_left || kp.has_right) ? 32u * MINW : 0u, unit, hk, b)) return;
-    const int g = (int)(unit % (uint32_t)G);
-    const int mb = num_m_blocks - 1 - (int)(unit / (uint32_t)G);
+    int g, mb, hk, b;
+    if (!xcd_rows_item(false, p.cu_seqlens_q != nullptr, (uint32_t)p.b, (uint32_t)p.h_k, (uint32_t)G, (uint32_t)num_m_blocks,
+                       (kp.has_left || kp.has_right) ? 32u * MINW : 0u, g, mb, hk, b)) return;
     const int head = hk * G + g;
 
     const BwdSeq si = bwd_seq(p, b);
@@ -598,9 +595,9 @@ template <typename K> static int bwd_set_smem(K kern, int bytes) {
 template <typename T, int D, int BN, int MINW, bool DROPOUT>
 int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDqCfg<T, D, BN> C;
-    const int64_t per_stream = (int64_t)((kp.p.seqlen_q + C::BM - 1) / C::BM) * (kp.p.h / kp.p.h_k);
-    if (per_stream * kp.p.h_k * kp.p.b <= 0) return 0;
-    const int64_t nblocks = xcd_grid(xcd_strided(kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k), kp.p.b, kp.p.h_k, per_stream);
+    const int64_t nmb = (kp.p.seqlen_q + C::BM - 1) / C::BM;
+    if (nmb * kp.p.h * kp.p.b <= 0) return 0;
+    const int64_t nblocks = xcd_rows_grid(false, kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k, kp.p.h / kp.p.h_k, nmb);
     if (nblocks == 0) return -2;
     auto kern = bwd_dq_kernel<T, D, BN, MINW, DROPOUT>;
     if (int e = bwd_set_smem(kern, C::SMEM)) return e;

@@ -519,17 +519,41 @@ inline int64_t xcd_grid(bool strided, int64_t batch, int64_t h_k, int64_t per_st
     const int64_t per_xcd = strided ? (batch * h_k + 7) / 8 * per_stream : (batch * h_k * per_stream + 7) / 8;
     return per_xcd * 8 > 0x7fffffffLL ? 0 : per_xcd * 8;
 }
-// Forward kernels: a stream's units are its row blocks (heavy, late ones first) x grouped q heads.
-FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, uint32_t slots, int& g, int& mb, int& hk, int& b) {
-    const uint32_t G = (uint32_t)(p.h / p.h_k);
+// Packed batches with one or two kv heads (MQA / GQA, or a tensor-parallel shard of them): whole
+// (sequence, kv head) streams cannot give every XCD a piece of every sequence, so in the forward
+// kernels the grouped q heads of a stream are cut into `parts` (h_k * parts = 8) and each part is
+// handed out as a stream of its own: the XCDs get equal work whatever the sequence lengths are
+// (64 sequences, 32 q heads on 1 kv head: 600-700 -> 940-960 TFLOP/s; 16 on 2: +17 %).  The parts
+// of a stream read its K/V through different L2s; with 4 kv heads (2 parts) that costs more than
+// the balance gains at head dim 64, and the dQ pass, which re-reads K and V per row block, loses
+// with 2 kv heads too, so the backward kernels keep whole streams (split = false).
+__host__ __device__ inline uint32_t xcd_parts(bool split, bool varlen, uint32_t h_k, uint32_t G) {
+    if (!split || !varlen || h_k > 2u) return 1u;
+    const uint32_t want = 8u / h_k;
+    return G % want == 0u ? want : 1u;
+}
+// Forward kernels and the dQ pass: a stream's units are its row blocks (heavy, late ones first) x
+// grouped q heads.
+FA_DEV bool xcd_rows_item(bool split, bool varlen, uint32_t batch, uint32_t h_k, uint32_t G, uint32_t nmb, uint32_t slots,
+                          int& g, int& mb, int& hk, int& b) {
+    const uint32_t parts = xcd_parts(split, varlen, h_k, G), Gp = G / parts, hp = h_k * parts;
     uint32_t unit;
-    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k, G * nmb, slots, unit, hk, b)) return false;
-    g = (int)(unit % G);
-    mb = (int)(nmb - 1u - unit / G);
+    int hkp;
+    if (!xcd_stream_unit(xcd_strided(varlen, batch, hp), batch, hp, Gp * nmb, slots, unit, hkp, b)) return false;
+    hk = (int)((uint32_t)hkp / parts);
+    g = (int)(((uint32_t)hkp % parts) * Gp + unit % Gp);
+    mb = (int)(nmb - 1u - unit / Gp);
     return true;
 }
+inline int64_t xcd_rows_grid(bool split, bool varlen, int64_t batch, int64_t h_k, int64_t G, int64_t nmb) {
+    const int64_t parts = xcd_parts(split, varlen, (uint32_t)h_k, (uint32_t)G);
+    return xcd_grid(xcd_strided(varlen, batch, h_k * parts), batch, h_k * parts, G / parts * nmb);
+}
+FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, uint32_t slots, int& g, int& mb, int& hk, int& b) {
+    return xcd_rows_item(true, p.cu_seqlens_q != nullptr, (uint32_t)p.b, (uint32_t)p.h_k, (uint32_t)(p.h / p.h_k), nmb, slots, g, mb, hk, b);
+}
 inline int64_t xcd_grid(const fa_fwd_params& p, int64_t nmb) {
-    return xcd_grid(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), p.b, p.h_k, (int64_t)(p.h / p.h_k) * nmb);
+    return xcd_rows_grid(true, p.cu_seqlens_q != nullptr, p.b, p.h_k, p.h / p.h_k, nmb);
 }
 
 }  // namespace fa

@@ -88,6 +88,9 @@ PACKED = [
     ([600, 1030, 90], 4, 2, 128, True),                                    # 6 < 8: contiguous eighths
     ([2300, 150, 2048, 900, 1700, 31, 1, 640], 2, 1, 128, True),           # 8 streams, ping-pong kernel
     ([700, 520, 64, 900, 1300, 200, 1024, 45], 8, 8, 256, False),          # pair kernel, no mask
+    ([900, 130, 1500, 64, 700, 1024, 333, 1200, 512], 8, 1, 128, True),   # MQA: the 8 q heads of a stream go to 8 XCDs (forward)
+    ([1100, 40, 513, 777, 260, 2100], 8, 2, 64, True),                     # GQA: 2 kv heads x 4 parts of 1 q head (forward)
+    ([600, 1030, 90, 300], 12, 2, 128, True),                              # 6 q heads per kv head: not cut
 ]
 
 
