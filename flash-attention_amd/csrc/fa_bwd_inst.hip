@@ -29,6 +29,11 @@ static int run(const BwdKParams& kp, hipStream_t stream) {
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers;
     // three at head dim 64 (168 registers), where the vector work per matrix instruction doubles
     if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, (FA_D == 64 ? 3 : 2), DROPOUT>(kp, stream)) return e;
+    // Fewer key blocks than CUs (one long sequence on one or two kv heads, say): two workgroups per
+    // key block, each accumulating half of the head dimension, fill the CUs at 3/4 of the work each.
+    typedef BwdDkv3Cfg<InstT, FA_D, FA_BWD_BM, 1> C1;
+    const int64_t key_blocks = (int64_t)((kp.p.seqlen_k + C1::BNW - 1) / C1::BNW) * kp.p.h_k * kp.p.b;
+    if (key_blocks < 256 && kp.p.seqlen_q >= 1024) return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 2, DROPOUT>(kp, stream);
     return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 1, DROPOUT>(kp, stream);
 #else
     if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
