@@ -99,7 +99,7 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
                 // least 256 to 512 keys: measured best trade between per-workgroup start-up cost and
                 // the tail left by ragged cache lengths on 256 CUs x 2 resident groups.
                 // With the caller's scratch word the kernel is persistent and takes longer chunks
-                // (4096 keys at batch 64 x 8 kv heads x 32k), their ragged remainders in eighths.
+                // (4096 keys at batch 64 x 8 kv heads x 32k), their ragged remainders in pieces of 512+ keys.
                 const int64_t streams = (int64_t)p.b * p.h_k;
                 // Chunks shorter than 512 keys are mostly start-up and merge (batch 4 x 32k: +22 % with
                 // 512 over 256); 256 only while 512-key chunks would leave resident slots empty.
@@ -128,12 +128,16 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
     r.splits = splits;
     r.len = len;
     // Persistent two-pass schedule: complete chunks first, then each sequence's ragged remainder in
-    // eighths of a chunk, drawn from a ticket counter.  Needs the caller's scratch word.
-    if (dec && automatic && splits > 1 && p.work_counter && len >= 1024 && splits + FA_DEC_SB <= FA_MAX_SPLITS) {
+    // up to eight pieces of a chunk, drawn from a ticket counter.  Needs the caller's scratch word.
+    // The pieces of a remainder stay at 512 keys or more (halves of a 1024-key chunk, quarters of a
+    // 2048-key one, eighths from 4096 on): shorter pieces are mostly start-up and merge (measured
+    // +6 % at batch 256 x 4k and at batch 64 x 8k with 16 grouped heads, nothing lost at config 5).
+    const int sb = len < 2048 ? 2 : len < 4096 ? 4 : FA_DEC_SB;
+    if (dec && automatic && splits > 1 && p.work_counter && len >= 1024 && splits + sb <= FA_MAX_SPLITS) {
         r.persistent = 1;
         r.sa = splits;
-        r.sb = FA_DEC_SB;
-        r.sub = len / FA_DEC_SB;
+        r.sb = sb;
+        r.sub = len / sb;
         r.splits = r.sa + r.sb;
     }
     return r;
