@@ -26,6 +26,11 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) {
         const bool masked = kp.has_right || kp.has_left;
         const bool long_keys = kp.p.seqlen_k >= (masked ? 2048 : 769);
+        // When the 256-row blocks of the ping-pong kernel would occupy no more than half of the 256
+        // CUs (a chunk of 1024 queries of one sequence with 32 heads: 128 blocks), the 128-row blocks
+        // of the pipelined kernel fill them: measured +12..25 % at 128 blocks, -11 % at 192.
+        const int64_t pp_wgs = (int64_t)((kp.p.seqlen_q + 255) / 256) * kp.p.h * kp.p.b;
+        if (FA_D >= 128 && long_keys && pp_wgs <= 128) return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
         if (FA_D >= 128 && long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
         return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }

@@ -44,7 +44,8 @@ DENSE = [
     (9, 600, 8, 8, 256, True, (-1, -1)),     # 72, head-dim-256 pair kernel
     (4, 300, 4, 2, 64, True, (100, 0)),      # 8, general kernel (fewer than 512 rows), window
     (3, 1536, 8, 8, 128, False, (200, 50)),  # 24, two-sided window on the pipelined kernel
-    (1, 4096, 8, 1, 128, True, (-1, -1)),    # 1 stream: units dealt to the XCDs one by one (ping-pong kernel)
+    (1, 8192, 8, 1, 128, True, (-1, -1)),    # 1 stream: units dealt to the XCDs one by one (ping-pong kernel)
+    (1, 4096, 8, 1, 128, True, (-1, -1)),    # the same with 128 blocks of 256 rows: pipelined kernel on long keys
     (2, 1024, 6, 2, 64, True, (-1, -1)),     # 4 streams, the same on the pipelined kernel
     (1, 2048, 4, 4, 128, False, (-1, -1)),   # 4 streams, no mask: contiguous eighths
 ]
