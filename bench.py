@@ -49,21 +49,39 @@ def _traffic(key):
         return None
 
 
+BLOCKS = 3   # timed blocks of `steps` launches each; the median block is reported, the fastest beside it
+
+
+class Timing(tuple):
+    """(ms, wall_ms) of the median block, with .ms_min = the fastest block's ms per step."""
+    def __new__(cls, ms, wall_ms, ms_min):
+        t = super().__new__(cls, (ms, wall_ms))
+        t.ms_min = ms_min
+        return t
+
+
 def time_steps(fn, steps, warmup):
+    """`warmup` untimed calls, then BLOCKS blocks of exactly `steps` calls, each bracketed by HIP events
+    on the stream the kernels are launched on (torch's current stream) and by a device synchronisation."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    return e0.elapsed_time(e1) / steps, wall_ms / steps
+    blocks = []
+    for _ in range(BLOCKS):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        blocks.append((e0.elapsed_time(e1) / steps, wall_ms / steps))
+    blocks.sort()
+    med = blocks[len(blocks) // 2]
+    return Timing(med[0], med[1], blocks[0][0])
 
 
 def bench_prefill(steps, warmup):
@@ -73,15 +91,42 @@ def bench_prefill(steps, warmup):
     torch.manual_seed(0)
     q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16) for _ in range(3))
     fn = lambda: flash_attn.flash_attn_func(q, k, v, causal=True)
-    ms, wall_ms = time_steps(fn, steps, warmup)
+    tm = time_steps(fn, steps, warmup)
+    ms, wall_ms = tm
     flops = 4.0 * b * s * s * h * d / 2
     tflops = flops / (ms * 1e-3) / 1e12
     return {
-        "ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
+        "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"),
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
                      "kernel": "fa::prefill_pp_kernel<bf16,128,64>", "flops_per_launch": flops},
     }
+
+
+def bench_mfma_peak(steps, warmup):
+    """What the matrix pipes sustain on MFMAs alone (fa_mfma_peak in the library): the clock of the fully
+    loaded part follows the switching activity of the operands, so the figure is taken on random bf16
+    operands (comparable to Gaussian q, k, v) and on zeros."""
+    import ctypes
+    import torch
+    from flash_attn import _native as nat
+    lib = nat.lib
+    lib.fa_mfma_peak.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p]
+    lib.fa_mfma_peak.restype = ctypes.c_int
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {"kernel": "fa::mfma_peak_kernel (independent v_mfma_f32_32x32x16_bf16, 4 waves per SIMD, operands in registers)"}
+    for name, rnd in (("random_bf16", 1), ("zeros", 0)):
+        flops = ctypes.c_int64(0)
+
+        def fn():
+            rc = lib.fa_mfma_peak(sink.data_ptr(), 1500, rnd, ctypes.byref(flops), stream)
+            if rc != 0:
+                raise RuntimeError("fa_mfma_peak failed: %d" % rc)
+        tm = time_steps(fn, max(3, steps // 3), max(2, warmup // 3))
+        res[name] = {"ms": tm[0], "ms_min": tm.ms_min, "tflops": flops.value / (tm[0] * 1e-3) / 1e12,
+                     "frac_of_published_peak": flops.value / (tm[0] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+    return res
 
 
 def bench_rotary(steps, warmup):
@@ -93,11 +138,12 @@ def bench_rotary(steps, warmup):
     ang = torch.rand(s, d // 2, device="cuda") * 6.28
     cos, sin = torch.cos(ang).to(torch.bfloat16), torch.sin(ang).to(torch.bfloat16)
     fn = lambda: apply_rotary(x, cos, sin, inplace=True)
-    ms, wall_ms = time_steps(fn, steps, warmup)
+    tm = time_steps(fn, steps, warmup)
+    ms, wall_ms = tm
     algo_bytes = 2 * x.numel() * x.element_size()
     gbs = algo_bytes / (ms * 1e-3) / 1e9
     return {
-        "ms": ms, "wall_ms": wall_ms, "gb_per_s": gbs,
+        "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "gb_per_s": gbs,
         "workload": "apply_rotary_emb bf16 (8, 8192, 32, 128) rotary_dim 128 in place",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                      "traffic": None, "kernel": "fa::rotary_kernel<bf16,bf16,u32>", "bytes_per_launch": algo_bytes},
@@ -114,11 +160,12 @@ def bench_backward(steps, warmup):
     out, _, _, _, _, lse, _, _ = nat.fwd(q, k, v, None, 0.0, scale, True, -1, -1, False, None)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     fn = lambda: nat.bwd(dout, q, k, v, out, lse, dq, dk, dv, 0.0, scale, True, -1, -1, None, None)
-    ms, wall_ms = time_steps(fn, steps, warmup)
+    tm = time_steps(fn, steps, warmup)
+    ms, wall_ms = tm
     flops = 2.5 * 4.0 * b * s * s * h * d / 2      # 5 products of 2 b h s^2 d / 2 (causal)
     tflops = flops / (ms * 1e-3) / 1e12
     return {
-        "ms": ms, "wall_ms": wall_ms, "tflops": tflops,
+        "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops,
         "workload": "flash_attn_func bwd bf16 batch=4 seqlen=8192 nheads=32 headdim=128 causal (dot + dQ + dK/dV kernels)",
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
@@ -139,10 +186,11 @@ def bench_varlen(steps, warmup):
     for d in (128, 256):
         q, k, v = (torch.randn(total, h, d, device="cuda", dtype=torch.bfloat16) for _ in range(3))
         fn = lambda: flash_attn.flash_attn_varlen_func(q, k, v, cu_d, cu_d, mx, mx, causal=True)
-        ms, wall_ms = time_steps(fn, steps, warmup)
+        tm = time_steps(fn, steps, warmup)
+        ms, wall_ms = tm
         flops = sum(4.0 * h * d * (int(l) * (int(l) + 1) / 2) for l in lens)
         tflops = flops / (ms * 1e-3) / 1e12
-        res["d%d" % d] = {"ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": total / (ms * 1e-3),
+        res["d%d" % d] = {"ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": total / (ms * 1e-3),
                           "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                        "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
                                        "kernel": "fa::prefill_pp_kernel<bf16,128,64>" if d == 128 else "fa::prefill_il_kernel<bf16,pair 256>",
@@ -159,12 +207,13 @@ def bench_gqa_window(steps, warmup):
     q = torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16)
     k, v = (torch.randn(b, s, hk, d, device="cuda", dtype=torch.bfloat16) for _ in range(2))
     fn = lambda: flash_attn.flash_attn_func(q, k, v, causal=True, window_size=(wl, 0))
-    ms, wall_ms = time_steps(fn, steps, warmup)
+    tm = time_steps(fn, steps, warmup)
+    ms, wall_ms = tm
     pairs = (wl + 1) * (wl + 2) // 2 + (s - wl - 1) * (wl + 1)       # sum_i min(i + 1, wl + 1)
     flops = 4.0 * d * pairs * b * h
     tflops = flops / (ms * 1e-3) / 1e12
     return {
-        "ms": ms, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
+        "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
         "workload": "flash_attn_func fwd bf16 batch=2 seqlen=16384 nheads=32 nheads_kv=8 headdim=128 causal window=(4096,0)",
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
@@ -185,11 +234,12 @@ def bench_fwd_bwd(steps, warmup):
         out, _, _, _, _, lse, _, _ = nat.fwd(q, k, v, None, 0.0, scale, True, -1, -1, False, None)
         nat.bwd(dout, q, k, v, out, lse, dq, dk, dv, 0.0, scale, True, -1, -1, None, None)
 
-    ms, wall_ms = time_steps(fn, steps, warmup)
+    tm = time_steps(fn, steps, warmup)
+    ms, wall_ms = tm
     flops = 3.5 * 4.0 * b * s * s * h * d / 2
     tflops = flops / (ms * 1e-3) / 1e12
     return {
-        "ms": ms, "wall_ms": wall_ms, "tflops": tflops,
+        "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops,
         "workload": "flash_attn_func fwd+bwd fp16 batch=2 seqlen=8192 nheads=16 headdim=128 causal",
         "published": {"a100_tflops": 182.0, "h100_tflops": 308.0, "vs_a100": tflops / 182.0, "vs_h100": tflops / 308.0,
                       "source": "reference assets/flash2_a100_fwd_bwd_benchmark.png, flash2_h100_fwd_bwd_benchmark.png, panel (d)"},
@@ -199,7 +249,6 @@ def bench_fwd_bwd(steps, warmup):
 def bench_decode(steps, warmup):
     import torch
     import flash_attn
-    from oracle import attention_oracle as orc
     b, cap, hk, h, d = 64, 32768, 8, 64, 128
     torch.manual_seed(0)
     k_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
@@ -208,26 +257,29 @@ def bench_decode(steps, warmup):
     kn = torch.randn(b, 1, hk, d, device="cuda", dtype=torch.bfloat16)
     vn = torch.randn(b, 1, hk, d, device="cuda", dtype=torch.bfloat16)
     cache_seqlens = torch.randint(1024, cap, (b,), dtype=torch.int32).cuda()   # [1024, 32767]
-    cos, sin = orc.rotary_table(cap, d, dtype=torch.bfloat16)
-    cos, sin = cos.cuda(), sin.cuda()
+    # cos / sin of position x inverse frequency, base 10000, as flash_attn/layers/rotary.py builds its cache
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    ang = torch.outer(torch.arange(cap, dtype=torch.float32), inv_freq)
+    cos, sin = torch.cos(ang).to(torch.bfloat16).cuda(), torch.sin(ang).to(torch.bfloat16).cuda()
     fn = lambda: flash_attn.flash_attn_with_kvcache(q, k_cache, v_cache, kn, vn, cos, sin, cache_seqlens,
                                                     causal=True, rotary_interleaved=True)
-    ms, wall_ms = time_steps(fn, steps, warmup)
+    tm = time_steps(fn, steps, warmup)
+    ms, wall_ms = tm
     keys = int((cache_seqlens.long() + 1).sum().item())
     algo_bytes = keys * hk * d * 2 * 2 + 2 * b * h * d * 2 + 2 * b * hk * d * 2 * 2
     gbs = algo_bytes / (ms * 1e-3) / 1e9
     return {
-        "ms": ms, "wall_ms": wall_ms, "gb_per_s": gbs, "tokens_per_s": b / (ms * 1e-3),
+        "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "gb_per_s": gbs, "tokens_per_s": b / (ms * 1e-3),
         "workload": "flash_attn_with_kvcache bf16 b64 cache(64,32768,8,128) hq64 append1+rotary128 causal",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": gbs / PEAK_HBM_GBS, "traffic": _traffic("decode_bf16_d128_b64_32k"),
+                     "frac": gbs / PEAK_HBM_GBS, "traffic": _traffic("decode_bf16_d128_b64_32k"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
                      "kernel": "fa::decode_persistent_kernel<bf16,128> (step = append_kv with ticket reset + decode + combine)", "bytes_per_launch": algo_bytes},
     }
 
 
 def cpu_baseline():
-    """Oracle on the host cores: 1 batch entry x 2 heads of the prefill workload (1/64 of the
-    (batch, head) pairs, which are independent), scaled to the whole batch."""
+    """Oracle on the host cores: 1 batch entry x 4 heads of the prefill workload (1/32 of the
+    (batch, head) pairs, which are independent), repeated for about 12 s."""
     import torch
     from oracle import attention_oracle as orc
     b, s, h, d = 4, 8192, 32, 128
@@ -279,15 +331,19 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     pre = bench_prefill(a.steps, a.warmup)
+    peak = bench_mfma_peak(a.steps, a.warmup)
+    pre["roofline"]["measured_peak"] = peak["random_bf16"]["tflops"]
+    pre["roofline"]["frac_of_measured_peak"] = pre["tflops"] / peak["random_bf16"]["tflops"]
     out = {
         "metric": "fwd TFLOP/s (bf16, hdim128, causal, 8k)",
         "value": pre["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": pre["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": pre["ms"], "ms_min": pre["ms_min"], "timed_blocks": BLOCKS, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "flash_attn_func fwd bf16 batch=4 seqlen=8192 nheads=32 headdim=128 causal",
                    "global_batch": 4, "seq_len": 8192},
         "tokens_per_s": pre["tokens_per_s"],
         "roofline": pre["roofline"],
+        "mfma_peak": peak,
     }
     if not a.no_decode:
         dec = bench_decode(a.steps, a.warmup)

@@ -40,6 +40,7 @@ def units():
     u.append(("fa_decode.hip", "decode.o", []))
     u.append(("fa_aux.hip", "aux.o", []))
     u.append(("fa_rotary.hip", "rotary.o", []))
+    u.append(("fa_peak.hip", "peak.o", []))
     u.append(("fa_api.hip", "api.o", []))
     return u
 

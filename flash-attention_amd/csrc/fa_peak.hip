@@ -1,0 +1,65 @@
+// Matrix-pipe microbenchmark: what one MI355X sustains on v_mfma_f32_32x32x16_bf16 alone.
+//
+// The published dense bf16 peak (2.5 PFLOP/s) is 256 CUs x 4 SIMDs x one 32x32x16 MFMA per 32 cycles at
+// 2.4 GHz.  With every CU busy the part does not hold 2.4 GHz: the clock follows the switching activity
+// of the operands, so the sustained rate depends on the DATA.  This kernel runs nothing but independent
+// MFMAs (one wave per SIMD, four accumulators in rotation, operands resident in registers) on operands
+// that are either random bf16 values (sign, three exponents around 1, random mantissa) or zeros, and the
+// benchmark reports both next to the attention kernels' rates.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "fa_mi355x.h"
+
+namespace fa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 peak_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float peak_f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t peak_u32x4;
+
+__global__ void __launch_bounds__(256) mfma_peak_kernel(float* sink, int iters, int random_operands) {
+    peak_u32x4 a[4], b[4];
+    uint32_t st = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            uint32_t va = 0, vb = 0;
+            if (random_operands) {
+                for (int hlf = 0; hlf < 2; hlf++) {   // bf16: sign, exponent 125..127, 7 random mantissa bits
+                    st = st * 1664525u + 1013904223u;
+                    const uint32_t r = st >> 8;
+                    va |= (((r & 1u) << 15) | ((125u + (r >> 1) % 3u) << 7) | ((r >> 4) & 0x7fu)) << (16 * hlf);
+                    st = st * 1664525u + 1013904223u;
+                    const uint32_t q = st >> 8;
+                    vb |= (((q & 1u) << 15) | ((118u + (q >> 1) % 3u) << 7) | ((q >> 4) & 0x7fu)) << (16 * hlf);
+                }
+            }
+            a[i][e] = va;
+            b[i][e] = vb;
+        }
+    peak_f32x16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(peak_bf16x8, a[j & 3]),
+                                                                 __builtin_bit_cast(peak_bf16x8, b[(j >> 2) & 3]), acc[j & 3], 0, 0, 0);
+    }
+    float res = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) res += acc[i][0] + acc[i][9];
+    if (res == 1.2345e-30f) *sink = res;        // keeps the accumulators alive; never true in practice
+}
+
+}  // namespace fa
+
+extern "C" int fa_mfma_peak(float* sink, int32_t iters, int32_t random_operands, int64_t* flops, void* hip_stream) {
+    if (!sink || iters <= 0 || !flops) return 1;
+    const int grid = 1024;                      // four workgroups of 4 waves per CU: every SIMD holds 4 waves
+    hipLaunchKernelGGL(fa::mfma_peak_kernel, dim3(grid), dim3(256), 0, (hipStream_t)hip_stream, sink, iters, random_operands);
+    *flops = (int64_t)grid * 4 * iters * 16 * 32768LL;
+    return (int)hipGetLastError();
+}

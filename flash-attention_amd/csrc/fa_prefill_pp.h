@@ -272,6 +272,60 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
             for (int nb = 0; nb < C::NB; nb++) mask_acc16(s_acc[nb], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
         }
+        if constexpr (!DROPOUT) {
+            // The tile is exponentiated against the reference max the row already has, and only the
+            // tile's row sum is looked at afterwards: at most 2^14 means no probability above 2^14 (safe
+            // in fp16 / bf16 and in the fp32 sums), so the reference stays and no row max is formed.
+            // A larger or non-finite sum in any row of the wave (always the case while a row has no
+            // reference: -inf makes every exponent +inf or NaN) takes the rare branch, which forms the
+            // exact row max from the untouched scores, moves the reference under the usual rule and
+            // exponentiates again.
+            auto exp_tile = [&](float msc) -> float {
+                float suma = 0.f, sumb = 0.f;
+#pragma unroll
+                for (int t16 = 0; t16 < C::PT; t16++) {
+                    const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
+                    u32x4 pk;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float e0 = fast_exp2(s_acc[nb][r8 + 2 * e] * sl2 - msc);
+                        const float e1 = fast_exp2(s_acc[nb][r8 + 2 * e + 1] * sl2 - msc);
+                        suma += e0;
+                        sumb += e1;
+                        pk[e] = pack2<T>(e0, e1);
+                    }
+                    pf[t16] = __builtin_bit_cast(v8, pk);
+                }
+                return suma + sumb;
+            };
+            float tsum = exp_tile(m_run * sl2);
+            float corr = 1.f;
+            if (__builtin_amdgcn_ballot_w64(!(tsum <= 16384.f)) != 0) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int nb = 0; nb < C::NB; nb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) mx = fmaxf(mx, s_acc[nb][r]);
+                mx = xhalf_max(mx);
+                // lazy reference max: move it only when the tile max exceeds it by more than 2^8 (exp2 domain)
+                const bool move = (mx - m_run) * sl2 > 8.f;       // false for NaN (-inf - -inf)
+                const float m_new = move ? mx : m_run;
+                corr = move ? fast_exp2((m_run - m_new) * sl2) : 1.f;   // m_run = -inf -> 0
+                l_run *= corr;
+                m_run = m_new;
+                tsum = exp_tile((m_run == -INFINITY) ? 0.f : m_run * sl2);
+            }
+            l_run += tsum;
+            // (tested on corr itself, not on a flag set in the branch above: with a flag the compiler
+            // merges this block into that branch and copies all of o_acc around it on every tile)
+            if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
+#pragma unroll
+                for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
+            }
+            return;
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int nb = 0; nb < C::NB; nb++)

@@ -236,6 +236,15 @@ int fa_varlen_bwd(const fa_bwd_params *p, void *hip_stream);
 /* sizeof(fa_bwd_params) as compiled into the library. */
 int32_t fa_sizeof_bwd_params(void);
 
+/*
+ * Matrix-pipe microbenchmark (measurement aid; no counterpart in the reference): launches a kernel that
+ * executes only independent v_mfma_f32_32x32x16_bf16 instructions on every SIMD of the device, `iters`
+ * x 16 per wave, on random bf16 operands (random_operands != 0) or on zeros, and writes the number of
+ * floating-point operations of the launch to *flops.  The caller times the launch on `hip_stream`.
+ * `sink` is 4 bytes of device memory (never written in practice).
+ */
+int fa_mfma_peak(float *sink, int32_t iters, int32_t random_operands, int64_t *flops, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

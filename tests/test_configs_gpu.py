@@ -130,14 +130,17 @@ def test_config5_decode_kvcache_rotary():
     before_v = {i: vc[i, : int(lens[i]) + 2].cpu() for i in sample}
     lens_d = lens.to(DEV)
     fa = _fa()
-    out = fa.flash_attn_with_kvcache(q, kc, vc, kn, vn, cos.to(DEV), sin.to(DEV), lens_d, causal=True,
-                                     rotary_interleaved=True)
-    assert not torch.isnan(out).any()
+    # the native entry point behind flash_attn_with_kvcache, which also returns the log-sum-exp
+    # (mha_fwd_kvcache, csrc/flash_attn/flash_api.cpp:1278)
+    import flash_attn._native as nat
+    out, lse = nat.fwd_kvcache(q, kc, vc, kn, vn, lens_d, cos.to(DEV), sin.to(DEV), None, None, d ** -0.5, True, -1, -1,
+                               True, 0)
+    assert not torch.isnan(out).any() and lse.shape == (b, h, 1)
     for i in sample:
         L = int(lens[i])
-        o_ref, _, k_ref, v_ref = orc.kvcache_forward(q[i:i + 1].cpu(), before_k[i][None], before_v[i][None],
-                                                     kn[i:i + 1].cpu(), vn[i:i + 1].cpu(), cos, sin,
-                                                     torch.tensor([L], dtype=torch.int32), causal=True)
+        o_ref, l_ref, k_ref, v_ref = orc.kvcache_forward(q[i:i + 1].cpu(), before_k[i][None], before_v[i][None],
+                                                         kn[i:i + 1].cpu(), vn[i:i + 1].cpu(), cos, sin,
+                                                         torch.tensor([L], dtype=torch.int32), causal=True)
         o_pt, _, _, _ = orc.kvcache_forward(q[i:i + 1].cpu(), before_k[i][None], before_v[i][None],
                                             kn[i:i + 1].cpu(), vn[i:i + 1].cpu(), cos, sin,
                                             torch.tensor([L], dtype=torch.int32), causal=True, upcast=False,
@@ -145,6 +148,7 @@ def test_config5_decode_kvcache_rotary():
         ok, err, bound = orc.tolerance_ok(out[i:i + 1].cpu(), o_ref, o_pt, 3.0, 1e-5)
         _say("   batch %d (len %d): err %.3e bound %.3e" % (i, L, err, bound))
         assert ok
+        assert orc.lse_ok(lse[i:i + 1].cpu(), l_ref, 1e-3)[0]                    # persistent kernel + merge
         assert torch.equal(vc[i, : L + 2].cpu(), v_ref[0])                       # V rows bit-exact
         assert torch.allclose(kc[i, : L + 2].cpu().float(), k_ref[0].float(), rtol=1e-3, atol=1e-3)
     # the appended V row of EVERY batch entry is the new value, bit for bit

@@ -1,0 +1,127 @@
+"""Log-sum-exp of the KV-cache path against the oracle (1e-3 relative, infinities exact).
+
+flash_attn_with_kvcache returns only `out`; the native entry point behind it returns
+[out, softmax_lse] like mha_fwd_kvcache (csrc/flash_attn/flash_api.cpp:1278).  Each case below names
+the kernel it is sized to reach: the persistent ticket-scheduled decode kernel with its merge of
+the partial results, the one-workgroup-per-chunk decode kernel (split and unsplit), and the tiled
+kernel in its split form (more than 16 packed query rows)."""
+import math
+import sys
+
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def _nat():
+    import flash_attn._native as nat
+    return nat
+
+
+def _gen(shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g).to(dtype)
+
+
+def _run(q, kc, vc, lens, kn=None, vn=None, cos=None, sin=None, causal=False, window=(-1, -1), num_splits=0,
+         interleaved=True):
+    nat = _nat()
+    d = q.shape[-1]
+    dev = lambda t: None if t is None else t.to(DEV)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    out, lse = nat.fwd_kvcache(dev(q), kc_d, vc_d, dev(kn), dev(vn), dev(lens), dev(cos), dev(sin), None, None,
+                               d ** -0.5, causal, window[0], window[1], interleaved, num_splits)
+    o_ref, l_ref, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, causal=causal, window_size=window,
+                                             rotary_interleaved=interleaved)
+    o_pt, _, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, causal=causal, window_size=window,
+                                        rotary_interleaved=interleaved, upcast=False, reorder_ops=True)
+    ok, err, bound = orc.tolerance_ok(out.cpu(), o_ref, o_pt, 3.0, 1e-5)
+    assert ok, (err, bound)
+    assert lse.shape == (q.shape[0], q.shape[2], q.shape[1])
+    ok, rel = orc.lse_ok(lse.cpu(), l_ref, 1e-3)
+    assert ok, rel
+    return lse.cpu(), l_ref
+
+
+@pytest.mark.parametrize("with_new", [False, True])
+def test_lse_persistent_decode_and_merge(with_new):
+    """One decode step over caches large enough for the ticket-scheduled kernel (it takes over from
+    about 4 million cached key rows per launch: 8 x 32768 x 16 here, chunks of 1024 keys): sequences
+    with many complete chunks plus a ragged remainder, one chunk plus a few keys, less than one chunk,
+    and an empty cache.  Every batch entry is checked against the oracle on its own slice."""
+    _say("kvcache_lse persistent", with_new)
+    nat = _nat()
+    dtype, d, cap, b, h = torch.bfloat16, 64, 32768, 8, 16
+    torch.manual_seed(5)
+    kc = torch.randn(b, cap, h, d, device=DEV, dtype=dtype)
+    vc = torch.randn(b, cap, h, d, device=DEV, dtype=dtype)
+    q = torch.randn(b, 1, h, d, device=DEV, dtype=dtype)
+    lens = torch.tensor([cap - 1, 1100, 3000, 5, 0, 20000, 1024, 2047], dtype=torch.int32)
+    kn = vn = cos = sin = None
+    if with_new:
+        kn = torch.randn(b, 1, h, d, device=DEV, dtype=dtype)
+        vn = torch.randn(b, 1, h, d, device=DEV, dtype=dtype)
+        cos, sin = orc.rotary_table(cap, d, dtype=dtype)
+    before = {i: (kc[i, : int(lens[i]) + 2].cpu(), vc[i, : int(lens[i]) + 2].cpu()) for i in range(b)}
+    # the plan the library makes for this call must be the persistent one, or the test proves nothing
+    p = nat.FaFwdParams()
+    p.b, p.h, p.h_k, p.seqlen_q, p.seqlen_k, p.d, p.dtype = b, h, h, 1, cap, d, 1
+    p.is_seqlens_k_cumulative = 0
+    p.softmax_scale = d ** -0.5
+    p.window_left = p.window_right = -1
+    for name in ("q", "k", "v", "o", "softmax_lse", "work_counter", "cu_seqlens_k"):
+        setattr(p, name, 256)          # non-null placeholders: planning reads no memory
+    import ctypes
+    n = ctypes.c_int32(0)
+    assert nat.lib.fa_plan_splits(ctypes.byref(p), 2, ctypes.byref(n)) == 0
+    assert n.value == cap // 1024 + 2, n.value      # 32 complete-chunk slots + 2 remainder slots of 512 keys
+    dev = lambda t: None if t is None else t.to(DEV)
+    out, lse = nat.fwd_kvcache(q, kc, vc, kn, vn, lens.to(DEV), dev(cos), dev(sin), None, None, d ** -0.5, True, -1, -1,
+                               True, 0)
+    for i in range(b):
+        L = torch.tensor([int(lens[i])], dtype=torch.int32)
+        sl = lambda t: None if t is None else t[i:i + 1].cpu()
+        args = (q[i:i + 1].cpu(), before[i][0][None], before[i][1][None], sl(kn), sl(vn), cos, sin, L)
+        o_ref, l_ref, _, _ = orc.kvcache_forward(*args, causal=True)
+        o_pt, _, _, _ = orc.kvcache_forward(*args, causal=True, upcast=False, reorder_ops=True)
+        ok, err, bound = orc.tolerance_ok(out[i:i + 1].cpu(), o_ref, o_pt, 3.0, 1e-5)
+        assert ok, (i, err, bound)
+        ok, rel = orc.lse_ok(lse[i:i + 1].cpu(), l_ref, 1e-3)
+        _say("   batch %d (len %d): err %.3e bound %.3e lse rel %.3e" % (i, int(lens[i]), err, bound, rel))
+        assert ok, (i, rel)
+    if not with_new:
+        assert torch.isposinf(lse[4]).all() and (out[4] == 0).all()      # empty cache, nothing appended
+
+
+@pytest.mark.parametrize("num_splits", [1, 4])
+def test_lse_decode_kernel_one_workgroup_per_chunk(num_splits):
+    """Explicit split counts take the one-workgroup-per-chunk decode kernel (unsplit, and split with
+    the stand-alone merge); the empty sequence sees no key: lse = +inf, out = 0."""
+    _say("kvcache_lse decode", num_splits)
+    dtype, d, cap, b, h, hk = torch.float16, 64, 1500, 3, 8, 2
+    q = _gen((b, 2, h, d), dtype, 1); kc = _gen((b, cap, hk, d), dtype, 2); vc = _gen((b, cap, hk, d), dtype, 3)
+    lens = torch.tensor([1500, 0, 333], dtype=torch.int32)
+    lse, l_ref = _run(q, kc, vc, lens, num_splits=num_splits)
+    assert torch.isposinf(lse[1]).all() and torch.isposinf(l_ref[1]).all()
+
+
+def test_lse_tiled_split_kernel():
+    """40 query rows x 4 grouped heads do not fit the decode kernel's 16 packed rows: the tiled kernel
+    runs in its split form.  With a causal mask and 10 cached keys the first rows of the second
+    sequence see nothing."""
+    _say("kvcache_lse tiled split")
+    dtype, d, cap, b, h, hk = torch.bfloat16, 128, 3000, 2, 8, 2
+    q = _gen((b, 40, h, d), dtype, 1); kc = _gen((b, cap, hk, d), dtype, 2); vc = _gen((b, cap, hk, d), dtype, 3)
+    lens = torch.tensor([2900, 10], dtype=torch.int32)
+    lse, l_ref = _run(q, kc, vc, lens, causal=True, num_splits=3)
+    assert torch.isposinf(l_ref[1, :, :30]).all() and torch.isposinf(lse[1, :, :30]).all()
+    _run(q, kc, vc, lens, causal=True, window=(100, 0), num_splits=0)
