@@ -8,6 +8,7 @@
 #include <string>
 #include <vector>
 #include <algorithm>
+#include <mutex>
 #include "fa_prefill.h"
 #include "fa_bwd.h"
 #include "fa_launch.h"
@@ -253,6 +254,35 @@ static int run_bwd(const fa_bwd_params* p, bool varlen, hipStream_t stream) {
 
 using namespace fa;
 
+// ------------------------------------------------------------------------------------------------
+// Device memory owned by the library, for the one entry point that must not allocate
+// (fa_fwd_kvcache_noalloc): the ticket word, lse_accum and o_accum of a split launch live in this array
+// instead of caller-provided buffers.  Every GPU the library runs on holds its own copy at its own
+// address until the process ends; `scratch` itself is only the host-side name of the symbol, the
+// address kernels may use is looked up once per device.
+// ------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[FA_NOALLOC_SCRATCH_BYTES];
+
+static const int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];          // device address of `scratch`, per device (0: not looked up yet)
+static std::mutex g_scratch_mutex;
+
+// address of the current device's copy of `scratch`, or nullptr (g_err says why)
+static unsigned char* scratch_of_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { fail_hip((int)e, "hipGetDevice"); return nullptr; }
+    if (dev < 0 || dev >= kMaxDevices) { fail("device index out of range for the no-allocation entry point"); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));      // resolves the symbol on the CURRENT device
+        if (e != hipSuccess || !ptr) { fail_hip((int)e, "hipGetSymbolAddress(scratch)"); return nullptr; }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return static_cast<unsigned char*>(g_scratch_ptr[dev]);
+}
+
 extern "C" {
 
 const char* fa_last_error(void) { return g_err.c_str(); }
@@ -351,6 +381,32 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
         if (int e = launch_append_kv(kp, reset_in_append ? kp.work_counter : nullptr, stream)) return fail_hip(e, "append_kv kernel launch");
     }
     return run_attention(kp, stream, reset_in_append);
+}
+
+int fa_fwd_kvcache_noalloc(const fa_fwd_params* p, void* hip_stream) {
+    g_err.clear();
+    if (!p) return fail("params is NULL");
+    unsigned char* base = scratch_of_current_device();
+    if (!base) return 2;
+    // layout inside the array: [0, 256) ticket words, then lse_accum, then o_accum (256-byte aligned)
+    fa_fwd_params q = *p;
+    q.work_counter = reinterpret_cast<int32_t*>(base);
+    q.o_accum = nullptr;
+    q.lse_accum = nullptr;
+    if (int r = check_common(&q)) return r;
+    const int splits = plan(q, q.p_dropout == 0.f).splits;
+    if (splits > 1) {
+        auto up256 = [](size_t x) { return (x + 255) / 256 * 256; };
+        const size_t rows = (size_t)q.b * q.h * q.seqlen_q;
+        const size_t lse_bytes = up256((size_t)splits * rows * sizeof(float));
+        const size_t o_bytes = (size_t)splits * rows * (size_t)((q.d + 31) / 32 * 32) * sizeof(float);
+        if (256 + lse_bytes + o_bytes > (size_t)FA_NOALLOC_SCRATCH_BYTES)
+            return fail("fa_fwd_kvcache_noalloc: the split accumulators of this problem exceed FA_NOALLOC_SCRATCH_BYTES; "
+                        "use fa_fwd_kvcache with caller-provided o_accum / lse_accum, or request num_splits = 1");
+        q.lse_accum = reinterpret_cast<float*>(base + 256);
+        q.o_accum = reinterpret_cast<float*>(base + 256 + lse_bytes);
+    }
+    return fa_fwd_kvcache(&q, hip_stream);
 }
 
 int32_t fa_sizeof_rotary_params(void) { return (int32_t)sizeof(fa_rotary_params); }

@@ -83,7 +83,7 @@ def _load():
             "(hipcc, gfx950). There is no fallback implementation." % _LIB_PATH)
     lib = ctypes.CDLL(_LIB_PATH)
     P = ctypes.POINTER(FaFwdParams)
-    for name in ("fa_fwd", "fa_varlen_fwd", "fa_fwd_kvcache"):
+    for name in ("fa_fwd", "fa_varlen_fwd", "fa_fwd_kvcache", "fa_fwd_kvcache_noalloc"):
         f = getattr(lib, name)
         f.argtypes = [P, ctypes.c_void_p]
         f.restype = ctypes.c_int
@@ -481,9 +481,12 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
 
 def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_, cache_batch_idx_,
                 out_, softmax_scale, is_causal, window_size_left, window_size_right,
-                is_rotary_interleaved, num_splits):
+                is_rotary_interleaved, num_splits, no_alloc=False, lse_=None):
     """KV-cache forward with optional append + rotary; mirrors mha_fwd_kvcache
-    (flash_api.cpp:1038-1279).  Returns [out, softmax_lse]."""
+    (flash_api.cpp:1038-1279).  Returns [out, softmax_lse].
+
+    no_alloc=True calls fa_fwd_kvcache_noalloc: the split accumulators and the ticket words live in
+    the library's own device array, and with out_ and lse_ given nothing is allocated here either."""
     q_dtype = q.dtype
     dt = _dtype_code(q_dtype)
     _check(kcache.dtype == q_dtype, "query and key must have the same dtype")
@@ -521,7 +524,13 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
     head_size = q_padded.shape[-1]
 
     with torch.cuda.device(q.device):
-        softmax_lse = torch.empty((batch_size, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
+        if lse_ is not None:
+            _check(lse_.dtype == torch.float32 and lse_.is_contiguous() and tuple(lse_.shape) == (batch_size, num_heads, seqlen_q),
+                   "lse_ must be a contiguous fp32 tensor of shape (batch_size, num_heads, seqlen_q)")
+            _check_device(lse_)
+            softmax_lse = lse_
+        else:
+            softmax_lse = torch.empty((batch_size, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
         p = FaFwdParams()
         p.q, p.k, p.v, p.o = q_padded.data_ptr(), kcache_padded.data_ptr(), vcache_padded.data_ptr(), out.data_ptr()
         p.softmax_lse = softmax_lse.data_ptr()
@@ -587,7 +596,9 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
             p.cache_batch_idx = cache_batch_idx_.data_ptr()
         _check(num_splits <= 128, "num_splits > 128 not supported")
         p.num_splits = max(int(num_splits), 0)
-        if seqlen_q > 0 and seqlen_k > 0:
+        if seqlen_q > 0 and seqlen_k > 0 and no_alloc:
+            _call(lib.fa_fwd_kvcache_noalloc, p, _stream(q.device))
+        elif seqlen_q > 0 and seqlen_k > 0:
             keep.append(_plan_and_alloc(p, 2, batch_size, num_heads, seqlen_q, head_size, q.device))
             _call(lib.fa_fwd_kvcache, p, _stream(q.device))
         else:

@@ -124,6 +124,23 @@ int fa_varlen_fwd(const fa_fwd_params *p, void *hip_stream);
 int fa_fwd_kvcache(const fa_fwd_params *p, void *hip_stream);
 
 /*
+ * fa_fwd_kvcache for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * mha_fwd_kvcache always allocates its split accumulators (flash_api.cpp:1241-1257).  Same arguments
+ * and results as fa_fwd_kvcache, except that p->o_accum, p->lse_accum and p->work_counter are ignored:
+ * the ticket words and the fp32 partial results of a split launch live in FA_NOALLOC_SCRATCH_BYTES of
+ * device memory that the library itself holds on every GPU it runs on (a static device array, kept
+ * until the process ends).  The call allocates and frees nothing.  A problem whose partials do not fit
+ * (splits x b x h x seqlen_q x (4 + 4 x d rounded up to 32) bytes + 256) is rejected with an error;
+ * num_splits = 1 always fits.  All calls on one GPU share the array: calls that overlap in time on the
+ * same GPU (two streams, two threads) race on it and must be serialised by the caller.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress): make one call before capturing a
+ * graph.
+ */
+#define FA_NOALLOC_SCRATCH_BYTES (48u << 20)
+int fa_fwd_kvcache_noalloc(const fa_fwd_params *p, void *hip_stream);
+
+/*
  * Resolves the split count the library will use for this problem, so that the caller can size
  * o_accum / lse_accum before the call (the reference does this inside mha_fwd / mha_fwd_kvcache,
  * flash_api.cpp:373-389, 1241-1257, with num_splits_heuristic :212-246; this library uses its
