@@ -283,6 +283,10 @@ static unsigned char* scratch_of_current_device() {
     return static_cast<unsigned char*>(g_scratch_ptr[dev]);
 }
 
+static __global__ void set_rng_state_kernel(uint64_t* dst, uint64_t seed, uint64_t offset) {
+    if (threadIdx.x == 0) { dst[0] = seed; dst[1] = offset; }
+}
+
 extern "C" {
 
 const char* fa_last_error(void) { return g_err.c_str(); }
@@ -407,6 +411,14 @@ int fa_fwd_kvcache_noalloc(const fa_fwd_params* p, void* hip_stream) {
         q.o_accum = reinterpret_cast<float*>(base + 256 + lse_bytes);
     }
     return fa_fwd_kvcache(&q, hip_stream);
+}
+
+int fa_set_rng_state(uint64_t* rng_state, uint64_t seed, uint64_t offset, void* hip_stream) {
+    g_err.clear();
+    if (!rng_state) return fail("rng_state is NULL");
+    hipLaunchKernelGGL(set_rng_state_kernel, dim3(1), dim3(64), 0, (hipStream_t)hip_stream, rng_state, seed, offset);
+    if (int e = (int)hipGetLastError()) return fail_hip(e, "rng state launch");
+    return 0;
 }
 
 int32_t fa_sizeof_rotary_params(void) { return (int32_t)sizeof(fa_rotary_params); }

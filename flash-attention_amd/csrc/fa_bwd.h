@@ -588,10 +588,6 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-template <typename K> static int bwd_set_smem(K kern, int bytes) {
-    return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 template <typename T, int D, int BN, int MINW, bool DROPOUT>
 int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
     typedef BwdDqCfg<T, D, BN> C;
@@ -600,7 +596,7 @@ int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
     const int64_t nblocks = xcd_rows_grid(false, kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k, kp.p.h / kp.p.h_k, nmb);
     if (nblocks == 0) return -2;
     auto kern = bwd_dq_kernel<T, D, BN, MINW, DROPOUT>;
-    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
+    if (int e = (int)FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
@@ -613,7 +609,7 @@ int launch_bwd_dkv3(const BwdKParams& kp, hipStream_t stream) {
     const int64_t nblocks = xcd_grid(xcd_strided(kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k), kp.p.b, kp.p.h_k, per_stream);
     if (nblocks == 0) return -2;
     auto kern = bwd_dkv3_kernel<T, D, BM, DPARTS, DROPOUT>;
-    if (int e = bwd_set_smem(kern, C::SMEM)) return e;
+    if (int e = (int)FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }

@@ -5,6 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include "fa_mi355x.h"
 
 namespace fa {
@@ -23,6 +24,21 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define FA_DEV __device__ __forceinline__
+
+// Lets `kern` use `bytes` of dynamic LDS.  The limit is a property of the kernel on a device, so it is
+// set on the first launch there and not again (each expansion of the macro has its own flags: one per
+// kernel instantiation and call site).
+#define FA_ALLOW_DYNAMIC_LDS(kern, bytes)                                                                  \
+    ([&]() -> hipError_t {                                                                                 \
+        static std::atomic<bool> done[64];                                                                 \
+        int dev = 0;                                                                                       \
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)                                      \
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (bytes)); \
+        if (done[dev].load(std::memory_order_acquire)) return hipSuccess;                                  \
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (bytes)); \
+        if (e == hipSuccess) done[dev].store(true, std::memory_order_release);                             \
+        return e;                                                                                          \
+    }())
 #define FA_LDS_PTR(T) __attribute__((address_space(3))) T*
 
 // Kernel-side view of one problem: the caller's description plus values the host derives once.

@@ -163,7 +163,9 @@ FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b
             if (row_valid && d0 < p.d) {
                 raw = ld_global16(qrow + d0);
                 if (kp.rotary_q && d0 < p.rotary_dim) {
-                    const int pos = si.sk_cache + ((p.is_causal || has_left || has_right) ? qi : 0);
+                    // (a full cache puts cache length + row past the cache: the table is only known to cover the
+                    // cache capacity, so the position stops at its last row)
+                    const int pos = min(si.sk_cache + ((p.is_causal || has_left || has_right) ? qi : 0), p.seqlen_k - 1);
                     const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
                     const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
                     float x[8];
@@ -359,7 +361,7 @@ static int launch_decode_t(const KParams& kp, hipStream_t stream) {
         const int resident = 256 * (D > 128 ? 1 : 2);          // workgroups the 256 CUs hold at once
         dim3 grid(total < resident ? total : resident), block(C::kThreads);
         auto kern = decode_persistent_kernel<T, D>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
         return (int)hipGetLastError();
@@ -367,12 +369,12 @@ static int launch_decode_t(const KParams& kp, hipStream_t stream) {
     dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b), block(C::kThreads);
     if (split) {
         auto kern = decode_kernel<T, D, true>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     } else {
         auto kern = decode_kernel<T, D, false>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     }

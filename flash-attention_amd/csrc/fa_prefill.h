@@ -100,7 +100,9 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
             if (valid && d0 < p.d) {
                 raw = ld_global16(qrow + d0);
                 if (kp.rotary_q && d0 < p.rotary_dim) {
-                    const int pos = si.sk_cache + ((p.is_causal || has_left || has_right) ? row : 0);
+                    // (a full cache puts cache length + row past the cache: the table is only known to cover the
+                    // cache capacity, so the position stops at its last row)
+                    const int pos = min(si.sk_cache + ((p.is_causal || has_left || has_right) ? row : 0), p.seqlen_k - 1);
                     const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
                     const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
                     float x[8];
@@ -325,17 +327,17 @@ int launch_prefill(KParams kp, hipStream_t stream) {
     hipError_t e;
     if (split) {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, true>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     } else if (kp.p.p_dropout > 0.f) {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, false, true>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     } else {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, false>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     }

@@ -91,6 +91,8 @@ def _load():
     lib.fa_plan_splits.restype = ctypes.c_int
     lib.fa_num_splits_heuristic_reference.argtypes = [ctypes.c_int32] * 4
     lib.fa_num_splits_heuristic_reference.restype = ctypes.c_int
+    lib.fa_set_rng_state.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_void_p]
+    lib.fa_set_rng_state.restype = ctypes.c_int
     lib.fa_last_error.argtypes = []
     lib.fa_last_error.restype = ctypes.c_char_p
     lib.fa_version.argtypes = []
@@ -161,25 +163,42 @@ def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+_NO_DROPOUT_STATE = {}     # device -> the (never read, never written) rng_state returned when p_dropout = 0
+
+
 def _dropout_state(p, p_dropout, return_softmax, gen_, batch, heads, seqlen_q, seqlen_k, dtype, device):
     """Seed / offset of the dropout mask taken from (and advancing) torch's generator for the device,
     like the reference does with its Philox state (flash_api.cpp:396-408), and the optional
-    probability tensor behind return_softmax (:351-357).  Returns (rng_state, s_dmask)."""
+    probability tensor behind return_softmax (:351-357).  Returns (rng_state, s_dmask).
+
+    Without dropout nothing is allocated: one placeholder tensor per device stands in for the
+    reference's empty rng_state.  With dropout the two words reach the device as arguments of a
+    one-thread kernel on the current stream (no pageable copy, no host synchronisation).  Under HIP
+    graph capture the generator cannot be advanced from the host per replay, so dropout is refused
+    there."""
     _check(0.0 <= p_dropout < 1.0, "p_dropout must be in [0, 1)")
-    rng_state = torch.empty((2,), dtype=torch.int64, device=device)
     s_dmask = None
     if return_softmax:
         _check(p_dropout > 0.0, "return_softmax is only supported when p_dropout > 0.0")
         s_dmask = torch.empty((batch, heads, _round_up(seqlen_q, 128), _round_up(seqlen_k, 128)), dtype=dtype, device=device)
         p.s_dmask, p.sdm_rows, p.sdm_cols = s_dmask.data_ptr(), s_dmask.shape[2], s_dmask.shape[3]
-    if p_dropout > 0.0:
-        gen = gen_ if gen_ is not None else torch.cuda.default_generators[device.index if device.index is not None
-                                                                       else torch.cuda.current_device()]
-        seed, offset = gen.initial_seed(), gen.get_offset()
-        gen.set_offset(offset + batch * heads * 32)
-        host = torch.tensor([ctypes.c_int64(seed).value, ctypes.c_int64(offset).value], dtype=torch.int64)
-        rng_state.copy_(host)
-        p.p_dropout, p.rng_state = p_dropout, rng_state.data_ptr()
+    if p_dropout <= 0.0:
+        key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+        if key not in _NO_DROPOUT_STATE:
+            _NO_DROPOUT_STATE[key] = torch.empty((2,), dtype=torch.int64, device=device)
+        return _NO_DROPOUT_STATE[key], s_dmask
+    _check(not torch.cuda.is_current_stream_capturing(),
+           "attention dropout cannot be captured in a HIP graph: its seed and offset come from the host-side generator")
+    rng_state = torch.empty((2,), dtype=torch.int64, device=device)
+    gen = gen_ if gen_ is not None else torch.cuda.default_generators[device.index if device.index is not None
+                                                                   else torch.cuda.current_device()]
+    seed, offset = gen.initial_seed(), gen.get_offset()
+    gen.set_offset(offset + batch * heads * 32)
+    rc = lib.fa_set_rng_state(ctypes.c_void_p(rng_state.data_ptr()), ctypes.c_uint64(seed & (2 ** 64 - 1)),
+                              ctypes.c_uint64(offset & (2 ** 64 - 1)), ctypes.c_void_p(_stream(device)))
+    if rc != 0:
+        raise RuntimeError(lib.fa_last_error().decode() or "libfa_mi355x: error %d" % rc)
+    p.p_dropout, p.rng_state = p_dropout, rng_state.data_ptr()
     return rng_state, s_dmask
 
 

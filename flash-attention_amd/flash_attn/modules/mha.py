@@ -114,6 +114,10 @@ class MHA(nn.Module):
         self.head_dim = self.embed_dim // num_heads
         qkv_dim = self.head_dim * (self.num_heads + 2 * self.num_heads_kv)
         if self.rotary_emb_dim > 0:
+            # the rotary kernels (stand-alone and inside the KV-cache call) move 16-byte granules of a pair
+            if self.rotary_emb_dim % 16 != 0 or self.rotary_emb_dim > self.head_dim:
+                raise ValueError("rotary_emb_dim must be divisible by 16 and at most head_dim (got %d for head_dim %d)"
+                                 % (self.rotary_emb_dim, self.head_dim))
             self.rotary_emb = RotaryEmbedding(self.rotary_emb_dim, base=rotary_emb_base, scale_base=rotary_emb_scale_base,
                                               interleaved=rotary_emb_interleaved, device=device)
         self.inner_attn = FlashSelfAttention(causal=causal, softmax_scale=softmax_scale, attention_dropout=dropout,
@@ -128,23 +132,19 @@ class MHA(nn.Module):
         return torch.empty(batch_size, max_seqlen, 2, self.num_heads_kv, self.head_dim, dtype=dtype,
                            device=self.out_proj.weight.device)
 
-    def _rotate_packed(self, q, k_part, nk, cu_seqlens, max_seqlen, ret):
-        """Rotary on packed (total, ...) q and k: every sequence starts at position 0."""
+    def _rotate_packed(self, x, cu_seqlens, max_seqlen):
+        """Rotary on packed heads x (total, heads, head_dim), every sequence starting at position 0.
+        Returns the rotated tensor.  When gradients are recorded the rotation is out of place and the
+        caller must go on with the RETURNED tensor: it carries the backward (the conjugate rotation),
+        which an in-place write into a view of the projection's output would bypass.  Without
+        gradients x is rotated in place and returned."""
         from flash_attn.layers.rotary import apply_rotary_emb
         assert self.rotary_emb.scale is None, "packed input does not support xPos"
-        self.rotary_emb._update_cos_sin_cache(max_seqlen, device=q.device, dtype=q.dtype)
-        cos, sin = self.rotary_emb._cos_cached, self.rotary_emb._sin_cached
-        total = q.shape[0]
-        if ret is not None:      # qkv packed: q and k heads are one run of 2h heads per token
-            qk = ret.view(total, 3 * self.num_heads, self.head_dim)[:, : 2 * self.num_heads]
-            apply_rotary_emb(qk, cos, sin, interleaved=self.rotary_emb.interleaved, inplace=True, cu_seqlens=cu_seqlens,
-                             max_seqlen=max_seqlen)
-            return ret
-        apply_rotary_emb(q, cos, sin, interleaved=self.rotary_emb.interleaved, inplace=True, cu_seqlens=cu_seqlens,
-                         max_seqlen=max_seqlen)
-        apply_rotary_emb(k_part[:, 0], cos, sin, interleaved=self.rotary_emb.interleaved, inplace=True,
-                         cu_seqlens=cu_seqlens, max_seqlen=max_seqlen)
-        return None
+        self.rotary_emb._update_cos_sin_cache(max_seqlen, device=x.device, dtype=x.dtype)
+        inplace = not (torch.is_grad_enabled() and x.requires_grad)
+        return apply_rotary_emb(x, self.rotary_emb._cos_cached, self.rotary_emb._sin_cached,
+                                interleaved=self.rotary_emb.interleaved, inplace=inplace, cu_seqlens=cu_seqlens,
+                                max_seqlen=max_seqlen)
 
     def _update_kv_cache(self, kv, inference_params):
         assert self.layer_idx is not None, "Generation requires layer_idx in the constructor"
@@ -194,14 +194,21 @@ class MHA(nn.Module):
             if self.num_heads_kv == self.num_heads:
                 qkv = qkv.view(total, 3, self.num_heads, self.head_dim)
                 if self.rotary_emb_dim > 0:
-                    qkv = self._rotate_packed(qkv[:, 0], qkv[:, :2], 2, cu_seqlens, max_seqlen, qkv)
+                    # q and k heads of a token are one run of 2 h heads: one launch rotates both
+                    qk = self._rotate_packed(qkv.view(total, 3 * self.num_heads, self.head_dim)[:, : 2 * self.num_heads],
+                                             cu_seqlens, max_seqlen)
+                    if qk.data_ptr() != qkv.data_ptr():      # rotated out of place: rebuild the packed tensor
+                        qkv = torch.cat([qk.view(total, 2, self.num_heads, self.head_dim), qkv[:, 2:]], dim=1)
                 context = self.inner_attn(qkv, **kw)
             else:
                 nq = self.num_heads * self.head_dim
                 q = qkv[..., :nq].reshape(total, self.num_heads, self.head_dim)
                 kv = qkv[..., nq:].reshape(total, 2, self.num_heads_kv, self.head_dim)
                 if self.rotary_emb_dim > 0:
-                    self._rotate_packed(q, kv[:, :1], 1, cu_seqlens, max_seqlen, None)
+                    q = self._rotate_packed(q, cu_seqlens, max_seqlen)
+                    k = self._rotate_packed(kv[:, 0], cu_seqlens, max_seqlen)
+                    if k.data_ptr() != kv.data_ptr():
+                        kv = torch.stack([k, kv[:, 1]], dim=1)
                 context = self.inner_cross_attn(q, kv, cu_seqlens_k=cu_seqlens, max_seqlen_k=max_seqlen, **kw)
             return self.out_proj(context.reshape(total, self.embed_dim))
         if inference_params is None:
@@ -212,9 +219,8 @@ class MHA(nn.Module):
             rotary_max_seqlen = inference_params.max_seqlen
         batch, seqlen = x.shape[:2]
         qkv = self.Wqkv(x)
-        # the fused rotary + append path needs something cached and a rotary_dim the kernel takes
-        fused = (inference_params is not None and inference_params.seqlen_offset > 0
-                 and self.rotary_emb_dim > 0 and self.rotary_emb_dim % 16 == 0)
+        # the fused rotary + append path needs something cached
+        fused = inference_params is not None and inference_params.seqlen_offset > 0 and self.rotary_emb_dim > 0
         if self.num_heads_kv == self.num_heads:
             qkv = qkv.view(batch, seqlen, 3, self.num_heads, self.head_dim)
             if fused:

@@ -1,22 +1,21 @@
-"""Decoding-side glue around `flash_attn_with_kvcache`: the per-generation state that attention layers
-read, the token loop, and HIP-graph capture of one decoding step.
+"""Decoding-side glue around `flash_attn_with_kvcache`: the state attention layers read while a model
+generates, token selection, the token loop, and replay of one decoding step from a HIP graph.
 
-Mirrors the parts of the reference's flash_attn/utils/generation.py that sit directly on the
-attention path: `InferenceParams` (:18-35), the top-k / top-p sampling helpers (:40-97), `decode`
-(:100-201), `allocate_inference_cache` (:585-601) and the graph cache (`DecodingCGCache`,
-`update_graph_cache`, `capture_graph`, :604-739).  A "model" here is any callable
-`model(input_ids, position_ids=None, inference_params=None, num_last_tokens=0)` that returns an
-object with a `.logits` tensor of shape (batch, tokens, vocab), as the reference's GPT models do.
+Covers what the reference keeps in flash_attn/utils/generation.py on the attention path:
+`InferenceParams` (:18-35), the top-k / top-p helpers and `sample` (:40-97), `decode` (:100-201) with
+the same arguments and result type, and the graph cache behind `cg=True` (:604-739).  A "model" is
+any callable `model(input_ids, position_ids=None, inference_params=None, num_last_tokens=0)` whose
+result has a `.logits` tensor of shape (batch, tokens, vocab), as the reference's GPT models do.
 
-What makes the captured step valid: inside the attention call nothing depends on device values on
-the host (no synchronisation), the split plan is a function of the cache SHAPE only, and the
-per-sequence lengths are read by the kernels from `lengths_per_sample`, which `run` updates in place
-before each replay.
+Why one captured step stays valid for every later step: nothing inside the attention call depends
+on device values on the host (no synchronisation), its split plan is a function of the cache SHAPE,
+and the kernels read the true per-sequence lengths from `lengths_per_sample`, which is rewritten on
+the device before each replay.  The step is captured at the largest cache fill, so every launch in
+the graph is sized for the longest sequence it will ever see.
 """
-import gc
 from collections import namedtuple
 from dataclasses import dataclass, field
-from typing import Callable, Optional
+from typing import Optional
 
 import torch
 from torch import Tensor
@@ -27,9 +26,9 @@ SampleDecoderOnlyOutput = namedtuple("SampleDecoderOnlyOutput", ["sequences", "s
 
 @dataclass
 class InferenceParams:
-    """State shared by the attention layers of a model while it generates: the cache geometry, how
-    many tokens every sequence already holds (`seqlen_offset`, or per sequence `lengths_per_sample`),
-    and the per-layer caches `key_value_memory_dict[layer_idx]` of shape
+    """What the attention layers of a generating model share: the cache geometry, how many tokens
+    every sequence already holds (`seqlen_offset`, or per sequence `lengths_per_sample`), and the
+    per-layer caches `key_value_memory_dict[layer_idx]`, each
     (max_batch_size, max_seqlen, 2, nheads_kv, headdim)."""
 
     max_seqlen: int
@@ -40,205 +39,221 @@ class InferenceParams:
     lengths_per_sample: Optional[Tensor] = None
 
     def reset(self, max_seqlen, max_batch_size):
-        self.max_seqlen = max_seqlen
-        self.max_batch_size = max_batch_size
-        self.seqlen_offset = 0
+        self.max_seqlen, self.max_batch_size, self.seqlen_offset = max_seqlen, max_batch_size, 0
         if self.lengths_per_sample is not None:
             self.lengths_per_sample.zero_()
 
 
+# ------------------------------------------------------------------------------------------------
+# token selection
+# ------------------------------------------------------------------------------------------------
+_NEG_INF = float("-inf")
+
+
 def modify_logits_for_top_k_filtering(logits, top_k):
-    """In place: everything below the k-th largest logit of a row becomes -inf."""
-    kth = torch.topk(logits, top_k)[0][..., -1, None]
-    logits.masked_fill_(logits < kth, float("-inf"))
+    """In place: a row keeps its top_k largest logits, the rest become -inf."""
+    smallest_kept = logits.topk(top_k, dim=-1).values[..., -1:]
+    logits.masked_fill_(logits < smallest_kept, _NEG_INF)
 
 
 def modify_logits_for_top_p_filtering(logits, top_p):
-    """In place: the low-probability tail whose total mass is at most 1 - top_p becomes -inf."""
-    if top_p <= 0.0 or top_p >= 1.0:
+    """In place: the least likely tokens whose probabilities add up to at most 1 - top_p become -inf."""
+    if not 0.0 < top_p < 1.0:
         return
-    sorted_logits, sorted_indices = torch.sort(logits, descending=False)
-    drop_sorted = sorted_logits.softmax(dim=-1).cumsum(dim=-1) <= (1 - top_p)
-    drop = drop_sorted.scatter(1, sorted_indices, drop_sorted)
-    logits.masked_fill_(drop, float("-inf"))
+    ascending, order = logits.sort(dim=-1)
+    tail = ascending.softmax(dim=-1).cumsum(dim=-1) <= 1.0 - top_p        # in sorted order
+    logits.masked_fill_(torch.zeros_like(tail).scatter_(-1, order, tail), _NEG_INF)
+
+
+def _draw(logits):
+    return torch.multinomial(logits.softmax(dim=-1), num_samples=1).squeeze(-1)
 
 
 def sample(logits, top_k=1, top_p=0.0, temperature=1.0):
-    """logits (batch, vocab) -> token ids (batch,).  top_k = 1 is greedy; top_k = 0 samples from the
-    whole vocabulary; top-k is applied before top-p."""
+    """logits (batch, vocab) -> token ids (batch,).  top_k = 1 is greedy, top_k = 0 draws from the whole
+    vocabulary; temperature and top-p apply after the top-k cut."""
     if top_k == 1:
         return logits.argmax(dim=-1)
-    if top_p > 0.0:
-        assert top_p <= 1.0, "top-p should be in (0, 1]."
+    assert top_p <= 1.0, "top-p should be in (0, 1]."
     if top_k > 0:
-        top_k = min(top_k, logits.size(-1))
-        logits_top, indices = torch.topk(logits, top_k, dim=-1)
+        kept, ids = logits.topk(min(top_k, logits.shape[-1]), dim=-1)
         if temperature != 1.0:
-            logits_top /= temperature
-        modify_logits_for_top_p_filtering(logits_top, top_p)
-        pick = torch.multinomial(torch.softmax(logits_top, dim=-1), num_samples=1).squeeze(dim=-1)
-        return indices[torch.arange(indices.shape[0], device=indices.device), pick]
-    logits_top = logits / temperature if temperature != 1.0 else logits.clone()
-    modify_logits_for_top_p_filtering(logits_top, top_p)
-    return torch.multinomial(torch.softmax(logits_top, dim=-1), num_samples=1).squeeze(dim=-1)
+            kept = kept / temperature
+        modify_logits_for_top_p_filtering(kept, top_p)
+        return ids.gather(-1, _draw(kept).unsqueeze(-1)).squeeze(-1)
+    scaled = logits / temperature if temperature != 1.0 else logits.clone()
+    modify_logits_for_top_p_filtering(scaled, top_p)
+    return _draw(scaled)
+
+
+# ------------------------------------------------------------------------------------------------
+# one decoding step as a HIP graph
+# ------------------------------------------------------------------------------------------------
+def allocate_inference_cache(max_batch_size, max_seqlen, nheads, headdim, layers, device, dtype=torch.float16):
+    """{layer_idx: (max_batch_size, max_seqlen, 2, nheads, headdim)}; `layers` an int or an iterable."""
+    assert dtype in (torch.float16, torch.bfloat16, torch.float32)
+    ids = range(layers) if isinstance(layers, int) else layers
+    return {i: torch.empty(max_batch_size, max_seqlen, 2, nheads, headdim, device=device, dtype=dtype) for i in ids}
+
+
+class DecodeStepGraph:
+    """`model` applied to (batch_size, n_tokens) new tokens against the KV caches in `state`, captured
+    once and replayed.  Owns the static input buffers of the graph; the output buffer belongs to the
+    graph's memory pool, so `run` hands out a copy."""
+
+    def __init__(self, model, state: InferenceParams, batch_size, n_tokens=1, pool=None, warmups=2):
+        device = next(iter(model.parameters())).device
+        self.state = state
+        self.tokens = torch.zeros(batch_size, n_tokens, dtype=torch.long, device=device)
+        self.positions = torch.zeros(batch_size, n_tokens, dtype=torch.long, device=device)
+        self.graph = torch.cuda.CUDAGraph()
+        call = lambda: model(self.tokens, position_ids=self.positions, inference_params=state,
+                             num_last_tokens=n_tokens).logits
+        # capture at the largest fill the cache allows; the caller's fill level is put back afterwards
+        fill = state.seqlen_offset
+        state.seqlen_offset = state.max_seqlen - n_tokens
+        state.lengths_per_sample.fill_(state.seqlen_offset)
+        try:
+            warm = torch.cuda.Stream()                          # default priority
+            warm.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(warm):
+                for _ in range(warmups):
+                    call()
+            warm.synchronize()
+            torch.cuda.current_stream().wait_stream(warm)
+            with torch.cuda.graph(self.graph, pool=pool):
+                self.logits = call()
+        finally:
+            state.seqlen_offset = fill
+            state.lengths_per_sample.fill_(fill)
+
+    def run(self, tokens, positions, lengths):
+        """lengths: an int or a (batch,) tensor: tokens every sequence holds before this step."""
+        if torch.is_tensor(lengths):
+            self.state.lengths_per_sample.copy_(lengths)
+        else:
+            self.state.lengths_per_sample.fill_(lengths)
+        self.tokens.copy_(tokens)
+        self.positions.copy_(positions)
+        self.graph.replay()
+        return self.logits.clone()
+
+
+class GraphedDecoder:
+    """The KV caches of one model at one geometry plus the captured steps that use them, keyed by
+    (batch, new tokens per step).  All graphs share one memory pool."""
+
+    def __init__(self, model, batch_size, max_seqlen, dtype=None, tensor_parallel=1):
+        first = next(iter(model.parameters()))
+        self.model, self.device, self.dtype = model, first.device, dtype or first.dtype
+        self.max_batch_size, self.max_seqlen = batch_size, max_seqlen
+        if hasattr(model, "allocate_inference_cache"):
+            caches = model.allocate_inference_cache(batch_size, max_seqlen, self.dtype)
+        else:
+            cfg = model.config
+            headdim = getattr(cfg, "head_dim", cfg.hidden_size // cfg.num_attention_heads)
+            caches = allocate_inference_cache(batch_size, max_seqlen, cfg.num_attention_heads // tensor_parallel,
+                                              headdim, cfg.num_hidden_layers, self.device, self.dtype)
+        self.inference_params = InferenceParams(
+            max_seqlen=max_seqlen, max_batch_size=batch_size, key_value_memory_dict=caches,
+            lengths_per_sample=torch.zeros(batch_size, dtype=torch.int32, device=self.device))
+        self.pool = torch.cuda.graphs.graph_pool_handle()
+        self.steps = {}
+
+    def fits(self, model, batch_size, max_seqlen, dtype=None):
+        first = next(iter(model.parameters()))
+        return (first.device, dtype or first.dtype) == (self.device, self.dtype) and \
+            batch_size <= self.max_batch_size and max_seqlen <= self.max_seqlen
+
+    def step(self, batch_size, n_tokens=1) -> DecodeStepGraph:
+        key = (batch_size, n_tokens)
+        if key not in self.steps:
+            with torch.inference_mode():
+                self.steps[key] = DecodeStepGraph(self.model, self.inference_params, batch_size, n_tokens, self.pool)
+        return self.steps[key]
+
+    def run(self, tokens, positions, lengths):
+        return self.step(tokens.shape[0], tokens.shape[1]).run(tokens, positions, lengths)
+
+
+def graphed_decoder(model, batch_size, max_seqlen, dtype=None, tensor_parallel=1) -> GraphedDecoder:
+    """The model's decoder cache (kept on the model as `_decoding_cache`), rebuilt when this request
+    does not fit its geometry, device or dtype."""
+    dec = getattr(model, "_decoding_cache", None)
+    if not isinstance(dec, GraphedDecoder) or not dec.fits(model, batch_size, max_seqlen, dtype):
+        model._decoding_cache = None                 # let the old caches and graphs go first
+        dec = GraphedDecoder(model, batch_size, max_seqlen, dtype, tensor_parallel)
+        model._decoding_cache = dec
+    return dec
+
+
+# ------------------------------------------------------------------------------------------------
+# the token loop
+# ------------------------------------------------------------------------------------------------
+class _Stepper:
+    """The model behind one generation: the prompt pass, then one call per new token, eager or
+    replayed from the captured step."""
+
+    def __init__(self, model, batch_size, max_length, use_graph):
+        self.model, self.batch_size = model, batch_size
+        self.graphs = graphed_decoder(model, batch_size, max_length) if use_graph else None
+        if use_graph:
+            self.state = self.graphs.inference_params
+            self.graphs.step(batch_size, 1)           # captured before the prompt pass touches the cache
+            self.state.reset(max_length, batch_size)  # lengths back to 0: the prompt's rotary positions start there
+        else:
+            self.state = InferenceParams(max_seqlen=max_length, max_batch_size=batch_size)
+
+    def prompt(self, input_ids):
+        self.state.seqlen_offset = 0
+        logits = self.model(input_ids, position_ids=None, inference_params=self.state, num_last_tokens=1).logits
+        self.state.seqlen_offset = input_ids.shape[1]
+        return logits[:, -1]
+
+    def advance(self, token):
+        """token (batch, 1) placed at position `seqlen_offset` of every sequence; returns its logits."""
+        filled = self.state.seqlen_offset
+        positions = torch.full((self.batch_size, 1), filled, dtype=torch.long, device=token.device)
+        if self.graphs is not None:
+            logits = self.graphs.run(token, positions, filled)
+        else:
+            logits = self.model(token, position_ids=positions, inference_params=self.state, num_last_tokens=1).logits
+        self.state.seqlen_offset = filled + 1
+        return logits[:, -1]
 
 
 @torch.inference_mode()
 def decode(input_ids, model, max_length, top_k=1, top_p=0.0, temperature=1.0, eos_token_id=None,
            teacher_outputs=None, vocab_size=None, tensor_parallel=1, cg=False, enable_timing=False):
-    """Prompt pass, then one token per step until max_length (or every sequence emitted eos).
-    input_ids (batch, seq_len), all sequences of one length.  With `teacher_outputs` (batch, len) the
-    next token is taken from there instead of being sampled.  With `cg` every single-token step is
-    a replay of one captured HIP graph.  Returns sequences (batch, <= max_length) and the per-step
-    logits (tuple of (batch, vocab))."""
+    """Prompt pass over input_ids (batch, seq_len; all sequences of one length), then one token per
+    step until the sequences hold max_length tokens or every sequence has just emitted eos.  With
+    `teacher_outputs` (batch, len) the token at a position comes from there while it lasts, else
+    from `sample`.  With `cg` every single-token step replays one captured HIP graph.  Returns
+    sequences (batch, <= max_length) and the logits each new token was chosen from, a tuple of
+    (batch, vocab) tensors."""
     assert tensor_parallel == 1, "one GPU: tensor parallel decoding is not part of this build"
-    batch_size, seqlen_og = input_ids.shape
-    teacher_len = teacher_outputs.shape[1] if teacher_outputs is not None else 0
-    if cg:
-        if not hasattr(model, "_decoding_cache"):
-            model._decoding_cache = None
-        model._decoding_cache = update_graph_cache(model, model._decoding_cache, batch_size, seqlen_og, max_length)
-        inference_params = model._decoding_cache.inference_params
-        inference_params.reset(max_length, batch_size)
-    else:
-        inference_params = InferenceParams(max_seqlen=max_length, max_batch_size=batch_size)
-
-    def get_logits(tokens):
-        decoding = inference_params.seqlen_offset > 0
-        position_ids = None
-        if decoding:
-            position_ids = torch.full((batch_size, 1), inference_params.seqlen_offset, dtype=torch.long,
-                                      device=tokens.device)
-        if cg and decoding:
-            logits = model._decoding_cache.run(tokens, position_ids, inference_params.seqlen_offset).squeeze(dim=1)
-        else:
-            logits = model(tokens, position_ids=position_ids, inference_params=inference_params,
-                           num_last_tokens=1).logits.squeeze(dim=1)
-        return logits[..., :vocab_size] if vocab_size is not None else logits
-
-    def next_token(logits):
-        if teacher_outputs is None or teacher_len <= inference_params.seqlen_offset:
-            token = sample(logits, top_k=top_k, top_p=top_p, temperature=temperature)
-        else:
-            token = teacher_outputs[:, inference_params.seqlen_offset]
-        return token.unsqueeze(1)
-
-    def finished(last):
-        if inference_params.seqlen_offset == 0:
-            return False
-        if eos_token_id is not None and (last == eos_token_id).all():
-            return True
-        return inference_params.seqlen_offset >= max_length - 1
-
-    start = torch.cuda.Event(enable_timing=enable_timing)
-    end = torch.cuda.Event(enable_timing=enable_timing)
+    batch_size = input_ids.shape[0]
+    taught = 0 if teacher_outputs is None else teacher_outputs.shape[1]
+    stepper = _Stepper(model, batch_size, max_length, cg)
+    clock = None
     if enable_timing:
-        start.record()
-    scores, sequences = [], [input_ids]
-    while not finished(sequences[-1]):
-        scores.append(get_logits(sequences[-1]))
-        inference_params.seqlen_offset += sequences[-1].shape[1]
-        sequences.append(next_token(scores[-1]))
-    if enable_timing:
-        end.record()
+        clock = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        clock[0].record()
+
+    pieces, scores = [input_ids], []
+    logits = stepper.prompt(input_ids)
+    while True:
+        scores.append(logits if vocab_size is None else logits[..., :vocab_size])
+        at = stepper.state.seqlen_offset                       # position the next token goes to
+        chosen = teacher_outputs[:, at] if at < taught else sample(scores[-1], top_k, top_p, temperature)
+        pieces.append(chosen.unsqueeze(1))
+        if at >= max_length - 1 or (eos_token_id is not None and bool((chosen == eos_token_id).all())):
+            break
+        logits = stepper.advance(pieces[-1])
+
+    if clock is not None:
+        clock[1].record()
         torch.cuda.synchronize()
-        print(f"Prompt processing + decoding time: {(start.elapsed_time(end)):.0f}ms")
-    output_cls = GreedySearchDecoderOnlyOutput if top_k == 1 else SampleDecoderOnlyOutput
-    return output_cls(sequences=torch.cat(sequences, dim=1), scores=tuple(scores))
-
-
-def allocate_inference_cache(max_batch_size, max_seqlen, nheads, headdim, layers, device, dtype=torch.float16):
-    """{layer_idx: (max_batch_size, max_seqlen, 2, nheads, headdim)}; `layers` an int or an iterable."""
-    assert dtype in (torch.float16, torch.bfloat16, torch.float32)
-    if isinstance(layers, int):
-        layers = range(layers)
-    shape = (max_batch_size, max_seqlen, 2, nheads, headdim)
-    return {i: torch.empty(shape, device=device, dtype=dtype) for i in layers}
-
-
-@dataclass
-class DecodingCGCache:
-    max_batch_size: int = 0
-    max_seqlen: int = 0
-    device = None
-    dtype = None
-    callables: dict = field(default_factory=dict)
-    mempool = None
-    inference_params: Optional[InferenceParams] = None
-    run: Optional[Callable] = None
-
-
-@torch.inference_mode()
-def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, decoding_seqlens=(1,), tensor_parallel=1,
-                       dtype=None, n_warmups=2):
-    """Make sure `cache` holds a captured step for (batch_size, each decoding_seqlen) at this cache
-    geometry, (re)allocating the KV cache and `lengths_per_sample` when the geometry grew."""
-    if cache is None:
-        cache = DecodingCGCache()
-    example = next(iter(model.parameters()))
-    device = example.device
-    if dtype is None:
-        dtype = example.dtype
-    if (device, dtype) != (cache.device, cache.dtype) or batch_size > cache.max_batch_size or max_seqlen > cache.max_seqlen:
-        cache.callables = {}
-        cache.mempool = None
-        cache.inference_params = None
-        gc.collect()
-        cache.device, cache.dtype = device, dtype
-        cache.max_batch_size, cache.max_seqlen = batch_size, max_seqlen
-        if hasattr(model, "allocate_inference_cache"):
-            kv = model.allocate_inference_cache(batch_size, max_seqlen, dtype)
-        else:
-            cfg = model.config
-            headdim = getattr(cfg, "head_dim", cfg.hidden_size // cfg.num_attention_heads)
-            kv = allocate_inference_cache(batch_size, max_seqlen, cfg.num_attention_heads // tensor_parallel, headdim,
-                                          cfg.num_hidden_layers, device, dtype)
-        lengths = torch.full((batch_size,), seqlen_og, dtype=torch.int32, device=device)
-        cache.inference_params = InferenceParams(max_seqlen=max_seqlen, max_batch_size=batch_size, seqlen_offset=seqlen_og,
-                                                 key_value_memory_dict=kv, lengths_per_sample=lengths)
-        cache.mempool = torch.cuda.graphs.graph_pool_handle()
-    for n in decoding_seqlens:
-        if (batch_size, n) not in cache.callables:
-            cache.callables[batch_size, n] = capture_graph(model, cache.inference_params, batch_size, max_seqlen,
-                                                           decoding_seqlen=n, mempool=cache.mempool, n_warmups=n_warmups)
-
-    def dispatch(input_ids, position_ids, seqlen):
-        return cache.callables[input_ids.shape[0], input_ids.shape[1]](input_ids, position_ids, seqlen)
-
-    cache.run = dispatch
-    cache.inference_params.seqlen_offset = 0
-    return cache
-
-
-def capture_graph(model, inference_params, batch_size, max_seqlen, decoding_seqlen=1, mempool=None, n_warmups=2):
-    """Capture one decoding step at the LARGEST cache fill (so that every launch is sized for it) and
-    return `run(input_ids, position_ids, seqlen)`, which sets the true lengths and replays."""
-    device = next(iter(model.parameters())).device
-    input_ids = torch.zeros((batch_size, decoding_seqlen), dtype=torch.long, device=device)
-    position_ids = torch.zeros((batch_size, decoding_seqlen), dtype=torch.long, device=device)
-    offset_before = inference_params.seqlen_offset
-    inference_params.seqlen_offset = max_seqlen - decoding_seqlen
-    inference_params.lengths_per_sample[:] = inference_params.seqlen_offset
-
-    side = torch.cuda.Stream()                      # default priority
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        for _ in range(n_warmups):
-            logits = model(input_ids, position_ids=position_ids, inference_params=inference_params,
-                           num_last_tokens=decoding_seqlen).logits
-        side.synchronize()
-    torch.cuda.current_stream().wait_stream(side)
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, pool=mempool):
-        logits = model(input_ids, position_ids=position_ids, inference_params=inference_params,
-                       num_last_tokens=decoding_seqlen).logits
-
-    def run(new_input_ids, new_position_ids, seqlen):
-        inference_params.lengths_per_sample[:] = seqlen
-        input_ids.copy_(new_input_ids)
-        position_ids.copy_(new_position_ids)
-        graph.replay()
-        return logits.clone()
-
-    inference_params.seqlen_offset = offset_before
-    return run
+        print(f"Prompt processing + decoding time: {clock[0].elapsed_time(clock[1]):.0f}ms")
+    result = GreedySearchDecoderOnlyOutput if top_k == 1 else SampleDecoderOnlyOutput
+    return result(sequences=torch.cat(pieces, dim=1), scores=tuple(scores))

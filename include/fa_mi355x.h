@@ -158,6 +158,14 @@ int fa_plan_splits(const fa_fwd_params *p, int32_t api, int32_t *num_splits);
 int fa_num_splits_heuristic_reference(int32_t batch_nheads_mblocks, int32_t num_sms,
                                       int32_t num_n_blocks, int32_t max_splits);
 
+/*
+ * Writes {seed, offset} to the two 64-bit words at rng_state (device memory) from a one-thread kernel
+ * on `hip_stream`: how the host side hands the dropout generator state to fa_fwd / fa_varlen_fwd
+ * without a host-to-device copy.  Stands where the reference stores its Philox seed and offset into
+ * rng_state inside the forward kernel (csrc/flash_attn/src/flash_fwd_kernel.h:1142-1148).
+ */
+int fa_set_rng_state(uint64_t *rng_state, uint64_t seed, uint64_t offset, void *hip_stream);
+
 /* Message of the last failure on the calling thread ("" if none). */
 const char *fa_last_error(void);
 

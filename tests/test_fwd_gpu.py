@@ -290,6 +290,37 @@ def test_kvcache_lengths_outside_the_cache_are_clamped(seqlen_q):
     assert torch.allclose(out[1, 0].float().cpu(), vn[1, 0].float().repeat_interleave(2, dim=0), atol=1e-3)
 
 
+@pytest.mark.parametrize("seqlen_q", [1, 40])
+def test_kvcache_rotary_positions_stay_inside_the_table(seqlen_q):
+    """A full (or nearly full) cache puts cache length + query row past the capacity; the rotary tables
+    are only required to cover the capacity (flash_api.cpp:1214), so q positions stop at the last
+    table row.  The tables here are the first `cap` rows of a buffer whose following rows are NaN: a
+    read past the table would poison the output.  The result must equal the one obtained with
+    tables that continue with copies of their last row."""
+    _say("kvcache_rotary_clamp", seqlen_q)
+    dtype, d, cap = torch.bfloat16, 64, 300
+    q = _gen((2, seqlen_q, 4, d), dtype, 1); kc = _gen((2, cap, 2, d), dtype, 2); vc = _gen((2, cap, 2, d), dtype, 3)
+    kn = _gen((2, seqlen_q, 2, d), dtype, 4); vn = _gen((2, seqlen_q, 2, d), dtype, 5)
+    cos, sin = orc.rotary_table(cap, d, dtype=dtype)
+    lens = torch.tensor([cap, cap - 3], dtype=torch.int32).to(DEV)
+    fa = _fa()
+    outs = []
+    for tail in (float("nan"), None):
+        big_c = torch.full((cap + 64, d // 2), float("nan"), dtype=dtype)
+        big_s = torch.full((cap + 64, d // 2), float("nan"), dtype=dtype)
+        big_c[:cap], big_s[:cap] = cos, sin
+        if tail is None:
+            big_c[cap:], big_s[cap:] = cos[-1], sin[-1]
+        big_c, big_s = big_c.to(DEV), big_s.to(DEV)
+        tc, ts = (big_c[:cap], big_s[:cap]) if tail is not None else (big_c, big_s)
+        kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+        outs.append(fa.flash_attn_with_kvcache(q.to(DEV), kc_d, vc_d, kn.to(DEV), vn.to(DEV), tc, ts, lens, causal=True,
+                                               rotary_interleaved=False))
+        assert not torch.isnan(kc_d).any()
+    assert not torch.isnan(outs[0]).any()
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_kvcache_strided_cache_views():
     """K and V caches as strided views of one (b, s, 2, h_k, d) tensor, as the reference's MHA module
     passes them (flash_attn/modules/mha.py:459-477)."""

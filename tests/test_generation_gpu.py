@@ -62,12 +62,12 @@ def test_mha_layer_matches_oracle(heads_kv, rotary_dim):
     torch.manual_seed(1)
     dtype, b, s, dim, h = torch.float16, 2, 150, 256, 4
     d = dim // h
+    if rotary_dim == 24:
+        with pytest.raises(ValueError, match="divisible by 16"):
+            MHA(dim, h, num_heads_kv=heads_kv, causal=True, layer_idx=0, rotary_emb_dim=rotary_dim, device=DEV, dtype=dtype)
+        return
     layer = MHA(dim, h, num_heads_kv=heads_kv, causal=True, layer_idx=0, rotary_emb_dim=rotary_dim, device=DEV, dtype=dtype)
     x = torch.randn(b, s, dim, device=DEV, dtype=dtype)
-    if rotary_dim == 24:
-        with pytest.raises(RuntimeError, match="divisible by 16"):
-            layer(x)
-        return
     with torch.no_grad():
         got = layer(x)
         qkv = layer.Wqkv(x).cpu()
@@ -167,6 +167,38 @@ def test_mha_packed_varlen_equals_per_sequence(heads_kv, rotary_dim):
             alone = layer(x[a:e][None])[0]
             err = (packed[a:e].float() - alone.float()).abs().max().item()
             assert err < 2e-2, (i, err)
+
+
+@pytest.mark.parametrize("heads_kv", [4, 2])
+def test_mha_packed_varlen_rotary_gradients(heads_kv):
+    """Training through the packed path with rotary: the gradients of the projection weights must be
+    those of the same sequences sent through the layer one at a time (the rotation's backward has to
+    run for the q and k parts of Wqkv)."""
+    from flash_attn.modules.mha import MHA
+    _say("mha varlen grad", heads_kv)
+    torch.manual_seed(7)
+    dtype, dim, h = torch.bfloat16, 256, 4
+    layer = MHA(dim, h, num_heads_kv=heads_kv, causal=True, layer_idx=0, rotary_emb_dim=32, device=DEV, dtype=dtype)
+    lens = [70, 1, 200, 33]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=DEV)
+    x = torch.randn(sum(lens), dim, device=DEV, dtype=dtype)
+    w = torch.randn(sum(lens), dim, device=DEV, dtype=dtype)
+
+    def grads(run):
+        layer.zero_grad(set_to_none=True)
+        (run().float() * w.float()).sum().backward()
+        return layer.Wqkv.weight.grad.float().clone(), layer.out_proj.weight.grad.float().clone()
+
+    g_packed = grads(lambda: layer(x, cu_seqlens=cu, max_seqlen=max(lens)))
+    g_alone = grads(lambda: torch.cat([layer(x[int(cu[i]):int(cu[i + 1])][None])[0] for i in range(len(lens))]))
+    for name, a, b in zip(("Wqkv", "out_proj"), g_packed, g_alone):
+        err = (a - b).abs().max().item()
+        _say("   %s grad: max diff %.3e of max %.3e" % (name, err, b.abs().max().item()))
+        assert err <= 2e-2 * b.abs().max().item(), (name, err)
+    # the q and k rows of Wqkv are the ones an in-place rotation without backward would get wrong
+    d = dim // h
+    qk_rows = slice(0, (h + heads_kv) * d)
+    assert (g_packed[0][qk_rows] - g_alone[0][qk_rows]).abs().max().item() <= 2e-2 * g_alone[0][qk_rows].abs().max().item()
 
 
 def test_flash_attention_wrappers_train_and_eval():
