@@ -72,6 +72,11 @@ static int check_common(const fa_fwd_params* p) {
     return 0;
 }
 
+// the caller lent enough zeroed words for the persistent decode kernel
+static bool counters_ok(const fa_fwd_params& p) {
+    return p.work_counter != nullptr && p.work_counter_len >= FA_WORK_COUNTER_WORDS;
+}
+
 // Split planning for 256 CUs.
 struct SplitPlan {
     int splits = 1;        // partial slots (what the caller allocates)
@@ -106,7 +111,7 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
                 // 512 over 256); 256 only while 512-key chunks would leave resident slots empty.
                 const int64_t minlen = streams * ((sk + FA_DEC_MINLEN - 1) / FA_DEC_MINLEN) < 2 * kNumCU ? 256 : FA_DEC_MINLEN;
                 int64_t len = rup(std::max<int64_t>(minlen, (int64_t)sk * streams / FA_DEC_SLOTS), 128);
-                if (p.work_counter) {
+                if (counters_ok(p)) {
                     const int64_t lp = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS_P), 128);
                     if (lp >= 1024) len = lp;
                 }
@@ -134,7 +139,7 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
     // 2048-key one, eighths from 4096 on): shorter pieces are mostly start-up and merge (measured
     // +6 % at batch 256 x 4k and at batch 64 x 8k with 16 grouped heads, nothing lost at config 5).
     const int sb = len < 2048 ? 2 : len < 4096 ? 4 : FA_DEC_SB;
-    if (dec && automatic && splits > 1 && p.work_counter && len >= 1024 && splits + sb <= FA_MAX_SPLITS) {
+    if (dec && automatic && splits > 1 && counters_ok(p) && len >= 1024 && splits + sb <= FA_MAX_SPLITS) {
         r.persistent = 1;
         r.sa = splits;
         r.sb = sb;
@@ -157,18 +162,14 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.split_len = 0;
     kp.num_m_blocks = 0;
     kp.rotary_q = 0;
-    kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = 0;
+    kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = 0;
     kp.work_counter = q.work_counter;
 }
 
-static int run_attention(KParams& kp, hipStream_t stream, bool counter_is_reset = false) {
+static int run_attention(KParams& kp, hipStream_t stream) {
     const fa_fwd_params& p = kp.p;
     int e;
     if (use_decode_kernel(p)) {
-        if (kp.dec_persistent && !counter_is_reset) {
-            e = launch_zero_counter(kp.work_counter, stream);
-            if (e) return fail_hip(e, "ticket reset launch");
-        }
         e = launch_decode(kp, stream);
         if (e) return fail_hip(e, "decode kernel launch");
     } else {
@@ -379,12 +380,14 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
     kp.rotary_q = kp.p.rotary_dim > 0;
     if (int r = resolve_splits(kp, kp.p, true)) return r;
     hipStream_t stream = (hipStream_t)hip_stream;
-    // the append launch also resets the ticket counter of a persistent decode launch (one launch less)
-    const bool reset_in_append = has_new && kp.dec_persistent && use_decode_kernel(kp.p);
-    if (has_new) {
-        if (int e = launch_append_kv(kp, reset_in_append ? kp.work_counter : nullptr, stream)) return fail_hip(e, "append_kv kernel launch");
+    // The persistent decode kernel appends the new rows itself: the item that reaches them writes them.
+    // With a left window bound some new rows may lie outside every query's window and would not be
+    // visited, so there the append stays a launch of its own, as for every other kernel.
+    kp.dec_append = has_new && kp.dec_persistent && use_decode_kernel(kp.p) && !kp.has_left;
+    if (has_new && !kp.dec_append) {
+        if (int e = launch_append_kv(kp, stream)) return fail_hip(e, "append_kv kernel launch");
     }
-    return run_attention(kp, stream, reset_in_append);
+    return run_attention(kp, stream);
 }
 
 int fa_fwd_kvcache_noalloc(const fa_fwd_params* p, void* hip_stream) {
@@ -392,9 +395,12 @@ int fa_fwd_kvcache_noalloc(const fa_fwd_params* p, void* hip_stream) {
     if (!p) return fail("params is NULL");
     unsigned char* base = scratch_of_current_device();
     if (!base) return 2;
-    // layout inside the array: [0, 256) ticket words, then lse_accum, then o_accum (256-byte aligned)
+    // layout inside the array: [0, kCounterBytes) the persistent decode kernel's counters (zero when the
+    // library is loaded, left zero by every launch), then lse_accum, then o_accum (256-byte aligned)
+    constexpr size_t kCounterBytes = 64u << 10;
     fa_fwd_params q = *p;
     q.work_counter = reinterpret_cast<int32_t*>(base);
+    q.work_counter_len = (int32_t)(kCounterBytes / sizeof(int32_t));
     q.o_accum = nullptr;
     q.lse_accum = nullptr;
     if (int r = check_common(&q)) return r;
@@ -404,11 +410,11 @@ int fa_fwd_kvcache_noalloc(const fa_fwd_params* p, void* hip_stream) {
         const size_t rows = (size_t)q.b * q.h * q.seqlen_q;
         const size_t lse_bytes = up256((size_t)splits * rows * sizeof(float));
         const size_t o_bytes = (size_t)splits * rows * (size_t)((q.d + 31) / 32 * 32) * sizeof(float);
-        if (256 + lse_bytes + o_bytes > (size_t)FA_NOALLOC_SCRATCH_BYTES)
+        if (kCounterBytes + lse_bytes + o_bytes > (size_t)FA_NOALLOC_SCRATCH_BYTES)
             return fail("fa_fwd_kvcache_noalloc: the split accumulators of this problem exceed FA_NOALLOC_SCRATCH_BYTES; "
                         "use fa_fwd_kvcache with caller-provided o_accum / lse_accum, or request num_splits = 1");
-        q.lse_accum = reinterpret_cast<float*>(base + 256);
-        q.o_accum = reinterpret_cast<float*>(base + 256 + lse_bytes);
+        q.lse_accum = reinterpret_cast<float*>(base + kCounterBytes);
+        q.o_accum = reinterpret_cast<float*>(base + kCounterBytes + lse_bytes);
     }
     return fa_fwd_kvcache(&q, hip_stream);
 }

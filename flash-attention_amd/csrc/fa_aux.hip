@@ -10,52 +10,13 @@
 
 namespace fa {
 
-// One wave per output row (b, h, i).  Lanes first reduce the per-split log-sum-exp values, then
-// stream the partial rows whose weight is non-zero.
+// One wave per output row (b, h, i): combine_row (fa_common.h).
 template <typename T>
 __global__ void __launch_bounds__(256) combine_kernel(const KParams kp) {
-    const fa_fwd_params& p = kp.p;
-    const int lane = threadIdx.x & 63;
-    const int64_t nrows = (int64_t)p.b * p.h * p.seqlen_q;
+    const int64_t nrows = (int64_t)kp.p.b * kp.p.h * kp.p.seqlen_q;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= nrows) return;
-    const int S = kp.num_splits;
-
-    float l0 = lane < S ? p.lse_accum[(int64_t)lane * nrows + row] : -INFINITY;
-    float l1 = lane + 64 < S ? p.lse_accum[(int64_t)(lane + 64) * nrows + row] : -INFINITY;
-    float mx = fmaxf(l0, l1);
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    const float mref = (mx == -INFINITY) ? 0.f : mx;
-    float sum = __expf(l0 - mref) + __expf(l1 - mref);
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
-    const bool dead = (sum == 0.f) || (sum != sum);
-    const float lse = dead ? INFINITY : __logf(sum) + mref;
-    const float w0 = dead ? 0.f : __expf(l0 - lse);
-    const float w1 = dead ? 0.f : __expf(l1 - lse);
-
-    const int i = (int)(row % p.seqlen_q);
-    const int h = (int)((row / p.seqlen_q) % p.h);
-    const int b = (int)(row / ((int64_t)p.seqlen_q * p.h));
-    if (lane == 0) p.softmax_lse[row] = lse;
-
-    // each lane owns 4 consecutive output dims per pass (64 lanes x 4 = 256 dims max)
-    const int d0 = lane * 4;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < S; s++) {
-        const float w = __shfl(s < 64 ? w0 : w1, s & 63);
-        if (w == 0.f) continue;   // wave-uniform
-        if (d0 < kp.d_rounded) {
-            const f32x4 v = *reinterpret_cast<const f32x4*>(p.o_accum + ((int64_t)s * nrows + row) * kp.d_rounded + d0);
-            acc += v * w;
-        }
-    }
-    if (d0 < p.d) {
-        int64_t off = (int64_t)i * p.o_row_stride + (int64_t)h * p.o_head_stride + (int64_t)b * p.o_batch_stride;
-        u32x2 v = {pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
-        st_global8(reinterpret_cast<T*>(p.o) + off + d0, v);
-    }
+    combine_row<T>(kp, row, threadIdx.x & 63);
 }
 
 int launch_combine(const KParams& kp, hipStream_t stream) {
@@ -69,9 +30,8 @@ int launch_combine(const KParams& kp, hipStream_t stream) {
 
 // One thread per 16-byte chunk of one new (token, kv-head) row.
 template <typename T>
-__global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp, int32_t* zero) {
+__global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp) {
     const fa_fwd_params& p = kp.p;
-    if (zero && blockIdx.x == 0 && threadIdx.x == 0) *zero = 0;     // ticket counter of the decode launch that follows
     const int cpr = p.d / 8;
     const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * cpr;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -104,13 +64,13 @@ __global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp, int32_
     st_global16(kdst + d0, raw);
 }
 
-int launch_append_kv(const KParams& kp, int32_t* zero, hipStream_t stream) {
+int launch_append_kv(const KParams& kp, hipStream_t stream) {
     const fa_fwd_params& p = kp.p;
     const int64_t total = (int64_t)p.b * p.seqlen_knew * p.h_k * (p.d / 8);
-    if (total == 0) return zero ? launch_zero_counter(zero, stream) : 0;
+    if (total == 0) return 0;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
-    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(append_kv_kernel<__bf16>, grid, block, 0, stream, kp, zero);
-    else hipLaunchKernelGGL(append_kv_kernel<_Float16>, grid, block, 0, stream, kp, zero);
+    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(append_kv_kernel<__bf16>, grid, block, 0, stream, kp);
+    else hipLaunchKernelGGL(append_kv_kernel<_Float16>, grid, block, 0, stream, kp);
     return (int)hipGetLastError();
 }
 

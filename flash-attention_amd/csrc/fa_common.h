@@ -52,8 +52,10 @@ struct KParams {
     int32_t has_left, has_right;  // window bounds active (after causal normalisation)
     int32_t rotary_q;      // rotate q on load
     // persistent decode schedule (see fa_decode.hip): dec_sa slots of split_len keys, then dec_sb
-    // slots of dec_sub keys for each sequence's ragged remainder; tickets from *work_counter
-    int32_t dec_persistent, dec_sa, dec_sb, dec_sub;
+    // slots of dec_sub keys for each sequence's ragged remainder; tickets from work_counter[0], workgroups
+    // that have left counted in [1].
+    // dec_append: the item that reaches rows [cache length, cache length + seqlen_knew) writes them
+    int32_t dec_persistent, dec_sa, dec_sb, dec_sub, dec_append;
     int32_t* work_counter;
 };
 
@@ -443,6 +445,63 @@ FA_DEV void store_tile_rows(const f32x16 (&acc)[DB], float sc, char* stage, int 
         const int rr = j * RPP + srow;
         const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
         if (rr < rows_ok && sch * 8 < cols_ok) st_global16(base + (int64_t)rr * row_stride + sch * 8, v);
+    }
+}
+
+// Log-sum-exp weighted merge of the split partials of one output row (b, h, i), by one wave: lanes first
+// reduce the per-split log-sum-exp values, then stream the partial rows whose weight is non-zero.
+// Reference: combine_attn_seqk_parallel, csrc/flash_attn/src/flash_fwd_kernel.h:1169-1327 (all splits
+// empty: lse = +inf, out = 0, :1233-1241).
+template <typename T>
+FA_DEV void combine_row(const KParams& kp, const int64_t row, const int lane) {
+    const fa_fwd_params& p = kp.p;
+    const int64_t nrows = (int64_t)p.b * p.h * p.seqlen_q;
+    const int S = kp.num_splits;
+
+    float l0 = lane < S ? p.lse_accum[(int64_t)lane * nrows + row] : -INFINITY;
+    float l1 = lane + 64 < S ? p.lse_accum[(int64_t)(lane + 64) * nrows + row] : -INFINITY;
+    float mx = fmaxf(l0, l1);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    const float mref = (mx == -INFINITY) ? 0.f : mx;
+    float sum = __expf(l0 - mref) + __expf(l1 - mref);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+    const bool dead = (sum == 0.f) || (sum != sum);
+    const float lse = dead ? INFINITY : __logf(sum) + mref;
+    const float w0 = dead ? 0.f : __expf(l0 - lse);
+    const float w1 = dead ? 0.f : __expf(l1 - lse);
+
+    const int i = (int)(row % p.seqlen_q);
+    const int h = (int)((row / p.seqlen_q) % p.h);
+    const int b = (int)(row / ((int64_t)p.seqlen_q * p.h));
+    if (lane == 0) p.softmax_lse[row] = lse;
+
+    // each lane owns 4 consecutive output dims (64 lanes x 4 = 256 dims max)
+    const int d0 = lane * 4;
+    // The partial rows are fetched eight at a time before any of them is used (one memory round trip per
+    // batch instead of one per split) and added in split order; a split of weight zero may never have been
+    // written, so its row is fetched but not used.
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    constexpr int BATCH = 8;
+    for (int s0 = 0; s0 < S; s0 += BATCH) {
+        f32x4 v[BATCH];
+        float w[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; j++) {
+            const int s = min(s0 + j, S - 1);
+            w[j] = s0 + j < S ? __shfl(s < 64 ? w0 : w1, s & 63) : 0.f;
+            const float* src = p.o_accum + ((int64_t)s * nrows + row) * kp.d_rounded + min(d0, kp.d_rounded - 4);
+            v[j] = *reinterpret_cast<const f32x4*>(src);
+        }
+#pragma unroll
+        for (int j = 0; j < BATCH; j++)
+            if (w[j] != 0.f) acc += v[j] * w[j];
+    }
+    if (d0 < p.d) {
+        int64_t off = (int64_t)i * p.o_row_stride + (int64_t)h * p.o_head_stride + (int64_t)b * p.o_batch_stride;
+        u32x2 v = {pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
+        st_global8(reinterpret_cast<T*>(p.o) + off + d0, v);
     }
 }
 

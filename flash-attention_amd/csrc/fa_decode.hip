@@ -46,7 +46,9 @@ enum ItemMode { kChunk = 0, kMacro = 1, kSub = 2 };
 
 // One (batch, kv head, key range) item: attention of the packed query rows over the range, written
 // as the final output (SPLIT = false) or as partial `slot` (SPLIT = true).
-template <typename T, int D, bool SPLIT>
+// APPEND: rows [cache length, cache length + seqlen_knew) are not in the cache yet; the item whose key range
+// holds them writes them first.  Every key belongs to exactly one item, so each row has one writer.
+template <typename T, int D, bool SPLIT, bool APPEND = false>
 FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b, const int slot,
                         const int mode, const int idx) {
     typedef DecodeCfg<T, D> C;
@@ -147,6 +149,36 @@ FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b
     if (has_right) lim_hi = min(lim_hi, qi + shift + wr);
     const int lim_lo = has_left ? qi + shift - wl : 0;
     const int tj = (lane & 15) >> 2, tq = lane & 3;
+
+    if constexpr (APPEND) {
+        // rows [cache length, cache length + seqlen_knew) that fall into this item's key range are not in the
+        // cache yet: the workgroup writes them (new keys rotated, values copied, exactly as append_kv_kernel)
+        // and waits until the stores have been performed before any wave loads its keys
+        const int a_lo = max(lo, si.sk_cache);
+        if (a_lo < hi) {
+            const int cpr = p.d / 8;
+            T* kdst = reinterpret_cast<T*>(const_cast<void*>(p.k)) + si.k_off + (int64_t)hk * p.k_head_stride;
+            T* vdst = reinterpret_cast<T*>(const_cast<void*>(p.v)) + si.v_off + (int64_t)hk * p.v_head_stride;
+            for (int e = tid; e < (hi - a_lo) * cpr; e += C::kThreads) {
+                const int n = a_lo + e / cpr, d0 = (e % cpr) * 8, t = n - si.sk_cache;
+                const T* vsrc = reinterpret_cast<const T*>(p.v_new) + (int64_t)b * p.vnew_batch_stride + (int64_t)t * p.vnew_row_stride + (int64_t)hk * p.vnew_head_stride;
+                const T* ksrc = reinterpret_cast<const T*>(p.k_new) + (int64_t)b * p.knew_batch_stride + (int64_t)t * p.knew_row_stride + (int64_t)hk * p.knew_head_stride;
+                st_global16(vdst + (int64_t)n * p.v_row_stride + d0, ld_global16(vsrc + d0));
+                u32x4 raw = ld_global16(ksrc + d0);
+                if (p.rotary_dim > 0 && d0 < p.rotary_dim) {
+                    const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)n * (p.rotary_dim / 2);
+                    const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)n * (p.rotary_dim / 2);
+                    float x[8];
+                    unpack8<T>(raw, x);
+                    rotary8<T>(x, ksrc, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
+                    raw = pack8<T>(x);
+                }
+                st_global16(kdst + (int64_t)n * p.k_row_stride + d0, raw);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+        }
+    }
 
     // the first K/V step is requested before anything else so that its latency overlaps the q
     // (and rotary table) fetches below
@@ -325,31 +357,44 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 
 // Persistent form: a fixed number of resident workgroups draw items from a ticket counter, in the
 // same cache-row-friendly order (kv head fastest), first the kMacro pass then the kSub pass.
-template <typename T, int D>
+//  * The item whose key range reaches the new rows appends them (APPEND, see decode_item): no append launch.
+//  * work_counter[0] is the ticket, work_counter[1] counts the workgroups that have left; the last one puts
+//    both back to zero, so the words are zero again when the kernel ends and no launch has to reset them.
+// Measured and not adopted: drawing the next ticket early (before the item: the returning atomic sits in front
+// of the item's first K/V loads in the wave's in-order memory queue, +7 % time; after the item's last load:
+// no change, the second resident workgroup of the CU already covers the round trip), and merging a (batch,
+// kv head)'s partials in the kernel by the last of its items to arrive (the partials must bypass the per-XCD
+// L2, every stream completes in the remainder pass at the very end of the launch, and 512 latency-bound
+// merges there cost 2-3 x the stand-alone merge kernel; cache write-back / invalidation fences at device scope
+// around every item instead cost three times the whole kernel).
+template <typename T, int D, bool APPEND>
 __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_ticket;
     const fa_fwd_params& p = kp.p;
     const int n_macro = p.b * kp.dec_sa * p.h_k;
     const int total = n_macro + p.b * kp.dec_sb * p.h_k;
+    int32_t* const ticket = kp.work_counter;
     for (;;) {
         __syncthreads();          // previous item is done with LDS and with s_ticket
-        if (threadIdx.x == 0) s_ticket = atomicAdd(kp.work_counter, 1);
+        if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         int t = s_ticket;
         if (t >= total) break;
-        if (t < n_macro) {
-            const int hk = t % p.h_k, s = (t / p.h_k) % kp.dec_sa, b = t / (p.h_k * kp.dec_sa);
-            decode_item<T, D, true>(kp, smem, hk, b, s, kMacro, s);
-        } else {
-            t -= n_macro;
-            const int hk = t % p.h_k, j = (t / p.h_k) % kp.dec_sb, b = t / (p.h_k * kp.dec_sb);
-            decode_item<T, D, true>(kp, smem, hk, b, kp.dec_sa + j, kSub, j);
+        const bool macro = t < n_macro;
+        const int per_b = macro ? kp.dec_sa : kp.dec_sb;
+        if (!macro) t -= n_macro;
+        const int hk = t % p.h_k, idx = (t / p.h_k) % per_b, b = t / (p.h_k * per_b);
+        decode_item<T, D, true, APPEND>(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
+    }
+    if (threadIdx.x == 0) {
+        const int gone = __hip_atomic_fetch_add(kp.work_counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (gone == (int)gridDim.x - 1) {     // every workgroup has drawn its last ticket
+            __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(kp.work_counter + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
-
-__global__ void zero_counter_kernel(int32_t* c) { if (threadIdx.x == 0) *c = 0; }
 
 template <typename T, int D>
 static int launch_decode_t(const KParams& kp, hipStream_t stream) {
@@ -360,10 +405,17 @@ static int launch_decode_t(const KParams& kp, hipStream_t stream) {
         const int total = kp.p.b * (kp.dec_sa + kp.dec_sb) * kp.p.h_k;
         const int resident = 256 * (D > 128 ? 1 : 2);          // workgroups the 256 CUs hold at once
         dim3 grid(total < resident ? total : resident), block(C::kThreads);
-        auto kern = decode_persistent_kernel<T, D>;
-        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+        if (kp.dec_append) {
+            auto kern = decode_persistent_kernel<T, D, true>;
+            e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
+            if (e != hipSuccess) return (int)e;
+            hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+        } else {
+            auto kern = decode_persistent_kernel<T, D, false>;
+            e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
+            if (e != hipSuccess) return (int)e;
+            hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+        }
         return (int)hipGetLastError();
     }
     dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b), block(C::kThreads);
@@ -378,11 +430,6 @@ static int launch_decode_t(const KParams& kp, hipStream_t stream) {
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     }
-    return (int)hipGetLastError();
-}
-
-int launch_zero_counter(int32_t* c, hipStream_t stream) {
-    hipLaunchKernelGGL(zero_counter_kernel, dim3(1), dim3(64), 0, stream, c);
     return (int)hipGetLastError();
 }
 

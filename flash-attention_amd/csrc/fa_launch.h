@@ -17,10 +17,9 @@ int prefill_block_n(int d_bucket);   // key-tile length of the prefill kernel fo
 int prefill_block_m(int d_bucket);
 
 int launch_decode(const KParams& kp, hipStream_t stream);      // small-q split-KV kernel
-int launch_zero_counter(int32_t* c, hipStream_t stream);     // ticket counter of the persistent decode
 int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials
-// k_new/v_new (+rotary) -> cache; also resets the ticket counter `zero` when it is not NULL
-int launch_append_kv(const KParams& kp, int32_t* zero, hipStream_t stream);
+// k_new/v_new (+rotary) -> cache
+int launch_append_kv(const KParams& kp, hipStream_t stream);
 int launch_attn_probs(const KParams& kp, hipStream_t stream);  // s_dmask: signed softmax probabilities (testing)
 int launch_rotary(const fa_rotary_params& p, hipStream_t stream);   // standalone rotary embedding
 

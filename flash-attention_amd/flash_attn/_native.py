@@ -45,7 +45,8 @@ class FaFwdParams(ctypes.Structure):
             "is_rotary_interleaved", "num_splits", "dtype")]
         + [("softmax_scale", ctypes.c_float), ("p_dropout", ctypes.c_float),
            ("rng_state", ctypes.c_void_p), ("s_dmask", ctypes.c_void_p),
-           ("sdm_rows", ctypes.c_int32), ("sdm_cols", ctypes.c_int32)]
+           ("sdm_rows", ctypes.c_int32), ("sdm_cols", ctypes.c_int32),
+           ("work_counter_len", ctypes.c_int32), ("reserved0", ctypes.c_int32)]
     )
 
 
@@ -202,12 +203,29 @@ def _dropout_state(p, p_dropout, return_softmax, gen_, batch, heads, seqlen_q, s
     return rng_state, s_dmask
 
 
+_COUNTERS = {}     # (device index, stream) -> zeroed int32 words lent to the persistent decode kernel
+
+
+def _counters(device, words):
+    """Counter words for launches on the current stream of `device`: zero when first handed out and left
+    zero by every launch, so one tensor per (device, stream) serves all calls (launches on one stream do
+    not overlap)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, _stream(device))
+    t = _COUNTERS.get(key)
+    if t is None or t.numel() < words:
+        t = torch.zeros((max(16, int(words)),), dtype=torch.int32, device=device)
+        _COUNTERS[key] = t
+    return t
+
+
 def _plan_and_alloc(params, api, batch, heads, seqlen_q, d, device):
     """Resolve the split count and allocate the fp32 partial buffers like the reference does
     (flash_api.cpp:373-389, 1241-1257).  The returned tensors must stay alive until launch."""
     n = ctypes.c_int32(0)
-    counter = torch.empty((1,), dtype=torch.int32, device=device)   # ticket scratch of the persistent decode
+    counter = _counters(device, 2)
     params.work_counter = counter.data_ptr()
+    params.work_counter_len = counter.numel()
     rc = lib.fa_plan_splits(ctypes.byref(params), api, ctypes.byref(n))
     if rc != 0:
         raise RuntimeError(lib.fa_last_error().decode())

@@ -58,10 +58,14 @@ typedef struct fa_fwd_params {
     const int32_t *cu_seqlens_k;    /* (b+1) prefix sums if is_seqlens_k_cumulative, else (b)
                                        per-batch key lengths (cache_seqlens), or NULL */
     const int32_t *cache_batch_idx; /* (b) row of k/v used (and updated) for batch i, or NULL */
-    int32_t *work_counter;          /* optional: one int32 of device scratch (any value; the library
-                                       resets it on the stream before use).  When set, split-KV
-                                       decode launches run as a persistent, ticket-scheduled kernel.
-                                       Must not be shared by calls that overlap on the GPU. */
+    int32_t *work_counter;          /* optional: work_counter_len (>= FA_WORK_COUNTER_WORDS) int32 words of
+                                       device memory that are ZERO before the first call that uses them;
+                                       every call leaves them zero again.  When set, split-KV decode
+                                       launches run as a persistent kernel whose workgroups draw (batch,
+                                       kv head, key chunk) items from a ticket and whose item that
+                                       reaches the new rows appends them to the cache (no append
+                                       launch).  Must not be shared by calls that overlap on the GPU.
+                                       NULL: one workgroup per chunk and a separate append launch. */
 
     int64_t q_batch_stride, q_row_stride, q_head_stride;
     int64_t k_batch_stride, k_row_stride, k_head_stride;
@@ -99,7 +103,12 @@ typedef struct fa_fwd_params {
      * of its CUDA MMA fragments) entry [i][j] is plainly row i, key j. */
     void *s_dmask;
     int32_t sdm_rows, sdm_cols;  /* >= seqlen_q, >= seqlen_k */
+    int32_t work_counter_len;    /* int32 words behind work_counter */
+    int32_t reserved0;
 } fa_fwd_params;
+
+/* words the persistent decode kernel needs behind work_counter: ticket, exit count */
+#define FA_WORK_COUNTER_WORDS 2
 
 /*
  * Dense batch forward.  Replaces mha_fwd (csrc/flash_attn/flash_api.cpp:248-424): same masking
@@ -131,7 +140,7 @@ int fa_fwd_kvcache(const fa_fwd_params *p, void *hip_stream);
  * the ticket words and the fp32 partial results of a split launch live in FA_NOALLOC_SCRATCH_BYTES of
  * device memory that the library itself holds on every GPU it runs on (a static device array, kept
  * until the process ends).  The call allocates and frees nothing.  A problem whose partials do not fit
- * (splits x b x h x seqlen_q x (4 + 4 x d rounded up to 32) bytes + 256) is rejected with an error;
+ * (splits x b x h x seqlen_q x (4 + 4 x d rounded up to 32) bytes + 64 KiB of counters) is rejected with an error;
  * num_splits = 1 always fits.  All calls on one GPU share the array: calls that overlap in time on the
  * same GPU (two streams, two threads) race on it and must be serialised by the caller.  The first call
  * on a device looks the array's address up (hipGetSymbolAddress): make one call before capturing a

@@ -80,6 +80,7 @@ def test_lse_persistent_decode_and_merge(with_new):
     p.window_left = p.window_right = -1
     for name in ("q", "k", "v", "o", "softmax_lse", "work_counter", "cu_seqlens_k"):
         setattr(p, name, 256)          # non-null placeholders: planning reads no memory
+    p.work_counter_len = 2
     import ctypes
     n = ctypes.c_int32(0)
     assert nat.lib.fa_plan_splits(ctypes.byref(p), 2, ctypes.byref(n)) == 0
