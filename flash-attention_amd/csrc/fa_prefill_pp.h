@@ -53,6 +53,19 @@ struct PPCfg {
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
+// -DFA_PP_TIMING: every workgroup records when it passes the stages of the kernel (shader-clock counter,
+// slots 0-5; constant 100 MHz counter at entry and exit, slots 6-7) for waves 0 and 4, into fa_pp_dbg, which
+// fa_pp_debug_read (fa_prefill_inst.hip) copies out.  Measurement builds only.
+#ifdef FA_PP_TIMING
+#define FA_PP_DBG_BLOCKS 32768      // workgroups with a record; launches with more blocks record only these
+__device__ long long fa_pp_dbg[FA_PP_DBG_BLOCKS * 2 * 16];
+#define FA_PP_STAMP(i) do { if (lane == 0 && (wave & 3) == 0 && blockIdx.x < FA_PP_DBG_BLOCKS) fa_pp_dbg[(blockIdx.x * 2 + group) * 16 + (i)] = __builtin_readcyclecounter(); } while (0)
+#define FA_PP_REALTIME(i) do { if (lane == 0 && (wave & 3) == 0 && blockIdx.x < FA_PP_DBG_BLOCKS) fa_pp_dbg[(blockIdx.x * 2 + group) * 16 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define FA_PP_STAMP(i) do {} while (0)
+#define FA_PP_REALTIME(i) do {} while (0)
+#endif
+
 template <typename T, int D, int BN, bool DROPOUT = false>
 __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     typedef PPCfg<T, D, BN> C;
@@ -64,16 +77,24 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const int wave = tid >> 6, lane = tid & 63;
     const int l32 = lane & 31, hh = lane >> 5;
     const int group = wave >> 2;
+    FA_PP_STAMP(0);
+    FA_PP_REALTIME(6);
+#ifdef FA_PP_TIMING
+    if (lane == 0 && wave == 0 && blockIdx.x < FA_PP_DBG_BLOCKS)      // HW_ID: which CU runs this workgroup
+        fa_pp_dbg[(blockIdx.x * 2) * 16 + 12] = (long long)__builtin_amdgcn_s_getreg((31 << 11) | 4);
+#endif
 
     // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
     const uint32_t G = (uint32_t)(p.h / p.h_k);
     int g, mb, hk, b;
     if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, (kp.has_left || kp.has_right) ? 32u : 0u, g, mb, hk, b)) return;
     const int head = hk * (int)G + g;
+    FA_PP_STAMP(8);       // work item known
 
     const SeqInfo si = seq_info(p, b);
     const int m0 = mb * C::BM;
     if (m0 >= si.sq) return;
+    FA_PP_STAMP(9);       // sequence bounds known
 
     const int shift = si.sk - si.sq;
     const int wl = p.window_left, wr = p.window_right;
@@ -92,29 +113,6 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 
     const int r0 = m0 + wave * 32;                // first query row of this wave
     const int row = r0 + l32;
-
-    v8 qf[C::KS];
-    {
-        const bool valid = row < si.sq;
-        const T* qrow = qg + (int64_t)row * p.q_row_stride;
-#pragma unroll
-        for (int dk = 0; dk < C::KS; dk++) {
-            const int d0 = dk * 16 + 8 * hh;
-            u32x4 raw = {0, 0, 0, 0};
-            if (valid && d0 < p.d) raw = ld_global16(qrow + d0);
-            qf[dk] = __builtin_bit_cast(v8, raw);
-        }
-    }
-
-    f32x16 o_acc[C::DB];
-#pragma unroll
-    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-    const float sl2 = kp.scale_log2;
-    Drop drop = {0, 0, 256, 1.f};
-    if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
 
     // visit i of the key loop handles key tile tile_of(i) and uses ring slot i % NS
 #ifdef FA_PP_ASCENDING
@@ -173,6 +171,41 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         }
         vtile += kDir * vstep;
     };
+
+    // The first tiles are requested before anything else is set up: the q rows, the accumulators and the
+    // per-lane LDS offsets below are all prepared while these requests are in flight.
+    if (nt > 0) {
+        fill_k(0);
+        fill_v(0);
+        if (nt > 1) { fill_k(1); fill_v(1); }
+        if (nt > 2) fill_k(2);
+    }
+    FA_PP_STAMP(1);
+
+    v8 qf[C::KS];
+    {
+        const bool valid = row < si.sq;
+        const T* qrow = qg + (int64_t)row * p.q_row_stride;
+#pragma unroll
+        for (int dk = 0; dk < C::KS; dk++) {
+            const int d0 = dk * 16 + 8 * hh;
+            u32x4 raw = {0, 0, 0, 0};
+            if (valid && d0 < p.d) raw = ld_global16(qrow + d0);
+            qf[dk] = __builtin_bit_cast(v8, raw);
+        }
+    }
+
+    FA_PP_STAMP(10);      // q loads issued
+    f32x16 o_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const float sl2 = kp.scale_log2;
+    Drop drop = {0, 0, 256, 1.f};
+    if constexpr (DROPOUT) drop = drop_init(p.rng_state, p.p_dropout, b, head, p.h);
+
 
     // Per-wave tile classes, as ranges of the absolute key-tile index t: the wave has visible keys
     // in tiles [ta_lo, ta_hi]; tiles in [tf_lo, tf_hi] are fully visible to all 32 rows (no masking).
@@ -379,15 +412,13 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     };
 
     if (nt > 0) {
-        // ---- prologue: request K(0), V(0), K(1), V(1), K(2); S = K(0) Q
-        fill_k(0);
-        fill_v(0);
-        if (nt > 1) { fill_k(1); fill_v(1); }
-        if (nt > 2) fill_k(2);
+        // ---- prologue: K(0), V(0), K(1), V(1), K(2) were requested above; S = K(0) Q
         wait_vmcnt<0>();
         __syncthreads();
+        FA_PP_STAMP(2);
         if (active(0)) qk(0);
         if (group == 1) __syncthreads();   // group 1 runs one phase behind group 0
+        FA_PP_STAMP(3);
 
         for (int i = 0; i < nt; i++) {
             // ---- Y(i): VALU phase (and requests for the tiles needed 3 iterations ahead)
@@ -407,6 +438,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             __syncthreads();
         }
         if (group == 0) __syncthreads();
+        FA_PP_STAMP(4);
     }
 
     // ---- epilogue
@@ -441,6 +473,11 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
         }
     }
+    FA_PP_STAMP(5);
+    FA_PP_REALTIME(7);
+#ifdef FA_PP_TIMING
+    if (lane == 0 && wave == 0 && blockIdx.x < FA_PP_DBG_BLOCKS) fa_pp_dbg[(blockIdx.x * 2) * 16 + 11] = nt;
+#endif
 }
 
 template <typename T, int D, int BN, bool DROPOUT>
