@@ -306,7 +306,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
     uint32_t unit;
     int hk, b;
     if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
-                         (uint32_t)(num_n_blocks * DPARTS), (kp.has_left || kp.has_right) ? 32u : 0u, unit, hk, b)) return;
+                         (uint32_t)(num_n_blocks * DPARTS), (kp.has_left || kp.has_right) ? 32u : 0u, (uint32_t)DPARTS, unit, hk, b)) return;
     const int dpart = (int)(unit % DPARTS);      // with DPARTS = 2 a workgroup accumulates half of the head dim
     const int nblk = (int)(unit / DPARTS);
 

@@ -563,7 +563,17 @@ __host__ __device__ inline bool xcd_strided(bool varlen, int64_t batch, int64_t 
 // The k streams then share the L2 (k x K/V of a short sequence is no more than one long one).
 // Callers pass slots = 0 (k = 1, one stream after the other) when no mask is active: all units of
 // a stream then cost the same and sharing the L2 only costs (measured -1..2 %).
-FA_DEV bool xcd_stream_unit(bool strided, uint32_t batch, uint32_t h_k, uint32_t per_stream, uint32_t slots,
+//
+// The hardware hands the workgroups of a grid to the 4 shader engines of an XCD in strict rotation and in
+// order: a workgroup waits for a free CU of its own engine, and every later workgroup waits behind it.
+// Dealing one dense stream's units out in falling cost gives one engine the heaviest unit of every four and
+// leaves the other three idle behind it (measured: 8 % of a causal 8k launch, 18 % at 4k).  `equal` is the
+// number of consecutive units of a stream that cost the same (the grouped q heads of a row block); for
+// dense batches k is rounded up so that k * equal is a multiple of 4: every four consecutive workgroups
+// then cost the same and each engine works through streams of its own at the same pace.  Packed batches
+// keep the smaller k: their streams differ in length, and giving an engine a stream of its own would
+// unbalance the engines instead.
+FA_DEV bool xcd_stream_unit(bool strided, uint32_t batch, uint32_t h_k, uint32_t per_stream, uint32_t slots, uint32_t equal,
                             uint32_t& unit, int& hk, int& b) {
     const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3, S = batch * h_k;
     uint32_t s;
@@ -580,7 +590,12 @@ FA_DEV bool xcd_stream_unit(bool strided, uint32_t batch, uint32_t h_k, uint32_t
         s = w / per_stream;
     } else {
         const uint32_t n_local = strided ? (S + 7u - x) >> 3 : S >> 3;       // streams of this XCD
-        const uint32_t k = max(1u, min((slots + per_stream - 1u) / per_stream, n_local));
+        uint32_t k = (slots + per_stream - 1u) / per_stream;
+        if (!strided && slots != 0u) {
+            const uint32_t m = (equal & 3u) == 0u ? 1u : (equal & 1u) == 0u ? 2u : 4u;
+            k = (k + m - 1u) / m * m;
+        }
+        k = max(1u, min(k, n_local));
         const uint32_t grp = j / (k * per_stream), first = grp * k;
         if (first >= n_local) return false;
         const uint32_t kk = min(k, n_local - first);                          // the last group may be short
@@ -620,10 +635,11 @@ FA_DEV bool xcd_rows_item(bool split, bool varlen, uint32_t batch, uint32_t h_k,
     const uint32_t parts = xcd_parts(split, varlen, h_k, G), Gp = G / parts, hp = h_k * parts;
     uint32_t unit;
     int hkp;
-    if (!xcd_stream_unit(xcd_strided(varlen, batch, hp), batch, hp, Gp * nmb, slots, unit, hkp, b)) return false;
+    if (!xcd_stream_unit(xcd_strided(varlen, batch, hp), batch, hp, Gp * nmb, slots, Gp, unit, hkp, b)) return false;
     hk = (int)((uint32_t)hkp / parts);
     g = (int)(((uint32_t)hkp % parts) * Gp + unit % Gp);
-    mb = (int)(nmb - 1u - unit / Gp);
+    const uint32_t u = unit / Gp;
+    mb = (int)(nmb - 1u - u);
     return true;
 }
 inline int64_t xcd_rows_grid(bool split, bool varlen, int64_t batch, int64_t h_k, int64_t G, int64_t nmb) {

@@ -57,7 +57,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     uint32_t unit;
     int hk, b;
     if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
-                         (uint32_t)(S * G * kp.num_m_blocks), (kp.has_left || kp.has_right) ? 32u * MINW : 0u, unit, hk, b)) return;
+                         (uint32_t)(S * G * kp.num_m_blocks), (kp.has_left || kp.has_right) ? 32u * MINW : 0u, (uint32_t)(S * G), unit, hk, b)) return;
     const int split = (int)(unit % (uint32_t)S); unit /= (uint32_t)S;
     const int g = (int)(unit % (uint32_t)G);
     const int mb = kp.num_m_blocks - 1 - (int)(unit / (uint32_t)G);
