@@ -103,6 +103,34 @@ def bench_prefill(steps, warmup):
     }
 
 
+def bench_head_dims(steps, warmup):
+    """Head dims between the buckets (bf16 causal, 4 x 8192, 32 heads): 96 runs on the 128-wide tiles and 192
+    on the 256-wide ones with the k-steps and output column blocks past the head dim left out; FLOPs are
+    counted at the real head dim."""
+    import torch
+    import flash_attn
+    b, s, h = 4, 8192, 32
+    res = {}
+    for d, kern in ((96, "fa::prefill_pp_kernel<bf16,128,64,false,96>"), (192, "fa::prefill_il_kernel<bf16,ILCfgPair<bf16,192>>")):
+        torch.manual_seed(0)
+        q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
+        with torch.no_grad():
+            tm = time_steps(lambda: flash_attn.flash_attn_func(q, k, v, causal=True), steps, warmup)
+        o = flash_attn.flash_attn_func(q, k, v, causal=True)
+        do = torch.randn_like(o)
+        tb = time_steps(lambda: torch.autograd.grad(o, (q, k, v), do, retain_graph=True), max(1, steps // 3), max(1, warmup // 3))
+        flops = 4.0 * b * s * s * h * d / 2
+        tf, tfb = flops / (tm[0] * 1e-3) / 1e12, 2.5 * flops / (tb[0] * 1e-3) / 1e12
+        res["d%d" % d] = {
+            "ms": tm[0], "ms_min": tm.ms_min, "tflops": tf,
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS,
+                         "traffic": None, "kernel": kern, "flops_per_launch": flops},
+            "backward": {"ms": tb[0], "ms_min": tb.ms_min, "tflops": tfb, "frac": tfb / PEAK_BF16_TFLOPS},
+        }
+        del q, k, v, o, do
+    return res
+
+
 def bench_mfma_peak(steps, warmup):
     """What the matrix pipes sustain on MFMAs alone (fa_mfma_peak in the library): the clock of the fully
     loaded part follows the switching activity of the operands, so the figure is taken on random bf16
@@ -354,6 +382,7 @@ def main():
         out["fwd_bwd"] = bench_fwd_bwd(a.steps, a.warmup)
         out["varlen"] = bench_varlen(a.steps, a.warmup)
         out["gqa_window"] = bench_gqa_window(a.steps, a.warmup)
+        out["head_dims"] = bench_head_dims(a.steps, a.warmup)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -87,21 +87,22 @@ __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdKParams kp) {
 // ------------------------------------------------------------------------------------------------
 // dQ: a workgroup owns 128 query rows of one (batch, head) and streams K / V tiles of BN keys.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int D, int BN>
+// DV: head dims the products run over (a multiple of 32, d <= DV <= D); tiles keep the LDS layout of the bucket D
+template <typename T, int D, int BN, int DV = D>
 struct BwdDqCfg {
     static constexpr int kThreads = 256, kWaves = 4, BM = 128;
-    static constexpr int NB = BN / 32, KS = D / 16, DB = D / 32, PT = BN / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int NB = BN / 32, KS = DV / 16, DB = DV / 32, PT = BN / 16, CPR = D / 8, ROWB = D * 2;
     static constexpr int TILE_BYTES = BN * ROWB;
     static constexpr int LOADS = BN * CPR / kThreads;
-    static constexpr int STAGE_BYTES = 32 * (DB * 64 + 16);      // a wave's dQ rows on their way out
+    static constexpr int STAGE_BYTES = stage_tile_bytes<DB>();   // a wave's dQ rows on their way out
     static constexpr int SMEM = 4 * TILE_BYTES > kWaves * STAGE_BYTES ? 4 * TILE_BYTES : kWaves * STAGE_BYTES;   // {K, V} x 2 stages
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
     static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
 };
 
-template <typename T, int D, int BN, int MINW, bool DROPOUT>
+template <typename T, int D, int BN, int MINW, bool DROPOUT, int DV = D>
 __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) {
-    typedef BwdDqCfg<T, D, BN> C;
+    typedef BwdDqCfg<T, D, BN, DV> C;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_bwd_params& p = kp.p;
@@ -271,10 +272,10 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 // head dimension of dK / dV (both form S and dP in full): the accumulators of all 256 columns would
 // not fit next to the resident K / V row in 256 registers.
 // ------------------------------------------------------------------------------------------------
-template <typename T, int D, int BM, int DPARTS>
+template <typename T, int D, int BM, int DPARTS, int DV = D>
 struct BwdDkv3Cfg {
     static constexpr int kThreads = 512, kWaves = 8, BNW = 128;
-    static constexpr int MBK = BM / 32, KS = D / 16, DB = D / 32 / DPARTS, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
+    static constexpr int MBK = BM / 32, KS = DV / 16, DB = DV / 32 / DPARTS, PT = BM / 16, CPR = D / 8, ROWB = D * 2;
     static constexpr int TILE_BYTES = BM * ROWB;
     static constexpr int LOADS = BM * CPR / kThreads;
     static constexpr int Q_OFF = 0;                                  // 3 stages
@@ -286,14 +287,14 @@ struct BwdDkv3Cfg {
     // the resident K / V rows come in through LDS where the idle ring stages and the hand-over hold them
     static constexpr bool STAGED_ROWS = 4 * 32 * ROWB <= 2 * TILE_BYTES && 4 * 32 * ROWB <= 2 * 4 * XBLK;
     static_assert(kWaves * 32 * (DB * 64 + 16) <= SMEM, "gradient rows are staged in the ring");
-    static_assert(BM % 32 == 0 && D % (32 * DPARTS) == 0 && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
+    static_assert(BM % 32 == 0 && DV % (32 * DPARTS) == 0 && DV <= D && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
     static_assert(SMEM <= 160 * 1024, "LDS budget");
     static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
 };
 
-template <typename T, int D, int BM, int DPARTS, bool DROPOUT>
+template <typename T, int D, int BM, int DPARTS, bool DROPOUT, int DV = D>
 __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
-    typedef BwdDkv3Cfg<T, D, BM, DPARTS> C;
+    typedef BwdDkv3Cfg<T, D, BM, DPARTS, DV> C;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_bwd_params& p = kp.p;
@@ -422,7 +423,7 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
             stage_rows_issue<T, D>(blk, [&](int r) { return min(kblk * 32 + r, last) * rs; }, p.d,
                                    (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)region)), lane);
             wait_vmcnt<0>();
-            stage_rows_read<T, D>(rf, smem + region, p.d, lane);
+            stage_rows_read<T, D, C::KS>(rf, smem + region, p.d, lane);
         } else {
             const T* row = blk + (int64_t)(kblk * 32 + l32) * rs;
 #pragma unroll
@@ -581,34 +582,34 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                        : reinterpret_cast<T*>(p.dv) + si.dv_off + (int64_t)j0w * p.dv_row_stride + (int64_t)hk * p.dv_head_stride;
     const float sc = role_ds ? p.softmax_scale : (DROPOUT ? 1.f / (1.f - p.p_dropout) : 1.f);
     const int col0 = dpart * C::DB * 32;
-    store_tile_rows<T, C::DB>(acc, sc, smem + wave * (32 * (C::DB * 64 + 16)), lane, obase + col0,
+    store_tile_rows<T, C::DB>(acc, sc, smem + wave * stage_tile_bytes<C::DB>(), lane, obase + col0,
                               role_ds ? p.dk_row_stride : p.dv_row_stride, si.sk - j0w, p.d - col0);
 }
 
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-template <typename T, int D, int BN, int MINW, bool DROPOUT>
+template <typename T, int D, int BN, int MINW, bool DROPOUT, int DV = D>
 int launch_bwd_dq(const BwdKParams& kp, hipStream_t stream) {
-    typedef BwdDqCfg<T, D, BN> C;
+    typedef BwdDqCfg<T, D, BN, DV> C;
     const int64_t nmb = (kp.p.seqlen_q + C::BM - 1) / C::BM;
     if (nmb * kp.p.h * kp.p.b <= 0) return 0;
     const int64_t nblocks = xcd_rows_grid(false, kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k, kp.p.h / kp.p.h_k, nmb);
     if (nblocks == 0) return -2;
-    auto kern = bwd_dq_kernel<T, D, BN, MINW, DROPOUT>;
+    auto kern = bwd_dq_kernel<T, D, BN, MINW, DROPOUT, DV>;
     if (int e = (int)FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();
 }
 
-template <typename T, int D, int BM, int DPARTS, bool DROPOUT>
+template <typename T, int D, int BM, int DPARTS, bool DROPOUT, int DV = D>
 int launch_bwd_dkv3(const BwdKParams& kp, hipStream_t stream) {
-    typedef BwdDkv3Cfg<T, D, BM, DPARTS> C;
+    typedef BwdDkv3Cfg<T, D, BM, DPARTS, DV> C;
     const int64_t per_stream = (int64_t)((kp.p.seqlen_k + C::BNW - 1) / C::BNW) * DPARTS;
     if (per_stream * kp.p.h_k * kp.p.b <= 0) return 0;
     const int64_t nblocks = xcd_grid(xcd_strided(kp.p.cu_seqlens_q != nullptr, kp.p.b, kp.p.h_k), kp.p.b, kp.p.h_k, per_stream);
     if (nblocks == 0) return -2;
-    auto kern = bwd_dkv3_kernel<T, D, BM, DPARTS, DROPOUT>;
+    auto kern = bwd_dkv3_kernel<T, D, BM, DPARTS, DROPOUT, DV>;
     if (int e = (int)FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::kThreads), C::SMEM, stream, kp);
     return (int)hipGetLastError();

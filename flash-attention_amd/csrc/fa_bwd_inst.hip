@@ -23,26 +23,33 @@ typedef _Float16 InstT;
 #ifndef FA_BWD_BM
 #define FA_BWD_BM (FA_D == 64 ? 128 : 64)
 #endif
-template <bool DROPOUT>
+// DV: head dims the products run over (head dims up to 96 on the 128 bucket, up to 192 on the 256 bucket)
+template <bool DROPOUT, int DV = FA_D>
 static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers;
     // three at head dim 64 (168 registers), where the vector work per matrix instruction doubles
-    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, (FA_D == 64 ? 3 : 2), DROPOUT>(kp, stream)) return e;
+    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, (FA_D == 64 ? 3 : 2), DROPOUT, DV>(kp, stream)) return e;
     // Fewer key blocks than CUs (one long sequence on one or two kv heads, say): two workgroups per
     // key block, each accumulating half of the head dimension, fill the CUs at 3/4 of the work each.
     typedef BwdDkv3Cfg<InstT, FA_D, FA_BWD_BM, 1> C1;
     const int64_t key_blocks = (int64_t)((kp.p.seqlen_k + C1::BNW - 1) / C1::BNW) * kp.p.h_k * kp.p.b;
     if (key_blocks < 256 && kp.p.seqlen_q >= 1024) return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 2, DROPOUT>(kp, stream);
-    return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 1, DROPOUT>(kp, stream);
+    return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 1, DROPOUT, DV>(kp, stream);
 #else
-    if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT>(kp, stream)) return e;
-    return launch_bwd_dkv3<InstT, FA_D, 32, 2, DROPOUT>(kp, stream);
+    if (int e = launch_bwd_dq<InstT, FA_D, 32, 1, DROPOUT, DV>(kp, stream)) return e;
+    return launch_bwd_dkv3<InstT, FA_D, 32, 2, DROPOUT, DV>(kp, stream);
 #endif
 }
 
 int FA_INST_NAME(FA_D)(const BwdKParams& kp, hipStream_t stream) {
-    return kp.p.p_dropout > 0.f ? run<true>(kp, stream) : run<false>(kp, stream);
+    if (kp.p.p_dropout > 0.f) return run<true>(kp, stream);
+#if FA_D == 128
+    if (kp.p.d <= 96) return run<false, 96>(kp, stream);
+#elif FA_D == 256
+    if (kp.p.d <= 192) return run<false, 192>(kp, stream);
+#endif
+    return run<false>(kp, stream);
 }
 
 #if FA_D == 64

@@ -320,10 +320,12 @@ template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_cols_at(const char*
 //
 // acc[blk] (+)= rows [32 blk, 32 blk + 32) of `tile`  x  bfrag[dk]   for blk < NBLK, dk < KS
 // (ZERO0 = false: the accumulators already hold the value the product is added to.)
-template <typename T, int D, int NBLK, int KS, int GRP, bool ZERO0 = true>
+// (GRP0 is the wanted group size; a product whose MFMA count it does not divide -- 6 k-steps of head dim 96 --
+// runs in groups of 3 or 2.)
+template <typename T, int D, int NBLK, int KS, int GRP0, bool ZERO0 = true>
 FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const typename Elem<T>::v8* bfrag) {
     typedef typename Elem<T>::v8 v8;
-    constexpr int TOTAL = NBLK * KS, NG = TOTAL / GRP;
+    constexpr int TOTAL = NBLK * KS, GRP = TOTAL % GRP0 == 0 ? GRP0 : TOTAL % 3 == 0 ? 3 : 2, NG = TOTAL / GRP;
     static_assert(TOTAL % GRP == 0, "group shape");
     // step st -> (k-step st / NBLK, row block st % NBLK): consecutive MFMAs go to different accumulators
     v8 a[2][GRP];
@@ -348,10 +350,10 @@ FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const t
     __builtin_amdgcn_sched_barrier(0);
 }
 // acc[db] += columns [32 db, 32 db + 32) of tile rows [16 t16, 16 t16 + 16), transposed  x  bfrag[t16]
-template <typename T, int D, int PT, int DB, int GRP>
+template <typename T, int D, int PT, int DB, int GRP0>
 FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], const typename Elem<T>::v8* bfrag) {
     typedef typename Elem<T>::v8 v8;
-    constexpr int TOTAL = PT * DB, NG = TOTAL / GRP;
+    constexpr int TOTAL = PT * DB, GRP = TOTAL % GRP0 == 0 ? GRP0 : TOTAL % 3 == 0 ? 3 : 2, NG = TOTAL / GRP;
     static_assert(TOTAL % GRP == 0, "group shape");
     v8 a[2][GRP];
 #pragma unroll
@@ -408,13 +410,13 @@ FA_DEV void stage_rows_issue(const T* base, RowOff row_off, int d, uint32_t lds_
         async_fill16(base, ((uint32_t)row_off(r) + (uint32_t)(c * 8)) * 2u, lds_region + j * 1024);
     }
 }
-template <typename T, int D>
-FA_DEV void stage_rows_read(typename Elem<T>::v8 (&rf)[D / 16], const char* region, int d, int lane) {
+template <typename T, int D, int KS = D / 16>
+FA_DEV void stage_rows_read(typename Elem<T>::v8 (&rf)[KS], const char* region, int d, int lane) {
     typedef typename Elem<T>::v8 v8;
     const int l32 = lane & 31, hh = lane >> 5;
     asm volatile("" ::: "memory");     // the region was written by the fills, not by anything the compiler saw
 #pragma unroll
-    for (int dk = 0; dk < D / 16; dk++) {
+    for (int dk = 0; dk < KS; dk++) {
         u32x4 a = *reinterpret_cast<const u32x4*>(region + l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16);
         if (dk * 16 + 8 * hh >= d) a = u32x4{0, 0, 0, 0};
         rf[dk] = __builtin_bit_cast(v8, a);
@@ -422,13 +424,17 @@ FA_DEV void stage_rows_read(typename Elem<T>::v8 (&rf)[D / 16], const char* regi
 }
 
 // A wave's 32 x (32 DB) accumulator tile (lane l32 = row, registers = columns) to global memory
-// through a wave-private LDS region of 32 * (64 DB + 16) bytes, so that every store instruction
+// through a wave-private LDS region of stage_tile_bytes<DB>() bytes, so that every store instruction
 // writes whole rows, 16 B per lane, instead of 8-byte pieces of 32 rows.  `base` points at row 0,
-// column 0 of the tile; rows >= rows_ok and columns >= cols_ok are not written.
+// column 0 of the tile; rows >= rows_ok and columns >= cols_ok are not written.  A row takes a power
+// of two of lanes (12 chunks of a 96-column tile: 16 lanes, 4 of them idle).
+template <int DB> constexpr int stage_row_lanes() { return DB * 4 <= 4 ? 4 : DB * 4 <= 8 ? 8 : DB * 4 <= 16 ? 16 : 32; }
+template <int DB> constexpr int stage_tile_bytes() { return 32 * (stage_row_lanes<DB>() * 16 + 16); }
 template <typename T, int DB>
 FA_DEV void store_tile_rows(const f32x16 (&acc)[DB], float sc, char* stage, int lane, T* base, int64_t row_stride,
                             int rows_ok, int cols_ok) {
-    constexpr int PITCH = DB * 64 + 16, CPR = DB * 4, RPP = 64 / CPR;
+    constexpr int CPR = DB * 4, CPP = stage_row_lanes<DB>(), PITCH = CPP * 16 + 16, RPP = 64 / CPP;
+    static_assert(DB <= 8, "row lanes");
     const int l32 = lane & 31, hh = lane >> 5;
 #pragma unroll
     for (int db = 0; db < DB; db++)
@@ -439,12 +445,12 @@ FA_DEV void store_tile_rows(const f32x16 (&acc)[DB], float sc, char* stage, int 
                              pack2<T>(acc[db][4 * q4 + 2] * sc, acc[db][4 * q4 + 3] * sc)};
             *reinterpret_cast<u32x2*>(stage + l32 * PITCH + d0 * 2) = v;
         }
-    const int srow = lane / CPR, sch = lane % CPR;
+    const int srow = lane / CPP, sch = lane % CPP;
 #pragma unroll
     for (int j = 0; j < 32 / RPP; j++) {
         const int rr = j * RPP + srow;
         const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
-        if (rr < rows_ok && sch * 8 < cols_ok) st_global16(base + (int64_t)rr * row_stride + sch * 8, v);
+        if (rr < rows_ok && sch < CPR && sch * 8 < cols_ok) st_global16(base + (int64_t)rr * row_stride + sch * 8, v);
     }
 }
 

@@ -33,14 +33,16 @@ namespace fa {
 #endif
 
 // One query-row group of 32 rows per wave, the whole head dimension in that wave (d <= 128).
-template <typename T, int D_, int BN_>
+// DV_: head dims the products run over (a multiple of 32, d <= DV_ <= D_); tiles keep the LDS layout of the
+// bucket D_ (head dim 96 runs on the 128 bucket with 6 of 8 k-steps and 3 of 4 output column blocks).
+template <typename T, int D_, int BN_, int DV_ = D_>
 struct ILCfg {
     static constexpr int D = D_, BN = BN_;
     static constexpr bool kPair = false;
     static constexpr int kThreads = 256;
     static constexpr int kWaves = 4;
     static constexpr int BM = kWaves * 32;
-    static constexpr int DH = D;                            // head-dim slice of one wave
+    static constexpr int DH = DV_;                          // head-dim slice of one wave
     static constexpr int NB = BN / 32;
     static constexpr int KS = DH / 16;
     static constexpr int DB = DH / 32;
@@ -63,14 +65,14 @@ struct ILCfg {
 // the two partial S tiles are exchanged through LDS and added (both waves then hold the same S
 // and run the same softmax), and each accumulates its own 128 columns of O.  8 waves, 128 rows
 // per workgroup, 32-key tiles, one workgroup per CU.
-template <typename T>
+template <typename T, int DV_ = 256>
 struct ILCfgPair {
     static constexpr int D = 256, BN = 32;
     static constexpr bool kPair = true;
     static constexpr int kThreads = 512;
     static constexpr int kWaves = 8;
     static constexpr int BM = (kWaves / 2) * 32;
-    static constexpr int DH = D / 2;
+    static constexpr int DH = DV_ / 2;                      // 128, or 96 for head dims up to 192
     static constexpr int NB = BN / 32;
     static constexpr int KS = DH / 16;
     static constexpr int DB = DH / 32;
@@ -570,8 +572,9 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2
     // output tile of the wave (32 rows x DH columns) through LDS (whole rows per store instruction); all ring reads are
     // behind the barrier that follows the last product and each wave uses its own region
     {
-        constexpr int PITCH = C::DH * 2 + 16;
         constexpr int OCPR = C::DH / 8;                 // 16 B chunks per output row of the wave
+        constexpr int OCPP = OCPR <= 8 ? 8 : 16;        // lanes per row in a store instruction (a power of two)
+        constexpr int PITCH = OCPP * 16 + 16;
         static_assert(C::kWaves * 32 * PITCH <= C::SMEM, "staging region");
         char* stage = smem + wave * (32 * PITCH);
 #pragma unroll
@@ -583,14 +586,14 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2
                                  pack2<T>(o_acc[db][4 * q4 + 2] * inv, o_acc[db][4 * q4 + 3] * inv)};
                 *reinterpret_cast<u32x2*>(stage + l32 * PITCH + d0 * 2) = v;
             }
-        constexpr int RPP = 64 / OCPR;
-        const int srow = lane / OCPR, sch = lane % OCPR;
+        constexpr int RPP = 64 / OCPP;
+        const int srow = lane / OCPP, sch = lane % OCPP;
         T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + dcol0 + sch * 8;
 #pragma unroll
         for (int j = 0; j < 32 / RPP; j++) {
             const int rr = j * RPP + srow;
             const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
-            if (r0 + rr < si.sq && dcol0 + sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
+            if (r0 + rr < si.sq && sch < OCPR && dcol0 + sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
         }
     }
 }
@@ -615,8 +618,16 @@ int launch_prefill_il_cfg(const KParams& kp, hipStream_t stream) {
     return kp.p.p_dropout > 0.f ? launch_prefill_il_one<T, C, true>(kp, stream) : launch_prefill_il_one<T, C, false>(kp, stream);
 }
 template <typename T, int D, int BN>
-int launch_prefill_il(const KParams& kp, hipStream_t stream) { return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream); }
+int launch_prefill_il(const KParams& kp, hipStream_t stream) {
+    if constexpr (D == 128) {
+        if (kp.p.d <= 96 && !(kp.p.p_dropout > 0.f)) return launch_prefill_il_one<T, ILCfg<T, D, BN, 96>, false>(kp, stream);
+    }
+    return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream);
+}
 template <typename T>
-int launch_prefill_il_pair(const KParams& kp, hipStream_t stream) { return launch_prefill_il_cfg<T, ILCfgPair<T>>(kp, stream); }
+int launch_prefill_il_pair(const KParams& kp, hipStream_t stream) {
+    if (kp.p.d <= 192 && !(kp.p.p_dropout > 0.f)) return launch_prefill_il_one<T, ILCfgPair<T, 192>, false>(kp, stream);
+    return launch_prefill_il_cfg<T, ILCfgPair<T>>(kp, stream);
+}
 
 }  // namespace fa

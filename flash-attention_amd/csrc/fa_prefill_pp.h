@@ -66,9 +66,14 @@ __device__ long long fa_pp_dbg[FA_PP_DBG_BLOCKS * 2 * 16];
 #define FA_PP_REALTIME(i) do {} while (0)
 #endif
 
-template <typename T, int D, int BN, bool DROPOUT = false>
+// DV: head dims the products run over (a multiple of 32, p.d <= DV <= D).  Tiles keep the LDS layout of the
+// bucket D; with DV < D the k-steps and output column blocks past DV are not computed (head dim 96 on the
+// 128 bucket: 6 of 8 k-steps of S, 3 of 4 column blocks of O).
+template <typename T, int D, int BN, bool DROPOUT = false, int DV = D>
 __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     typedef PPCfg<T, D, BN> C;
+    static_assert(DV % 32 == 0 && DV <= D, "computed head dims");
+    constexpr int KSV = DV / 16, DBV = DV / 32;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_fwd_params& p = kp.p;
@@ -182,12 +187,12 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     }
     FA_PP_STAMP(1);
 
-    v8 qf[C::KS];
+    v8 qf[KSV];
     {
         const bool valid = row < si.sq;
         const T* qrow = qg + (int64_t)row * p.q_row_stride;
 #pragma unroll
-        for (int dk = 0; dk < C::KS; dk++) {
+        for (int dk = 0; dk < KSV; dk++) {
             const int d0 = dk * 16 + 8 * hh;
             u32x4 raw = {0, 0, 0, 0};
             if (valid && d0 < p.d) raw = ld_global16(qrow + d0);
@@ -196,9 +201,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     }
 
     FA_PP_STAMP(10);      // q loads issued
-    f32x16 o_acc[C::DB];
+    f32x16 o_acc[DBV];
 #pragma unroll
-    for (int db = 0; db < C::DB; db++)
+    for (int db = 0; db < DBV; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o_acc[db][r] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
@@ -225,20 +230,20 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 
     // ---- S^T = K Q^T.  Fragment reads run LA matrix instructions ahead of their use and are
     // interleaved one-for-one with the MFMAs.
-    int kofs[C::KS];
+    int kofs[KSV];
 #pragma unroll
-    for (int dk = 0; dk < C::KS; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dk * 2 + hh, l32) * 16;
+    for (int dk = 0; dk < KSV; dk++) kofs[dk] = l32 * C::ROWB + swz_k<D>(dk * 2 + hh, l32) * 16;
     f32x16 s_acc[C::NB];
     auto qk = [&](int i) {
         // one address register per k-step, advanced to the tile's ring slot once; every other
         // displacement is an instruction immediate
         const int slot = (i & (C::NS - 1)) * C::TILE;
-        const char* kb[C::KS];
+        const char* kb[KSV];
 #pragma unroll
-        for (int dk = 0; dk < C::KS; dk++) kb[dk] = smem + (slot + kofs[dk]);
-        constexpr int NF = C::NB * C::KS;          // fragments in (nb, dk) order
+        for (int dk = 0; dk < KSV; dk++) kb[dk] = smem + (slot + kofs[dk]);
+        constexpr int NF = C::NB * KSV;          // fragments in (nb, dk) order
         constexpr int LA = FA_PP_LA;
-        auto frag_ptr = [&](int f) { return kb[f % C::KS] + (f / C::KS) * 32 * C::ROWB; };
+        auto frag_ptr = [&](int f) { return kb[f % KSV] + (f / KSV) * 32 * C::ROWB; };
         u32x4 fr[LA];
 #pragma unroll
         for (int e = 0; e < LA; e++) fr[e] = *reinterpret_cast<const u32x4*>(frag_ptr(e));
@@ -248,7 +253,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             for (int r = 0; r < 16; r++) s_acc[nb][r] = 0.f;
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            s_acc[f / C::KS] = Elem<T>::mfma32(__builtin_bit_cast(v8, fr[f % LA]), qf[f % C::KS], s_acc[f / C::KS]);
+            s_acc[f / KSV] = Elem<T>::mfma32(__builtin_bit_cast(v8, fr[f % LA]), qf[f % KSV], s_acc[f / KSV]);
             if (f + LA < NF) fr[f % LA] = *reinterpret_cast<const u32x4*>(frag_ptr(f + LA));
         }
         __builtin_amdgcn_sched_group_barrier(0x100, LA, 0);      // look-ahead reads
@@ -261,20 +266,20 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 
     // ---- O^T += V^T P^T, same interleave with two transposing reads per MFMA
     const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
-    int vofs[C::DB];
+    int vofs[DBV];
 #pragma unroll
-    for (int db = 0; db < C::DB; db++)
+    for (int db = 0; db < DBV; db++)
         vofs[db] = (4 * hh + tj) * C::ROWB + swz_v<D>(db * 4 + dhalf * 2 + (tq >> 1), 4 * hh + tj) * 16 + (tq & 1) * 8;
     v8 pf[C::PT];
     auto pv = [&](int i) {
         const int slot = (C::NS + (i & (C::NS - 1))) * C::TILE;
-        const char* vb[C::DB];
+        const char* vb[DBV];
 #pragma unroll
-        for (int db = 0; db < C::DB; db++) vb[db] = smem + (slot + vofs[db]);
-        constexpr int NF = C::PT * C::DB;          // fragments in (t16, db) order
+        for (int db = 0; db < DBV; db++) vb[db] = smem + (slot + vofs[db]);
+        constexpr int NF = C::PT * DBV;          // fragments in (t16, db) order
         constexpr int LA = FA_PP_LA;
         auto fetch = [&](int f) {
-            const int t16 = f / C::DB, db = f % C::DB;
+            const int t16 = f / DBV, db = f % DBV;
             const u32x2 lo = lds_read_tr16(vb[db] + t16 * 16 * C::ROWB);
             const u32x2 hi = lds_read_tr16(vb[db] + (t16 * 16 + 8) * C::ROWB);
             return (u32x4){lo[0], lo[1], hi[0], hi[1]};
@@ -284,7 +289,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         for (int e = 0; e < LA; e++) fr[e] = fetch(e);
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            o_acc[f % C::DB] = Elem<T>::mfma32(__builtin_bit_cast(v8, fr[f % LA]), pf[f / C::DB], o_acc[f % C::DB]);
+            o_acc[f % DBV] = Elem<T>::mfma32(__builtin_bit_cast(v8, fr[f % LA]), pf[f / DBV], o_acc[f % DBV]);
             if (f + LA < NF) fr[f % LA] = fetch(f + LA);
         }
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * LA, 0);  // look-ahead reads
@@ -353,7 +358,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             // merges this block into that branch and copies all of o_acc around it on every tile)
             if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
 #pragma unroll
-                for (int db = 0; db < C::DB; db++)
+                for (int db = 0; db < DBV; db++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
             }
@@ -372,7 +377,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             const float corr = move ? fast_exp2((m_run - m_new) * sl2) : 1.f;   // m_run = -inf -> 0
             l_run *= corr;
 #pragma unroll
-            for (int db = 0; db < C::DB; db++)
+            for (int db = 0; db < DBV; db++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
             m_run = m_new;
@@ -455,7 +460,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         constexpr int PITCH = C::ROWB + 16;
         char* stage = smem + wave * (32 * PITCH);
 #pragma unroll
-        for (int db = 0; db < C::DB; db++)
+        for (int db = 0; db < DBV; db++)
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const int d0 = db * 32 + 8 * q4 + 4 * hh;
@@ -480,7 +485,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #endif
 }
 
-template <typename T, int D, int BN, bool DROPOUT>
+template <typename T, int D, int BN, bool DROPOUT, int DV = D>
 int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     typedef PPCfg<T, D, BN> C;
     kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
@@ -489,7 +494,7 @@ int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     const int64_t nblocks = xcd_grid(kp.p, kp.num_m_blocks);
     if (nblocks == 0) return -2;
     dim3 grid((unsigned)nblocks), block(C::kThreads);
-    auto kern = prefill_pp_kernel<T, D, BN, DROPOUT>;
+    auto kern = prefill_pp_kernel<T, D, BN, DROPOUT, DV>;
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
@@ -497,7 +502,11 @@ int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
 }
 template <typename T, int D, int BN>
 int launch_prefill_pp(const KParams& kp, hipStream_t stream) {
-    return kp.p.p_dropout > 0.f ? launch_prefill_pp_one<T, D, BN, true>(kp, stream) : launch_prefill_pp_one<T, D, BN, false>(kp, stream);
+    if (kp.p.p_dropout > 0.f) return launch_prefill_pp_one<T, D, BN, true>(kp, stream);
+    if constexpr (D == 128) {
+        if (kp.p.d <= 96) return launch_prefill_pp_one<T, D, BN, false, 96>(kp, stream);
+    }
+    return launch_prefill_pp_one<T, D, BN, false>(kp, stream);
 }
 
 }  // namespace fa

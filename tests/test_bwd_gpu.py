@@ -154,7 +154,7 @@ def test_backward_varlen_packed_forms(d):
                      qkv[a:e, 2][None], dout[a:e][None], causal=True)
 
 
-@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("d", [64, 80, 96, 128, 160, 192, 256])
 @pytest.mark.parametrize("mode", ["causal", "local"])
 def test_backward_long_sequences(d, mode):
     """Lengths at which the forward runs its long-sequence kernels and the backward streams many tiles."""

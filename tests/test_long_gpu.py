@@ -84,7 +84,8 @@ def test_pipelined_kernel_rectangular(sq, sk, dtype, mode):
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
-@pytest.mark.parametrize("case", ["full_2304", "causal_4200", "local_4500", "rect_causal", "rect_local", "d96_full"])
+@pytest.mark.parametrize("case", ["full_2304", "causal_4200", "local_4500", "rect_causal", "rect_local", "d96_full",
+                                  "d96_causal", "d80_local", "d72_rect_causal"])
 def test_pingpong_kernel(case):
     _say("ping-pong", case)
     dtype = torch.bfloat16
@@ -99,6 +100,12 @@ def test_pingpong_kernel(case):
         b, h, sq, sk, causal, window = 3, 8, 2000, 4500, True, (-1, -1)     # 192 row blocks of 256: more than half the CUs
     elif case == "rect_local":
         b, h, sq, sk, causal, window = 2, 8, 4300, 2100, False, (700, 50)      # sq > sk: leading rows see nothing
+    elif case == "d96_causal":       # head dims 65..96 take the kernel's 96-column variant
+        b, h, sq, sk, causal, window, d = 1, 8, 4200, 4200, True, (-1, -1), 96
+    elif case == "d80_local":
+        b, h, sq, sk, causal, window, d = 1, 8, 4500, 4500, False, (1000, 300), 80
+    elif case == "d72_rect_causal":
+        b, h, sq, sk, causal, window, d = 3, 8, 2000, 4500, True, (-1, -1), 72
     else:
         b, h, sq, sk, causal, window, d = 2, 8, 2100, 2100, False, (-1, -1), 96
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
