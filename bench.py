@@ -220,7 +220,8 @@ def bench_varlen(steps, warmup):
         tflops = flops / (ms * 1e-3) / 1e12
         res["d%d" % d] = {"ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": total / (ms * 1e-3),
                           "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                                       "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                                       "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("varlen_bf16_d%d_64seq_h16" % d),
+                                       "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
                                        "kernel": "fa::prefill_pp_kernel<bf16,128,64>" if d == 128 else "fa::prefill_il_kernel<bf16,pair 256>",
                                        "flops_per_launch": flops}}
         del q, k, v
@@ -337,6 +338,9 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", default=None,
+                    choices=["prefill", "mfma_peak", "decode", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
+                    help="run one leg alone and print its record (for profiler runs: the trace then holds that leg's kernels only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
                          "FETCH_SIZE / WRITE_SIZE can be scaled against a kernel of known traffic")
@@ -358,6 +362,12 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if a.only:
+        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "decode": bench_decode, "rotary": bench_rotary,
+               "backward": bench_backward, "fwd_bwd": bench_fwd_bwd, "varlen": bench_varlen, "gqa_window": bench_gqa_window,
+               "head_dims": bench_head_dims}[a.only]
+        print(json.dumps({"only": a.only, "steps": a.steps, "warmup": a.warmup, a.only: leg(a.steps, a.warmup)}))
+        return
     pre = bench_prefill(a.steps, a.warmup)
     peak = bench_mfma_peak(a.steps, a.warmup)
     pre["roofline"]["measured_peak"] = peak["random_bf16"]["tflops"]

@@ -1,0 +1,83 @@
+"""Model of how an MI355X hands the workgroups of a grid to the CUs of one XCD, used to choose the work order
+of the forward and backward kernels (xcd_stream_unit in csrc/fa_common.h).
+
+Observed with per-workgroup time stamps and HW_ID (benchmarks/pp_stage_timing.py): the workgroups that fall
+to an XCD go to its 4 shader engines in strict rotation and in order.  Workgroup j waits until engine j mod 4
+has a free CU (8 CUs per engine; one 8-wave workgroup of these kernels fills a CU), and workgroup j + 1 is
+not started before workgroup j, even if its own engine has idle CUs.  `in_order` replays that rule,
+`any_free_cu` is the ideal dispatcher for comparison.  Cost of a workgroup of the ping-pong forward kernel:
+1.68 us per key tile + 12.2 us (from the same stamps).
+
+    python flash-attention_amd/benchmarks/dispatch_model.py
+
+prints, for the causal benchmark shape (16 streams of 32 row blocks per XCD) and for packed batches of 64
+sequences of U[128, 4096] tokens on 16 heads, the time an XCD needs and the fraction of it its CUs are busy.
+"""
+import heapq
+import random
+
+
+def cost(tiles):
+    return 1.68 * tiles + 12.2 if tiles > 0 else 1.0       # a workgroup with nothing to do still takes a slot
+
+
+def in_order(costs, engines=4, cus=8):
+    free = [[0.0] * cus for _ in range(engines)]
+    t_prev = end = 0.0
+    for j, c in enumerate(costs):
+        f = free[j % engines]
+        t = max(t_prev, heapq.heappop(f))
+        heapq.heappush(f, t + c)
+        t_prev, end = t, max(end, t + c)
+    return end, sum(costs) / (end * engines * cus)
+
+
+def any_free_cu(costs, cus=32):
+    free = [0.0] * cus
+    end = 0.0
+    for c in costs:
+        t = heapq.heappop(free)
+        heapq.heappush(free, t + c)
+        end = max(end, t + c)
+    return end, sum(costs) / (end * cus)
+
+
+def interleaved(streams, k):
+    """streams: per stream the tile counts of its units, heaviest first.  k streams at a time, unit-major."""
+    out = []
+    for g in range(0, len(streams), k):
+        grp = streams[g:g + k]
+        for u in range(max(len(s) for s in grp)):
+            out += [cost(s[u]) if u < len(s) else cost(0) for s in grp]
+    return out
+
+
+def causal_stream(length, units, rows=256, bn=64):
+    """tile counts of the row blocks of a causal sequence, last block first; `units` blocks are launched"""
+    t = []
+    for mb in range(units - 1, -1, -1):
+        t.append(0 if mb * rows >= length else (min((mb + 1) * rows, length) + bn - 1) // bn)
+    return t
+
+
+def show(name, costs):
+    a, b = in_order(costs), any_free_cu(costs)
+    print("  %-44s in-order rotation %6.0f us, CUs busy %.3f | any free CU %6.0f us, %.3f" % (name, a[0], a[1], b[0], b[1]))
+
+
+if __name__ == "__main__":
+    print("bf16 (4, 8192, 32, 128) causal: 16 streams per XCD, 32 row blocks each")
+    dense = [causal_stream(8192, 32) for _ in range(16)]
+    for k in (1, 2, 4):
+        show("%d stream%s at a time" % (k, "" if k == 1 else "s"), interleaved(dense, k))
+    for seed in range(4):
+        rng = random.Random(seed)
+        lens = [rng.randint(128, 4096) for _ in range(64)]
+        units = (max(lens) + 255) // 256
+        print("packed batch, 64 sequences U[128, 4096], 16 heads (an XCD gets 2 heads of every sequence), draw %d" % seed)
+        two_heads = [causal_stream(n, units) for n in lens for _ in range(2)]
+        show("as shipped: 2 streams at a time", interleaved(two_heads, 2))
+        show("4 streams at a time", interleaved(two_heads, 4))
+        by_len = [causal_stream(n, (n + 255) // 256) for n in sorted(lens, reverse=True) for _ in range(2)]
+        show("sorted by length, no empty units, 4 at a time", interleaved(by_len, 4))
+        show("all workgroups in falling cost", sorted(interleaved(two_heads, 2), reverse=True))
