@@ -91,9 +91,10 @@ struct ILCfgPair {
 
 // Occupancy: two workgroups per CU at head dim 128 (about 250 registers); at head dim 64, where the
 // vector work per matrix instruction doubles and a third wave per SIMD adds the issue slots it needs,
-// three workgroups in 168 registers each (measured +3..10 %).
+// three workgroups in 168 registers each (measured +3..10 %); the dropout variant, whose mask arithmetic
+// does not fit 168 registers without spilling, stays at two.
 template <typename T, typename C, bool DROPOUT = false>
-__global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2) prefill_il_kernel(const KParams kp) {
+__global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROPOUT) ? 3 : 2) prefill_il_kernel(const KParams kp) {
     constexpr int D = C::D, BN = C::BN;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -106,7 +107,7 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64) ? 3 : 2
     const int G = p.h / p.h_k;
     int g, mb, hk, b;
     if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks,
-                       !(kp.has_left || kp.has_right) ? 0u : C::kPair ? 32u : (C::D == 64 ? 96u : 64u), g, mb, hk, b)) return;
+                       !(kp.has_left || kp.has_right) ? 0u : C::kPair ? 32u : ((C::D == 64 && !DROPOUT) ? 96u : 64u), g, mb, hk, b)) return;
     const int head = hk * G + g;
 
     const SeqInfo si = seq_info(p, b);
