@@ -164,6 +164,7 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.rotary_q = 0;
     kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = 0;
     kp.work_counter = q.work_counter;
+    kp.work_items = nullptr;
 }
 
 static int run_attention(KParams& kp, hipStream_t stream) {
@@ -319,6 +320,12 @@ int fa_plan_splits(const fa_fwd_params* p, int32_t api, int32_t* num_splits) {
     if (api != 0 && api != 2) return fail("api must be 0 (fa_fwd) or 2 (fa_fwd_kvcache)");
     *num_splits = plan(*p, true).splits;
     return 0;
+}
+
+int64_t fa_work_list_words(const fa_fwd_params* p) {
+    if (!p || p->h_k <= 0 || p->h <= 0 || p->h % p->h_k != 0) return FA_WORK_COUNTER_WORDS;
+    const int64_t w = work_list_words(*p);
+    return w > FA_WORK_COUNTER_WORDS ? w : FA_WORK_COUNTER_WORDS;
 }
 
 int fa_fwd(const fa_fwd_params* p, void* hip_stream) {

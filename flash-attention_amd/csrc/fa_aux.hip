@@ -28,6 +28,114 @@ int launch_combine(const KParams& kp, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------------
+// Work list of a packed (variable-length) forward launch.
+//
+// The hardware hands the workgroups that fall to an XCD to its 4 shader engines in strict rotation and in
+// order (see xcd_stream_unit).  The arithmetic order of packed batches cannot follow that rule well: it
+// does not know the lengths, so the row blocks a short sequence does not have are empty workgroups in the
+// middle of the order, and streams of unequal length run side by side.  This kernel reads cu_seqlens_q on
+// the device and writes, per XCD, the list the attention kernel then walks: sequences by falling length
+// (so neighbouring streams cost about the same), four streams at a time, row block by row block from the
+// last (heaviest under a causal mask) down, and nothing for row blocks that do not exist.  The slots of
+// the grid past the end of a list exit at once, after all work has been handed out.
+// XCD x owns q heads of kv-head parts x, x + 8, ... of every sequence (h_k * parts is a multiple of 8), as
+// in the arithmetic order.  One workgroup per XCD.
+// ------------------------------------------------------------------------------------------------
+struct WorkListParams {
+    const int32_t* cu_seqlens_q;
+    int32_t b, h_k, G, parts, block_m, nmb, per_xcd;
+    int32_t* out;            // kWorkListHeaderWords counts, then 8 lists of per_xcd two-word slots
+};
+__global__ void __launch_bounds__(1024) work_list_kernel(const WorkListParams w) {
+    __shared__ int len_s[kWorkListMaxBatch];
+    __shared__ int order_s[kWorkListMaxBatch];       // rank -> batch index
+    __shared__ int scan_s[256];
+    const int x = blockIdx.x, t = threadIdx.x, nb = w.b;
+    for (int i = t; i < nb; i += 1024) len_s[i] = max(w.cu_seqlens_q[i + 1] - w.cu_seqlens_q[i], 0);
+    __syncthreads();
+    for (int i = t; i < nb; i += 1024) {
+        const int li = len_s[i];
+        int r = 0;
+        for (int j = 0; j < nb; j++) r += (len_s[j] > li || (len_s[j] == li && j < i)) ? 1 : 0;
+        order_s[r] = i;
+    }
+    __syncthreads();
+    const int Gp = w.G / w.parts, E = (w.h_k * w.parts / 8) * Gp;     // streams per sequence on this XCD
+    const int ns = nb * E, ng = (ns + 3) / 4;
+    // (a length beyond the seqlen_q the grid was sized for is the caller's error; it must not overrun the list)
+    auto units = [&](int s) { return s < ns ? min((len_s[order_s[s / E]] + w.block_m - 1) / w.block_m, w.nmb) : 0; };
+    // Four threads per owner: owner o holds groups [o * gpt, (o + 1) * gpt), thread j of it writes stream j of
+    // each.  Items before an owner's groups: inclusive scan over the owners' totals.
+    const int o = t >> 2, jj = t & 3;
+    const int gpt = (ng + 255) / 256;
+    const int g_lo = min(o * gpt, ng), g_hi = min(g_lo + gpt, ng);
+    int mine = 0;
+    for (int g = g_lo; g < g_hi; g++) mine += units(4 * g) + units(4 * g + 1) + units(4 * g + 2) + units(4 * g + 3);
+    if (jj == 0) scan_s[o] = mine;
+    __syncthreads();
+    const int owners = min(256, (ng + gpt - 1) / gpt);      // owners with work; the others hold zero
+    for (int d = 1; d < owners; d <<= 1) {
+        const int v = (jj == 0 && o >= d) ? scan_s[o - d] : 0;
+        __syncthreads();
+        if (jj == 0) scan_s[o] += v;
+        __syncthreads();
+    }
+    int off = scan_s[o] - mine;
+    if (t == 0) w.out[x] = owners > 0 ? scan_s[owners - 1] : 0;
+    int32_t* list = w.out + kWorkListHeaderWords + (size_t)x * w.per_xcd * 2;
+    for (int g = g_lo; g < g_hi; g++) {
+        int u[4];
+        for (int j = 0; j < 4; j++) u[j] = units(4 * g + j);
+        const int s = 4 * g + jj;
+        if (s < ns) {
+            const int bb = order_s[s / E], e = s % E;
+            const int hkp = x + 8 * (e / Gp);
+            const int head = (hkp / w.parts) * w.G + (hkp % w.parts) * Gp + e % Gp;
+            const int mine_u = u[jj];
+            for (int un = 0; un < mine_u; un++) {
+                // unit-major inside the group; lengths fall with the stream index, so the streams that still
+                // have unit `un` are a prefix of the group
+                const int pos = off + min(u[0], un) + min(u[1], un) + min(u[2], un) + min(u[3], un) + jj;
+                list[2 * pos] = bb;
+                list[2 * pos + 1] = (int32_t)(((uint32_t)head << 16) | (uint32_t)(mine_u - 1 - un));
+            }
+        }
+        off += u[0] + u[1] + u[2] + u[3];
+    }
+}
+
+static bool work_list_applies(const fa_fwd_params& p) {
+    if (!p.cu_seqlens_q || p.b <= 0 || p.b > kWorkListMaxBatch || p.h >= 65536) return false;
+    const uint32_t G = (uint32_t)(p.h / p.h_k), parts = xcd_parts(true, true, (uint32_t)p.h_k, G);
+    return ((uint32_t)p.h_k * parts) % 8u == 0u;
+}
+int64_t work_list_words(const fa_fwd_params& p) {
+    if (!work_list_applies(p)) return 0;
+    // the smallest row block (128 rows) gives the longest lists
+    const int64_t nmb = (p.seqlen_q + 127) / 128;
+    return FA_WORK_COUNTER_WORDS + kWorkListHeaderWords + 2 * xcd_grid(p, nmb);
+}
+int prepare_work_list(KParams& kp, int block_m, int64_t nblocks, hipStream_t stream) {
+    const fa_fwd_params& p = kp.p;
+    kp.work_items = nullptr;
+    if (!work_list_applies(p) || !kp.work_counter || nblocks <= 0 || (nblocks & 7) != 0) return 0;
+    if ((p.seqlen_q + block_m - 1) / block_m >= 65536) return 0;
+    if ((int64_t)p.work_counter_len < FA_WORK_COUNTER_WORDS + kWorkListHeaderWords + 2 * nblocks) return 0;
+    WorkListParams w;
+    w.cu_seqlens_q = p.cu_seqlens_q;
+    w.b = p.b; w.h_k = p.h_k; w.G = p.h / p.h_k;
+    w.parts = (int32_t)xcd_parts(true, true, (uint32_t)p.h_k, (uint32_t)w.G);
+    w.block_m = block_m;
+    w.nmb = (p.seqlen_q + block_m - 1) / block_m;
+    w.per_xcd = (int32_t)(nblocks / 8);
+    w.out = kp.work_counter + FA_WORK_COUNTER_WORDS;
+    hipLaunchKernelGGL(work_list_kernel, dim3(8), dim3(1024), 0, stream, w);
+    if (int e = (int)hipGetLastError()) return e;
+    kp.work_items = w.out;
+    return 0;
+}
+
 // One thread per 16-byte chunk of one new (token, kv-head) row.
 template <typename T>
 __global__ void __launch_bounds__(256) append_kv_kernel(const KParams kp) {

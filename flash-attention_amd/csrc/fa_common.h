@@ -57,7 +57,13 @@ struct KParams {
     // dec_append: the item that reaches rows [cache length, cache length + seqlen_knew) writes them
     int32_t dec_persistent, dec_sa, dec_sb, dec_sub, dec_append;
     int32_t* work_counter;
+    // Packed batches: work list built on the device from cu_seqlens_q just before the launch (work_list_kernel,
+    // fa_aux.hip), or NULL.  8 item counts, then for XCD x a list of (gridDim.x / 8) slots of two words:
+    // batch index, (q head << 16) | row block.
+    const int32_t* work_items;
 };
+constexpr int kWorkListHeaderWords = 8;
+constexpr int kWorkListMaxBatch = 2048;      // sequences the list builder ranks (quadratic, in LDS)
 
 template <typename T> struct Elem;
 template <> struct Elem<__bf16> {
@@ -652,8 +658,21 @@ inline int64_t xcd_rows_grid(bool split, bool varlen, int64_t batch, int64_t h_k
     const int64_t parts = xcd_parts(split, varlen, (uint32_t)h_k, (uint32_t)G);
     return xcd_grid(xcd_strided(varlen, batch, h_k * parts), batch, h_k * parts, G / parts * nmb);
 }
-FA_DEV bool xcd_work_item(const fa_fwd_params& p, uint32_t nmb, uint32_t slots, int& g, int& mb, int& hk, int& b) {
-    return xcd_rows_item(true, p.cu_seqlens_q != nullptr, (uint32_t)p.b, (uint32_t)p.h_k, (uint32_t)(p.h / p.h_k), nmb, slots, g, mb, hk, b);
+FA_DEV bool xcd_work_item(const KParams& kp, uint32_t nmb, uint32_t slots, int& g, int& mb, int& hk, int& b) {
+    const fa_fwd_params& p = kp.p;
+    const uint32_t G = (uint32_t)(p.h / p.h_k);
+    if (kp.work_items) {
+        const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+        if (j >= (uint32_t)kp.work_items[x]) return false;      // the slots past the list come last in the grid
+        const int32_t* it = kp.work_items + kWorkListHeaderWords + ((size_t)x * (gridDim.x >> 3) + j) * 2;
+        b = it[0];
+        const uint32_t w = (uint32_t)it[1], head = w >> 16;
+        mb = (int)(w & 0xffffu);
+        hk = (int)(head / G);
+        g = (int)(head % G);
+        return true;
+    }
+    return xcd_rows_item(true, p.cu_seqlens_q != nullptr, (uint32_t)p.b, (uint32_t)p.h_k, G, nmb, slots, g, mb, hk, b);
 }
 inline int64_t xcd_grid(const fa_fwd_params& p, int64_t nmb) {
     return xcd_rows_grid(true, p.cu_seqlens_q != nullptr, p.b, p.h_k, p.h / p.h_k, nmb);

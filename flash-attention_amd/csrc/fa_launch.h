@@ -22,6 +22,11 @@ int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split
 int launch_append_kv(const KParams& kp, hipStream_t stream);
 int launch_attn_probs(const KParams& kp, hipStream_t stream);  // s_dmask: signed softmax probabilities (testing)
 int launch_rotary(const fa_rotary_params& p, hipStream_t stream);   // standalone rotary embedding
+// Packed batches: builds the work list of a forward launch of `nblocks` workgroups with row blocks of
+// `block_m` rows in kp.p.work_counter and sets kp.work_items, when the batch qualifies and the caller lent
+// enough words (fa_work_list_words); otherwise leaves kp.work_items NULL.
+int prepare_work_list(KParams& kp, int block_m, int64_t nblocks, hipStream_t stream);
+int64_t work_list_words(const fa_fwd_params& p);    // words behind work_counter that make every packed launch qualify
 
 #define FA_DECL_BWD(name) int name(const BwdKParams& kp, hipStream_t stream);
 FA_DECL_BWD(launch_bwd_bf16_64)

@@ -24,6 +24,7 @@
 // of O that a moved max needs is applied after the step's matrix instructions.
 #pragma once
 #include "fa_common.h"
+#include "fa_launch.h"
 #include "fa_prefill_pp.h"
 
 namespace fa {
@@ -106,7 +107,7 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
 
     const int G = p.h / p.h_k;
     int g, mb, hk, b;
-    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks,
+    if (!xcd_work_item(kp, (uint32_t)kp.num_m_blocks,
                        !(kp.has_left || kp.has_right) ? 0u : C::kPair ? 32u : ((C::D == 64 && !DROPOUT) ? 96u : 64u), g, mb, hk, b)) return;
     const int head = hk * G + g;
 
@@ -607,6 +608,7 @@ int launch_prefill_il_one(KParams kp, hipStream_t stream) {
     const int64_t nblocks = xcd_grid(kp.p, kp.num_m_blocks);
     if (nblocks == 0) return -2;
     dim3 grid((unsigned)nblocks), block(C::kThreads);
+    if (int e = prepare_work_list(kp, C::BM, nblocks, stream)) return e;
     auto kern = prefill_il_kernel<T, C, DROPOUT>;
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;

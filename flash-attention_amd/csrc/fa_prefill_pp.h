@@ -26,6 +26,7 @@
 // keeping every probability <= 256 (exact in the final normalisation, safe in fp16/bf16).
 #pragma once
 #include "fa_common.h"
+#include "fa_launch.h"
 
 namespace fa {
 
@@ -92,7 +93,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
     const uint32_t G = (uint32_t)(p.h / p.h_k);
     int g, mb, hk, b;
-    if (!xcd_work_item(p, (uint32_t)kp.num_m_blocks, (kp.has_left || kp.has_right) ? 32u : 0u, g, mb, hk, b)) return;
+    if (!xcd_work_item(kp, (uint32_t)kp.num_m_blocks, (kp.has_left || kp.has_right) ? 32u : 0u, g, mb, hk, b)) return;
     const int head = hk * (int)G + g;
     FA_PP_STAMP(8);       // work item known
 
@@ -494,6 +495,7 @@ int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     const int64_t nblocks = xcd_grid(kp.p, kp.num_m_blocks);
     if (nblocks == 0) return -2;
     dim3 grid((unsigned)nblocks), block(C::kThreads);
+    if (int e = prepare_work_list(kp, C::BM, nblocks, stream)) return e;
     auto kern = prefill_pp_kernel<T, D, BN, DROPOUT, DV>;
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;

@@ -89,6 +89,8 @@ def _load():
         f.argtypes = [P, ctypes.c_void_p]
         f.restype = ctypes.c_int
     lib.fa_plan_splits.argtypes = [P, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32)]
+    lib.fa_work_list_words.argtypes = [P]
+    lib.fa_work_list_words.restype = ctypes.c_int64
     lib.fa_plan_splits.restype = ctypes.c_int
     lib.fa_num_splits_heuristic_reference.argtypes = [ctypes.c_int32] * 4
     lib.fa_num_splits_heuristic_reference.restype = ctypes.c_int
@@ -206,6 +208,10 @@ def _dropout_state(p, p_dropout, return_softmax, gen_, batch, heads, seqlen_q, s
 _COUNTERS = {}     # (device index, stream) -> zeroed int32 words lent to the persistent decode kernel
 
 
+_RETIRED = []
+WORK_LIST = True      # packed forward launches lend the library room for its device-built work list
+
+
 def _counters(device, words):
     """Counter words for launches on the current stream of `device`: zero when first handed out and left
     zero by every launch, so one tensor per (device, stream) serves all calls (launches on one stream do
@@ -214,6 +220,8 @@ def _counters(device, words):
     key = (index, _stream(device))
     t = _COUNTERS.get(key)
     if t is None or t.numel() < words:
+        if t is not None:
+            _RETIRED.append(t)      # a captured graph may still point at it
         t = torch.zeros((max(16, int(words)),), dtype=torch.int32, device=device)
         _COUNTERS[key] = t
     return t
@@ -376,6 +384,11 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
         rng_state, s_dmask = _dropout_state(p, p_dropout, return_softmax, gen_, batch_size, num_heads, max_seqlen_q,
                                             max_seqlen_k, q_dtype, q.device)
         if total_q > 0 and max_seqlen_q > 0:
+            # room for the work list the library builds from cu_seqlens_q on the device (WORK_LIST = False: the
+            # arithmetic order, for tests that compare the two)
+            words = lib.fa_work_list_words(ctypes.byref(p)) if WORK_LIST else 2
+            counter = _counters(q.device, words)
+            p.work_counter, p.work_counter_len = counter.data_ptr(), counter.numel()
             _call(lib.fa_varlen_fwd, p, _stream(q.device))
         elif s_dmask is not None:
             s_dmask.zero_()

@@ -59,13 +59,18 @@ typedef struct fa_fwd_params {
                                        per-batch key lengths (cache_seqlens), or NULL */
     const int32_t *cache_batch_idx; /* (b) row of k/v used (and updated) for batch i, or NULL */
     int32_t *work_counter;          /* optional: work_counter_len (>= FA_WORK_COUNTER_WORDS) int32 words of
-                                       device memory that are ZERO before the first call that uses them;
-                                       every call leaves them zero again.  When set, split-KV decode
-                                       launches run as a persistent kernel whose workgroups draw (batch,
-                                       kv head, key chunk) items from a ticket and whose item that
-                                       reaches the new rows appends them to the cache (no append
-                                       launch).  Must not be shared by calls that overlap on the GPU.
-                                       NULL: one workgroup per chunk and a separate append launch. */
+                                       device memory whose first FA_WORK_COUNTER_WORDS words are ZERO before
+                                       the first call that uses them; every call leaves those zero again.
+                                       When set, split-KV decode launches run as a persistent kernel whose
+                                       workgroups draw (batch, kv head, key chunk) items from a ticket and
+                                       whose item that reaches the new rows appends them to the cache (no
+                                       append launch).  Words past the first FA_WORK_COUNTER_WORDS are
+                                       scratch with no required contents: when there are at least
+                                       fa_work_list_words(p) words, fa_varlen_fwd first builds its work
+                                       list there on the device (sequences by falling length, no empty
+                                       workgroups between working ones).  Must not be shared by calls
+                                       that overlap on the GPU.  NULL: one workgroup per chunk, a
+                                       separate append launch, arithmetic work order. */
 
     int64_t q_batch_stride, q_row_stride, q_head_stride;
     int64_t k_batch_stride, k_row_stride, k_head_stride;
@@ -109,6 +114,14 @@ typedef struct fa_fwd_params {
 
 /* words the persistent decode kernel needs behind work_counter: ticket, exit count */
 #define FA_WORK_COUNTER_WORDS 2
+
+/*
+ * Words behind work_counter with which every launch of fa_varlen_fwd on these params (b, h, h_k, seqlen_q =
+ * max_seqlen_q) can build its work list; FA_WORK_COUNTER_WORDS when the batch does not qualify (more than
+ * 2048 sequences, or kv heads that do not spread evenly over the 8 XCDs).  No counterpart in the
+ * reference, whose grid order is fixed (flash_fwd_launch_template.h:33-77).  Results do not depend on it.
+ */
+int64_t fa_work_list_words(const fa_fwd_params *p);
 
 /*
  * Dense batch forward.  Replaces mha_fwd (csrc/flash_attn/flash_api.cpp:248-424): same masking
