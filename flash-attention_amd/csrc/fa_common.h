@@ -491,19 +491,26 @@ FA_DEV void combine_row(const KParams& kp, const int64_t row, const int lane) {
 
     // each lane owns 4 consecutive output dims (64 lanes x 4 = 256 dims max)
     const int d0 = lane * 4;
-    // The partial rows are fetched eight at a time before any of them is used (one memory round trip per
-    // batch instead of one per split) and added in split order; a split of weight zero may never have been
-    // written, so its row is fetched but not used.
+    // Only the splits of non-zero weight are fetched (a split of weight zero may never have been written: the
+    // slots past a sequence's length), eight rows at a time before any of them is used (one memory round
+    // trip per batch instead of one per split), and added in split order.  The set of splits is the same
+    // for all lanes of the wave, so the walk over it is scalar.
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     constexpr int BATCH = 8;
-    for (int s0 = 0; s0 < S; s0 += BATCH) {
+    uint64_t m0 = __builtin_amdgcn_ballot_w64(w0 != 0.f), m1 = __builtin_amdgcn_ballot_w64(w1 != 0.f);
+    while ((m0 | m1) != 0) {
         f32x4 v[BATCH];
         float w[BATCH];
+        int last = 0;
 #pragma unroll
         for (int j = 0; j < BATCH; j++) {
-            const int s = min(s0 + j, S - 1);
-            w[j] = s0 + j < S ? __shfl(s < 64 ? w0 : w1, s & 63) : 0.f;
-            const float* src = p.o_accum + ((int64_t)s * nrows + row) * kp.d_rounded + min(d0, kp.d_rounded - 4);
+            int sidx = -1;
+            if (m0 != 0) { sidx = __builtin_ctzll(m0); m0 &= m0 - 1; }
+            else if (m1 != 0) { sidx = 64 + __builtin_ctzll(m1); m1 &= m1 - 1; }
+            w[j] = sidx >= 0 ? __shfl(sidx < 64 ? w0 : w1, sidx & 63) : 0.f;
+            if (sidx >= 0) last = sidx;
+            // (past the end of the set the last row is fetched again, with weight zero)
+            const float* src = p.o_accum + ((int64_t)last * nrows + row) * kp.d_rounded + min(d0, kp.d_rounded - 4);
             v[j] = *reinterpret_cast<const f32x4*>(src);
         }
 #pragma unroll
