@@ -162,7 +162,7 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.split_len = 0;
     kp.num_m_blocks = 0;
     kp.rotary_q = 0;
-    kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = 0;
+    kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = kp.dec_compact = 0;
     kp.work_counter = q.work_counter;
     kp.work_items = nullptr;
 }
@@ -200,6 +200,7 @@ static int resolve_splits(KParams& kp, const fa_fwd_params& p, bool allow_split)
     kp.split_len = r.len;
     kp.dec_persistent = r.persistent;
     kp.dec_sa = r.sa; kp.dec_sb = r.sb; kp.dec_sub = r.sub;
+    kp.dec_compact = r.persistent && !kp.has_left && p.b <= kDecCompactMaxBatch;
     if (s > 1 && (!p.o_accum || !p.lse_accum)) return fail("o_accum and lse_accum are required when the key range is split (see fa_plan_splits)");
     return 0;
 }

@@ -55,13 +55,16 @@ struct KParams {
     // slots of dec_sub keys for each sequence's ragged remainder; tickets from work_counter[0], workgroups
     // that have left counted in [1].
     // dec_append: the item that reaches rows [cache length, cache length + seqlen_knew) writes them
-    int32_t dec_persistent, dec_sa, dec_sb, dec_sub, dec_append;
+    // dec_compact: the tickets cover only the slots that hold keys (the kernel counts them per batch entry
+    // from the lengths); the merge then derives which slots were written from the lengths as well
+    int32_t dec_persistent, dec_sa, dec_sb, dec_sub, dec_append, dec_compact;
     int32_t* work_counter;
     // Packed batches: work list built on the device from cu_seqlens_q just before the launch (work_list_kernel,
     // fa_aux.hip), or NULL.  8 item counts, then for XCD x a list of (gridDim.x / 8) slots of two words:
     // batch index, (q head << 16) | row block.
     const int32_t* work_items;
 };
+constexpr int kDecCompactMaxBatch = 1024;    // batch entries whose slot counts the persistent decode kernel scans in LDS
 constexpr int kWorkListHeaderWords = 8;
 constexpr int kWorkListMaxBatch = 2048;      // sequences the list builder ranks (quadratic, in LDS)
 
@@ -464,14 +467,24 @@ FA_DEV void store_tile_rows(const f32x16 (&acc)[DB], float sc, char* stage, int 
 // reduce the per-split log-sum-exp values, then stream the partial rows whose weight is non-zero.
 // Reference: combine_attn_seqk_parallel, csrc/flash_attn/src/flash_fwd_kernel.h:1169-1327 (all splits
 // empty: lse = +inf, out = 0, :1233-1241).
+FA_DEV void dec_slot_counts(const KParams& kp, int b, int& n_macro, int& n_sub);
 template <typename T>
 FA_DEV void combine_row(const KParams& kp, const int64_t row, const int lane) {
     const fa_fwd_params& p = kp.p;
     const int64_t nrows = (int64_t)p.b * p.h * p.seqlen_q;
     const int S = kp.num_splits;
 
-    float l0 = lane < S ? p.lse_accum[(int64_t)lane * nrows + row] : -INFINITY;
-    float l1 = lane + 64 < S ? p.lse_accum[(int64_t)(lane + 64) * nrows + row] : -INFINITY;
+    // which partial slots hold a result: all of them, or (compact persistent decode schedule, whose kernel
+    // visits and writes only the slots with keys) the leading complete chunks and the leading pieces of the
+    // remainder, as dec_slot_counts gives them
+    int n_a = S, n_b = 0, s_a = S;
+    if (kp.dec_compact) {
+        s_a = kp.dec_sa;
+        dec_slot_counts(kp, (int)(row / ((int64_t)p.seqlen_q * p.h)), n_a, n_b);
+    }
+    auto written = [&](int s) { return s < S && (s < s_a ? s < n_a : s - s_a < n_b); };
+    float l0 = written(lane) ? p.lse_accum[(int64_t)lane * nrows + row] : -INFINITY;
+    float l1 = written(lane + 64) ? p.lse_accum[(int64_t)(lane + 64) * nrows + row] : -INFINITY;
     float mx = fmaxf(l0, l1);
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
@@ -560,6 +573,17 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
     }
     s.q_row0 = 0;
     return s;
+}
+
+// Persistent decode schedule without a left window bound: the keys of batch entry b are [0, hi), hi = the
+// sequence's length (a right bound of the mask never hides keys from the last query row).  Slots with keys:
+// the first n_macro complete chunks of split_len keys, and the first n_sub pieces of dec_sub keys of the
+// remainder (decode_item, kMacro / kSub).
+FA_DEV void dec_slot_counts(const KParams& kp, int b, int& n_macro, int& n_sub) {
+    const int hi = seq_info(kp.p, b).sk;
+    const int whole = hi / kp.split_len;
+    n_macro = min(kp.dec_sa, whole);
+    n_sub = min(kp.dec_sb, (hi - whole * kp.split_len + kp.dec_sub - 1) / kp.dec_sub);
 }
 
 // Which work item a workgroup of the tiled forward and backward kernels takes.  Block ids are dealt round-robin

@@ -371,9 +371,41 @@ template <typename T, int D, bool APPEND>
 __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_ticket;
+    // compact schedule: s_pm[b] / s_ps[b] = slots with keys (complete chunks / remainder pieces) of the batch
+    // entries before b; tickets then number only those slots, batch entry by batch entry, kv heads fastest
+    __shared__ int s_pm[kDecCompactMaxBatch + 1], s_ps[kDecCompactMaxBatch + 1];
     const fa_fwd_params& p = kp.p;
-    const int n_macro = p.b * kp.dec_sa * p.h_k;
-    const int total = n_macro + p.b * kp.dec_sb * p.h_k;
+    int n_macro = p.b * kp.dec_sa * p.h_k;
+    int total = n_macro + p.b * kp.dec_sb * p.h_k;
+    if (kp.dec_compact) {
+        for (int bb = threadIdx.x; bb < p.b; bb += blockDim.x) {
+            int nm, ns;
+            dec_slot_counts(kp, bb, nm, ns);
+            s_pm[bb + 1] = nm;
+            s_ps[bb + 1] = ns;
+        }
+        __syncthreads();
+        if (threadIdx.x < 64) {        // one wave turns the counts into running sums, 64 entries at a time
+            const int lane = threadIdx.x;
+            int carry_m = 0, carry_s = 0;
+            for (int base = 0; base < p.b; base += 64) {
+                const int i = base + lane;
+                int vm = i < p.b ? s_pm[i + 1] : 0, vs = i < p.b ? s_ps[i + 1] : 0;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) {
+                    const int um = __shfl_up(vm, o), us = __shfl_up(vs, o);
+                    if (lane >= o) { vm += um; vs += us; }
+                }
+                if (i < p.b) { s_pm[i + 1] = carry_m + vm; s_ps[i + 1] = carry_s + vs; }
+                carry_m += __shfl(vm, 63);
+                carry_s += __shfl(vs, 63);
+            }
+            if (lane == 0) { s_pm[0] = 0; s_ps[0] = 0; }
+        }
+        __syncthreads();
+        n_macro = s_pm[p.b] * p.h_k;
+        total = n_macro + s_ps[p.b] * p.h_k;
+    }
     int32_t* const ticket = kp.work_counter;
     for (;;) {
         __syncthreads();          // previous item is done with LDS and with s_ticket
@@ -382,9 +414,23 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kern
         int t = s_ticket;
         if (t >= total) break;
         const bool macro = t < n_macro;
-        const int per_b = macro ? kp.dec_sa : kp.dec_sb;
         if (!macro) t -= n_macro;
-        const int hk = t % p.h_k, idx = (t / p.h_k) % per_b, b = t / (p.h_k * per_b);
+        int hk, idx, b;
+        if (kp.dec_compact) {
+            const int* pre = macro ? s_pm : s_ps;
+            hk = t % p.h_k;
+            const int q = t / p.h_k;            // q-th slot with keys of its pass: the batch entry is the last b with pre[b] <= q
+            int lo_b = 0, hi_b = p.b;           // invariant: pre[lo_b] <= q < pre[hi_b]
+            while (hi_b - lo_b > 1) {
+                const int mid = (lo_b + hi_b) >> 1;
+                if (pre[mid] <= q) lo_b = mid; else hi_b = mid;
+            }
+            b = lo_b;
+            idx = q - pre[b];
+        } else {
+            const int per_b = macro ? kp.dec_sa : kp.dec_sb;
+            hk = t % p.h_k; idx = (t / p.h_k) % per_b; b = t / (p.h_k * per_b);
+        }
         decode_item<T, D, true, APPEND>(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
     }
     if (threadIdx.x == 0) {

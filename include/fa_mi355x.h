@@ -36,7 +36,8 @@ extern "C" {
  *   o      like q
  *   softmax_lse  (b, h, seqlen_q) fp32, natural log; +inf for a row that sees no key
  *   o_accum      (num_splits, b, h, seqlen_q, d_rounded) fp32, d_rounded = d rounded up to 32
- *   lse_accum    (num_splits, b, h, seqlen_q) fp32
+ *   lse_accum    (num_splits, b, h, seqlen_q) fp32   (scratch of the call: slots that hold no keys may be left
+ *                                                    unwritten)
  * Masking is bottom-right aligned: query i sees key j iff
  *   i + sk - sq - window_left <= j <= i + sk - sq + window_right and j < sk,
  * a negative window bound meaning unbounded; is_causal forces window_right = 0.
