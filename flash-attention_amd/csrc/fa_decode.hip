@@ -360,7 +360,8 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 //  * The item whose key range reaches the new rows appends them (APPEND, see decode_item): no append launch.
 //  * work_counter[0] is the ticket, work_counter[1] counts the workgroups that have left; the last one puts
 //    both back to zero, so the words are zero again when the kernel ends and no launch has to reset them.
-// Measured and not adopted: drawing the next ticket early (before the item: the returning atomic sits in front
+// Measured and not adopted: drawing the next ticket when an item's key loop ends, so that the counter's round
+// trip runs under the merge and the output stores (+1 % on the step); drawing it early (before the item: the returning atomic sits in front
 // of the item's first K/V loads in the wave's in-order memory queue, +7 % time; after the item's last load:
 // no change, the second resident workgroup of the CU already covers the round trip), and merging a (batch,
 // kv head)'s partials in the kernel by the last of its items to arrive (the partials must bypass the per-XCD
@@ -407,11 +408,16 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kern
         total = n_macro + s_ps[p.b] * p.h_k;
     }
     int32_t* const ticket = kp.work_counter;
-    for (;;) {
-        __syncthreads();          // previous item is done with LDS and with s_ticket
-        if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        int t = s_ticket;
+    // the first item of a workgroup is the one its block id names (no round trip to the counter before any
+    // work starts); the tickets drawn afterwards continue behind the grid
+    for (bool first = true;; first = false) {
+        int t = (int)blockIdx.x;
+        if (!first) {
+            __syncthreads();          // previous item is done with LDS and with s_ticket
+            if (threadIdx.x == 0) s_ticket = (int)gridDim.x + __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            t = s_ticket;
+        }
         if (t >= total) break;
         const bool macro = t < n_macro;
         if (!macro) t -= n_macro;
