@@ -108,3 +108,46 @@ def test_work_list_words_reported_through_the_c_abi():
     assert nat.lib.fa_work_list_words(ctypes.byref(p)) == 2
     p.h, p.h_k, p.b = 16, 16, 5000                                 # more sequences than the builder ranks
     assert nat.lib.fa_work_list_words(ctypes.byref(p)) == 2
+
+
+@pytest.mark.parametrize("lens,h,hk,d", [
+    ([2300, 700, 4100, 128, 3000, 2048, 513, 1, 3500, 2600], 16, 16, 128),     # 256-row blocks, 2 heads of a sequence per XCD
+    ([600, 1500, 0, 1030, 777, 512, 64, 2000], 32, 8, 64),                        # 128-row blocks, 4 grouped heads, an empty sequence
+    ([2500, 900, 3100, 2200, 640], 8, 1, 128),                                     # MQA: 8 parts of one q head
+])
+def test_device_built_list_is_a_permutation_of_the_row_blocks(lens, h, hk, d):
+    """Reads the list back from the lent words after a launch: every (sequence, q head, row block) that
+    exists appears exactly once, on the XCD that owns its head, and nothing else appears."""
+    _say("list contents", lens, h, hk, d)
+    nat = _nat()
+    total, mx = sum(lens), max(lens)
+    gen = torch.Generator().manual_seed(11)
+    q = torch.randn(total, h, d, generator=gen).to(torch.bfloat16).to(DEV)
+    k, v = (torch.randn(total, hk, d, generator=gen).to(torch.bfloat16).to(DEV) for _ in range(2))
+    cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32).to(DEV)
+    nat.varlen_fwd(q, k, v, None, cu, cu, mx, mx, 0.0, d ** -0.5, False, True, -1, -1, False, None)
+    torch.cuda.synchronize()
+    dev = q.device
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), nat._stream(dev))
+    words = nat._COUNTERS[key].cpu().tolist()
+    assert words[0] == 0 and words[1] == 0                 # the ticket words stay zero
+    counts, body = words[2:10], words[10:]
+    block_m = 256 if d == 128 else 128                     # ping-pong kernel / pipelined kernel
+    n_mb = [(n + block_m - 1) // block_m for n in lens]
+    nmb_max = (mx + block_m - 1) // block_m
+    per_xcd = len(lens) * h // 8 * nmb_max                 # slots per XCD list
+    G = h // hk
+    parts = 1 if hk > 2 or G % (8 // hk) else 8 // hk
+    Gp = G // parts
+    seen = set()
+    for x in range(8):
+        assert 0 <= counts[x] <= per_xcd
+        for j in range(counts[x]):
+            b, w = body[(x * per_xcd + j) * 2], body[(x * per_xcd + j) * 2 + 1]
+            head, mb = (w >> 16) & 0xffff, w & 0xffff
+            assert 0 <= b < len(lens) and head < h and mb < n_mb[b], (x, j, b, head, mb)
+            hkp = (head // G) * parts + (head % G) // Gp       # kv head part the q head belongs to
+            assert hkp % 8 == x, "q head %d on XCD %d" % (head, x)
+            assert (b, head, mb) not in seen
+            seen.add((b, head, mb))
+    assert len(seen) == sum(n_mb) * h
