@@ -102,7 +102,7 @@ def test_backward_kvpacked_gqa(d, mode):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("mode", ["full", "causal", "local"])
-@pytest.mark.parametrize("d", [32, 64, 111, 128, 256])
+@pytest.mark.parametrize("d", [32, 64, 96, 111, 128, 160, 256])
 def test_backward_varlen(d, mode, dtype):
     """Packed sequences with different q and k lengths per sequence, an empty and a one-token one.
     Each sequence's gradients equal those of that sequence attended alone."""

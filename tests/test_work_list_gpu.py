@@ -35,6 +35,7 @@ CASES = [
     ([600, 1500, 90, 1030, 777, 512, 64, 2000, 1200], 16, 16, 64, True, (-1, -1)),               # pipelined kernel, head dim 64
     ([600, 1500, 90, 1030, 777, 512, 64, 2000, 1200], 8, 8, 256, True, (-1, -1)),                # pair kernel, head dim 256
     ([600, 1500, 90, 1030, 777, 512], 16, 8, 192, True, (-1, -1)),                               # pair kernel, 192 columns
+    ([2300, 700, 4100, 128, 3000, 2048, 513, 1], 16, 16, 96, True, (-1, -1)),                    # ping-pong kernel, 96 columns
     ([600, 1030, 90, 300, 2100], 12, 2, 128, True, (-1, -1)),                                    # 6 q heads per kv head: no list
     ([1, 2, 3], 8, 8, 128, True, (-1, -1)),                                                       # general kernel (short): no list
 ]
