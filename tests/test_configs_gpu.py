@@ -1,12 +1,16 @@
 """The five benchmark configurations at their full sizes on the GPU.
 
-The whole problem runs through the public API; the CPU oracle then checks a seeded SAMPLE of
-(batch, head) pairs / sequences / cache rows (the units are independent, and the full score tensors
-would be tens of GB), under the reference's tolerance rule (tests/test_flash_attn.py:648-650) with
+The whole problem runs through the public API; the CPU oracle then checks a SAMPLE of (batch, head)
+pairs / sequences / cache rows (the units are independent, and the full score tensors would be tens
+of GB): fixed corner units plus units drawn anew on every run (the draw's seed is printed, and
+FA_SAMPLE_SEED replays it), under the reference's tolerance rule (tests/test_flash_attn.py:648-650) with
 log-sum-exp within 1e-3 relative.  Size-independent properties (bit-repeatability, split-count
 invariance, appended cache rows) are checked on the whole output."""
 import math
+import os
+import random
 import sys
+import time
 
 import pytest
 import torch
@@ -20,6 +24,15 @@ DEV = "cuda"
 def _say(*a):
     print(*a, flush=True)
     sys.stdout.flush()
+
+
+def _drawn(n, *ranges):
+    """n index tuples drawn anew on every run, one index below each of `ranges`"""
+    seed = int(os.environ.get("FA_SAMPLE_SEED", time.time_ns() % (1 << 31)))
+    rng = random.Random(seed)
+    picks = [tuple(rng.randrange(r) for r in ranges) for _ in range(n)]
+    _say("   sample drawn with FA_SAMPLE_SEED=%d: %s" % (seed, picks))
+    return picks
 
 
 def _fa():
@@ -51,7 +64,7 @@ def test_config2_bf16_causal_8k():
     fa = _fa()
     out, lse, _ = fa.flash_attn_func(q, k, v, softmax_scale=1 / math.sqrt(128), causal=True, return_attn_probs=True)
     assert not torch.isnan(out).any() and torch.isfinite(lse).all()
-    _check_heads(out, lse, q, k, v, [(0, 0), (3, 31), (1, 17)], 1, causal=True, softmax_scale=1 / math.sqrt(128))
+    _check_heads(out, lse, q, k, v, [(0, 0), (3, 31), (1, 17)] + _drawn(2, b, h), 1, causal=True, softmax_scale=1 / math.sqrt(128))
     out2, lse2, _ = fa.flash_attn_func(q, k, v, softmax_scale=1 / math.sqrt(128), causal=True, return_attn_probs=True)
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
     # first row of every (batch, head) sees exactly one key: out = v[0], lse = scale * q0.k0
@@ -82,7 +95,7 @@ def test_config3_gqa_sliding_window_16k():
     v = torch.randn(b, s, hk, d, device=DEV, dtype=torch.bfloat16)
     out, lse, _ = _fa().flash_attn_func(q, k, v, causal=True, window_size=(4096, 0), return_attn_probs=True)
     assert not torch.isnan(out).any()
-    _check_heads(out, lse, q, k, v, [(0, 3), (1, 30)], h // hk, causal=True, window_size=(4096, 0))
+    _check_heads(out, lse, q, k, v, [(0, 3), (1, 30)] + _drawn(1, b, h), h // hk, causal=True, window_size=(4096, 0))
 
 
 @pytest.mark.parametrize("d", [128, 256])
@@ -100,15 +113,15 @@ def test_config4_varlen_64_sequences(d):
     assert out.shape == q.shape and lse.shape == (64, h, mx)
     assert not torch.isnan(out).any()
     order = torch.argsort(lens)
-    for i in (int(order[0]), int(order[31]), int(order[-1]), 7):     # shortest, median, longest, one more
+    units = [(int(order[j]), hh) for j in (0, 31, -1) for hh in (0, 11)] + [(7, 0), (7, 11)]   # shortest, median, longest, one more
+    for i, hh in units + _drawn(3, 64, h):
         a, e = int(cu[i]), int(cu[i + 1])
-        for hh in (0, 11):
-            qs, ks, vs = (t[a:e, hh:hh + 1][None].cpu() for t in (q, k, v))
-            o_ref, l_ref, o_pt = orc.attention_reference_pair(qs, ks, vs, causal=True)
-            ok, err, bound = orc.tolerance_ok(out[a:e, hh:hh + 1][None].cpu(), o_ref, o_pt, 2.0, 1e-5)
-            _say("   seq %d (len %d) head %d: err %.3e bound %.3e" % (i, e - a, hh, err, bound))
-            assert ok
-            assert orc.lse_ok(lse[i, hh:hh + 1, : e - a][None].cpu(), l_ref)[0]
+        qs, ks, vs = (t[a:e, hh:hh + 1][None].cpu() for t in (q, k, v))
+        o_ref, l_ref, o_pt = orc.attention_reference_pair(qs, ks, vs, causal=True)
+        ok, err, bound = orc.tolerance_ok(out[a:e, hh:hh + 1][None].cpu(), o_ref, o_pt, 2.0, 1e-5)
+        _say("   seq %d (len %d) head %d: err %.3e bound %.3e" % (i, e - a, hh, err, bound))
+        assert ok
+        assert orc.lse_ok(lse[i, hh:hh + 1, : e - a][None].cpu(), l_ref)[0]
 
 
 def test_config5_decode_kvcache_rotary():
@@ -125,7 +138,7 @@ def test_config5_decode_kvcache_rotary():
     lens = torch.randint(1024, cap, (b,), dtype=torch.int32)
     lens[0], lens[1] = 1024, cap - 1
     cos, sin = orc.rotary_table(cap, d, dtype=torch.bfloat16)
-    sample = [0, 1, 17, 63]
+    sample = sorted(set([0, 1, 17, 63] + [i for (i,) in _drawn(2, b)]))
     before_k = {i: kc[i, : int(lens[i]) + 2].cpu() for i in sample}
     before_v = {i: vc[i, : int(lens[i]) + 2].cpu() for i in sample}
     lens_d = lens.to(DEV)

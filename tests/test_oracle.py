@@ -260,6 +260,24 @@ def test_tolerance_rule_detects_errors():
     assert orc.lse_ok(lse * (1 + 5e-4), lse)[0] and not orc.lse_ok(lse * 1.01, lse)[0]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sq,sk,d,kw", [(64, 64, 32, dict(causal=True)), (128, 512, 64, dict()),
+                                        (96, 777, 128, dict(window_size=(100, 20))), (256, 2048, 128, dict(causal=True))])
+def test_tolerance_rule_is_bounded_above(dtype, sq, sk, d, kw):
+    """The allowance the rule hands to a kernel is `mult` x the error of the low-precision CPU run, so that
+    run must not be loose.  Every output is a convex combination of rows of v: rounding it to the 16-bit
+    type costs at most eps/2 * max|v|, and on these inputs the products and the softmax in 16-bit
+    arithmetic add less than as much again.  So the run stays within one eps * max|v| of the fp32 run
+    (measured: 0.03-0.5), and a kernel held to twice that is held to two units in the last place of the
+    largest output."""
+    eps = torch.finfo(dtype).eps
+    for seed in range(3):
+        q, k, v = (_randn(1, s, 2, d, dtype=dtype, seed=10 * seed + i) for i, s in enumerate((sq, sk, sk)))
+        ref, _, pt = orc.attention_reference_pair(q, k, v, **kw)
+        err = (pt.float() - ref.float()).abs().max().item()
+        assert 0 < err <= eps * v.float().abs().max().item(), (seed, err)
+
+
 # ---------------------------------------------------------------------------------------------
 # backward restatement
 # ---------------------------------------------------------------------------------------------
