@@ -28,8 +28,9 @@ template <bool DROPOUT, int DV = FA_D>
 static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
     // two workgroups (8 waves) per CU: the key tile is sized so that the kernel stays within 256 registers;
-    // three at head dim 64 (168 registers), where the vector work per matrix instruction doubles
-    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, (FA_D == 64 ? 3 : 2), DROPOUT, DV>(kp, stream)) return e;
+    // three at head dim 64 (168 registers), where the vector work per matrix instruction doubles -- without
+    // dropout: the mask words do not fit in 168 registers (19 spilled, 7-15 % slower than two workgroups)
+    if (int e = launch_bwd_dq<InstT, FA_D, FA_DQ_BN, (FA_D == 64 && !DROPOUT ? 3 : 2), DROPOUT, DV>(kp, stream)) return e;
     // Fewer key blocks than CUs (one long sequence on one or two kv heads, say): two workgroups per
     // key block, each accumulating half of the head dimension, fill the CUs at 3/4 of the work each.
     typedef BwdDkv3Cfg<InstT, FA_D, FA_BWD_BM, 1> C1;

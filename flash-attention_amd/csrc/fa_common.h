@@ -556,20 +556,23 @@ FA_DEV SeqInfo seq_info(const fa_fwd_params& p, int b) {
         s.q_off = (int64_t)b * p.q_batch_stride;
         s.o_off = (int64_t)b * p.o_batch_stride;
     }
+    // the four strides are read as values before the branch: a choice between the ADDRESSES of two fields
+    // makes the compiler keep a copy of them in per-lane scratch memory and index it
+    const int64_t k_row = p.k_row_stride, v_row = p.v_row_stride, k_batch = p.k_batch_stride, v_batch = p.v_batch_stride;
     if (p.cu_seqlens_k && p.is_seqlens_k_cumulative) {
         int r0 = p.cu_seqlens_k[b];
         s.sk_cache = p.cu_seqlens_k[b + 1] - r0;
         s.sk = s.sk_cache;
-        s.k_off = (int64_t)r0 * p.k_row_stride;
-        s.v_off = (int64_t)r0 * p.v_row_stride;
+        s.k_off = (int64_t)r0 * k_row;
+        s.v_off = (int64_t)r0 * v_row;
     } else {
         const int bk = p.cache_batch_idx ? p.cache_batch_idx[b] : b;
         // a cache length outside [0, capacity] is a caller error; clamped so that no key, rotary
         // table row or appended row beyond the cache is ever touched
         s.sk_cache = p.cu_seqlens_k ? min(max(p.cu_seqlens_k[b], 0), p.seqlen_k) : p.seqlen_k;
         s.sk = min(s.sk_cache + p.seqlen_knew, p.seqlen_k);
-        s.k_off = (int64_t)bk * p.k_batch_stride;
-        s.v_off = (int64_t)bk * p.v_batch_stride;
+        s.k_off = (int64_t)bk * k_batch;
+        s.v_off = (int64_t)bk * v_batch;
     }
     s.q_row0 = 0;
     return s;
