@@ -236,7 +236,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
                 for (int r = 0; r < 16; r++) {
                     const float pv = fast_exp2(s_acc[0][r] * sl2 - lse2);
                     float dpv = dp_acc[0][r];
-                    if constexpr (DROPOUT) dpv = (keep >> r) & 1u ? dpv * drop.rp : 0.f;   // gradient through the dropped P
+                    if constexpr (DROPOUT) dpv = drop_gate_bwd<D>(dpv * drop.rp, keep, r);   // gradient through the dropped P
                     s_acc[0][r] = pv * (dpv - dsum);
                 }
                 dsf[2 * nb] = pack_acc8<T>(s_acc[0], 0);
@@ -504,9 +504,9 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                     for (int e = 0; e < 4; e++) {
                         const int r = 4 * q4 + e;
                         const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
-                        const bool kept = !DROPOUT || ((keep >> r) & 1u);
-                        xo[r] = kept ? pv : -pv;               // sign bit = dropped
-                        s_acc[mb][r] = kept ? pv : 0.f;
+                        // sign bit = dropped (pv >= 0)
+                        xo[r] = DROPOUT ? __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv) | (~drop_word_bwd<D>(keep, r) & 0x80000000u)) : pv;
+                        s_acc[mb][r] = DROPOUT ? drop_gate_bwd<D>(pv, keep, r) : pv;
                     }
                 }
                 *reinterpret_cast<f16x8*>(xw + ((mb * 2) * 64 + lane) * 16) = pack_acc8<_Float16>(xo, 0);

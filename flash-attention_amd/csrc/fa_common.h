@@ -187,38 +187,77 @@ FA_DEV bool drop_keep(const Drop& d, int i, int j) {          // one element (an
     const uint32_t w = drop_hash(d, (uint32_t)i >> 1, (uint32_t)j >> 1);
     return ((w >> (8 * ((i & 1) * 2 + (j & 1)))) & 0xffu) < d.thresh;
 }
-// Bit r of the result = keep for accumulator register r of a 32 x 32 block whose lane owns ROW `row`
-// and whose registers walk keys kb0 + 8 (r >> 2) + 4 hh + (r & 3)   (kb0 a multiple of 32).
-FA_DEV uint32_t drop_keep16_row(const Drop& d, int row, int kb0, int hh) {
-    uint32_t bits = 0;
-    const uint32_t sh = (row & 1) * 16;
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const uint32_t j2 = (uint32_t)(kb0 + 8 * q + 4 * hh) >> 1;
-        const uint32_t wa = drop_hash(d, (uint32_t)row >> 1, j2) >> sh;
-        const uint32_t wb = drop_hash(d, (uint32_t)row >> 1, j2 + 1) >> sh;
-        bits |= (uint32_t)((wa & 0xffu) < d.thresh) << (4 * q);
-        bits |= (uint32_t)(((wa >> 8) & 0xffu) < d.thresh) << (4 * q + 1);
-        bits |= (uint32_t)((wb & 0xffu) < d.thresh) << (4 * q + 2);
-        bits |= (uint32_t)(((wb >> 8) & 0xffu) < d.thresh) << (4 * q + 3);
-    }
-    return bits;
+// The two kernels' geometries below give a lane one line of 2 x 2 blocks and its neighbour (lane ^ 1) the
+// other line of the SAME blocks, so the pair shares the hashes: each lane hashes half of the blocks, tests all
+// four bytes of every word it made, and hands the neighbour's flags over with one DPP move.  The four bytes of
+// a word are tested two at a time: byte + (256 - thresh) carries into bit 8 exactly when the byte is not
+// below thresh.  Both functions must be called by all 64 lanes together.
+FA_DEV uint32_t lane_xor1(uint32_t x) {    // x of lane ^ 1 (quad_perm [1, 0, 3, 2])
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xf, 0xf, true);
 }
-// Same for a block whose lane owns KEY `key` and whose registers walk rows rb0 + 8 (r >> 2) + 4 hh + (r & 3).
-FA_DEV uint32_t drop_keep16_key(const Drop& d, int key, int rb0, int hh) {
-    uint32_t bits = 0;
-    const uint32_t sh = (key & 1) * 8;
+// te: bit 8 / bit 24 set = byte 0 / byte 2 of w is dropped; to: the same for byte 1 / byte 3
+FA_DEV void drop_flags(const Drop& d, uint32_t w, uint32_t& te, uint32_t& to) {
+    const uint32_t add = (256u - d.thresh) * 0x00010001u;
+    te = ((w & 0x00ff00ffu) + add) & 0x01000100u;
+    to = (((w >> 8) & 0x00ff00ffu) + add) & 0x01000100u;
+}
+// Bit r of the result = keep for accumulator register r of a 32 x 32 block whose lane owns ROW `row`
+// and whose registers walk keys kb0 + 8 (r >> 2) + 4 hh + (r & 3)   (kb0 a multiple of 32).  Lanes l and
+// l ^ 1 must own rows 2 m and 2 m + 1 (rows follow the lane number from an even base) with the same kb0, hh.
+FA_DEV uint32_t drop_keep16_row(const Drop& d, int row, int kb0, int hh) {
+    const uint32_t odd = (uint32_t)row & 1u;          // this lane hashes the blocks of registers 8 odd .. 8 odd + 7
+    const uint32_t j2 = (uint32_t)(kb0 + 16 * (int)odd + 4 * hh) >> 1;
+    uint32_t acc = 0;      // bits 8..15: dropped flags of the even row for those 8 registers, bits 24..31: of the odd row
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const uint32_t i2 = (uint32_t)(rb0 + 8 * q + 4 * hh) >> 1;
-        const uint32_t wa = drop_hash(d, i2, (uint32_t)key >> 1) >> sh;
-        const uint32_t wb = drop_hash(d, i2 + 1, (uint32_t)key >> 1) >> sh;
-        bits |= (uint32_t)((wa & 0xffu) < d.thresh) << (4 * q);
-        bits |= (uint32_t)(((wa >> 16) & 0xffu) < d.thresh) << (4 * q + 1);
-        bits |= (uint32_t)((wb & 0xffu) < d.thresh) << (4 * q + 2);
-        bits |= (uint32_t)(((wb >> 16) & 0xffu) < d.thresh) << (4 * q + 3);
+    for (int k = 0; k < 4; k++) {
+        uint32_t te, to;
+        drop_flags(d, drop_hash(d, (uint32_t)row >> 1, j2 + 4 * (k >> 1) + (k & 1)), te, to);
+        acc |= (te | (to << 1)) << (2 * k);
     }
-    return bits;
+    const uint32_t sh = 8u + 16u * odd;
+    const uint32_t mine = (acc >> sh) & 0xffu, theirs = (lane_xor1(acc) >> sh) & 0xffu;
+    return ~((mine << (8u * odd)) | (theirs << (8u - 8u * odd))) & 0xffffu;
+}
+// Same for a block whose lane owns KEY `key` and whose registers walk rows rb0 + 8 (r >> 2) + 4 hh + (r & 3);
+// lanes l and l ^ 1 must own keys 2 m and 2 m + 1 with the same rb0, hh.
+FA_DEV uint32_t drop_keep16_key(const Drop& d, int key, int rb0, int hh) {
+    const uint32_t odd = (uint32_t)key & 1u;
+    const uint32_t i2 = (uint32_t)(rb0 + 16 * (int)odd + 4 * hh) >> 1;
+    // bits 8 + 2 k / 24 + 2 k: dropped flags of rows 2 k / 2 k + 1 of this lane's 8 registers, for the even / odd key
+    uint32_t acc_e = 0, acc_o = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        uint32_t te, to;
+        drop_flags(d, drop_hash(d, i2 + 4 * (k >> 1) + (k & 1), (uint32_t)key >> 1), te, to);
+        acc_e |= te << (2 * k);
+        acc_o |= to << (2 * k);
+    }
+    const uint32_t mine = odd ? acc_o : acc_e, theirs = lane_xor1(odd ? acc_e : acc_o);
+    auto in_order = [](uint32_t x) { return ((x >> 8) & 0x55u) | ((x >> 23) & 0xaau); };
+    return ~((in_order(mine) << (8u * odd)) | (in_order(theirs) << (8u - 8u * odd))) & 0xffffu;
+}
+
+// x where bit r of `keep` is set, +0 otherwise: the bit is spread over a word (one bit-field extract) and
+// masks x, one instruction fewer than test + select
+// (as an instruction: written with shifts or the bit-field intrinsic, the compiler turns it back into test +
+// select and holds one 64-bit lane mask per element in scalar registers)
+FA_DEV uint32_t drop_word(uint32_t keep, int r) {
+    uint32_t m;
+    asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(m) : "v"(keep), "n"(r));
+    return m;
+}
+FA_DEV float drop_gate(float x, uint32_t keep, int r) {
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & drop_word(keep, r));
+}
+// For the backward kernels: at head dims above 64 the same in plain C++, where the compiler's own choice is the
+// faster one (the asm statement stands outside the instruction groups their schedules are built from:
+// -7 % at head dim 128, +4 % at 64).
+template <int D> FA_DEV uint32_t drop_word_bwd(uint32_t keep, int r) {
+    if constexpr (D <= 64) return drop_word(keep, r);
+    else return (uint32_t)((int32_t)(keep << (31 - r)) >> 31);
+}
+template <int D> FA_DEV float drop_gate_bwd(float x, uint32_t keep, int r) {
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & drop_word_bwd<D>(keep, r));
 }
 
 // Rotary embedding of 8 consecutive elements [d0, d0+8) of one row, fp32 math.

@@ -241,7 +241,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                     for (int nb = 0; nb < C::NB; nb++) {
                         const uint32_t keep = drop_keep16_row(drop, r0 + l32, n0 + nb * 32, hh);
 #pragma unroll
-                        for (int r = 0; r < 16; r++) s_acc[rb][nb][r] = (keep >> r) & 1u ? s_acc[rb][nb][r] : 0.f;
+                        for (int r = 0; r < 16; r++) s_acc[rb][nb][r] = drop_gate(s_acc[rb][nb][r], keep, r);
                     }
                 }
                 if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {

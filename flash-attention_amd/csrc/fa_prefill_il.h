@@ -336,7 +336,7 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
                 suma += e0;
                 sumb += e1;
                 if constexpr (DROPOUT)
-                    pk[e] = pack2<T>((keep[nb] >> (r8 + 2 * e)) & 1u ? e0 : 0.f, (keep[nb] >> (r8 + 2 * e + 1)) & 1u ? e1 : 0.f);
+                    pk[e] = DROPOUT ? pack2<T>(drop_gate(e0, keep[nb], r8 + 2 * e), drop_gate(e1, keep[nb], r8 + 2 * e + 1)) : pack2<T>(e0, e1);
                 else
                     pk[e] = pack2<T>(e0, e1);
             }
@@ -494,8 +494,9 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
                         suma += e0;
                         sumb += e1;
                         if constexpr (DROPOUT)
-                            pk[pr] = pack2<T>((keep[(2 * pr) / 16] >> ((2 * pr) % 16)) & 1u ? e0 : 0.f,
-                                              (keep[(2 * pr + 1) / 16] >> ((2 * pr + 1) % 16)) & 1u ? e1 : 0.f);
+                            pk[pr] = DROPOUT ? pack2<T>(drop_gate(e0, keep[(2 * pr) / 16], (2 * pr) % 16),
+                                                        drop_gate(e1, keep[(2 * pr + 1) / 16], (2 * pr + 1) % 16))
+                                             : pack2<T>(e0, e1);
                         else
                             pk[pr] = pack2<T>(e0, e1);
                     }

@@ -311,7 +311,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
             for (int nb = 0; nb < C::NB; nb++) mask_acc16(s_acc[nb], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
         }
-        if constexpr (!DROPOUT) {
+        {
             // The tile is exponentiated against the reference max the row already has, and only the
             // tile's row sum is looked at afterwards: at most 2^14 means no probability above 2^14 (safe
             // in fp16 / bf16 and in the fp32 sums), so the reference stays and no row max is formed.
@@ -319,6 +319,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             // reference: -inf makes every exponent +inf or NaN) takes the rare branch, which forms the
             // exact row max from the untouched scores, moves the reference under the usual rule and
             // exponentiates again.
+            uint32_t keep[C::NB];
+#pragma unroll
+            for (int nb = 0; nb < C::NB; nb++) keep[nb] = DROPOUT ? drop_keep16_row(drop, row, tt * BN + nb * 32, hh) : 0xffffu;
             auto exp_tile = [&](float msc) -> float {
                 float suma = 0.f, sumb = 0.f;
 #pragma unroll
@@ -331,7 +334,10 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
                         const float e1 = fast_exp2(s_acc[nb][r8 + 2 * e + 1] * sl2 - msc);
                         suma += e0;
                         sumb += e1;
-                        pk[e] = pack2<T>(e0, e1);
+                        // the row sum is of the undropped probabilities; dropped entries leave the second
+                        // product only, and 1 / (1 - p) is applied once in the epilogue
+                        pk[e] = DROPOUT ? pack2<T>(drop_gate(e0, keep[nb], r8 + 2 * e), drop_gate(e1, keep[nb], r8 + 2 * e + 1))
+                                        : pack2<T>(e0, e1);
                     }
                     pf[t16] = __builtin_bit_cast(v8, pk);
                 }
@@ -363,57 +369,6 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
                     for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
             }
-            return;
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s_acc[nb][r]);
-        mx = xhalf_max(mx);
-        // lazy reference max: move it only when the tile max exceeds it by more than 2^8 (exp2 domain)
-        const bool move = (mx - m_run) * sl2 > 8.f;       // false for NaN (-inf - -inf)
-        if (__builtin_amdgcn_ballot_w64(move) != 0) {
-            const float m_new = move ? mx : m_run;
-            const float corr = move ? fast_exp2((m_run - m_new) * sl2) : 1.f;   // m_run = -inf -> 0
-            l_run *= corr;
-#pragma unroll
-            for (int db = 0; db < DBV; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o_acc[db][r] *= corr;
-            m_run = m_new;
-        }
-        const float msc = (m_run == -INFINITY) ? 0.f : m_run * sl2;
-        float suma = 0.f, sumb = 0.f;
-#pragma unroll
-        for (int nb = 0; nb < C::NB; nb++)
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float e0 = fast_exp2(s_acc[nb][r] * sl2 - msc);
-                const float e1 = fast_exp2(s_acc[nb][r + 1] * sl2 - msc);
-                s_acc[nb][r] = e0;
-                s_acc[nb][r + 1] = e1;
-                suma += e0;
-                sumb += e1;
-            }
-        l_run += suma + sumb;
-        if constexpr (DROPOUT) {
-            // the row sum is of the undropped probabilities; dropped entries leave the second product
-            // only, and 1 / (1 - p) is applied once in the epilogue
-#pragma unroll
-            for (int nb = 0; nb < C::NB; nb++) {
-                const uint32_t keep = drop_keep16_row(drop, row, tt * BN + nb * 32, hh);
-#pragma unroll
-                for (int r = 0; r < 16; r++) s_acc[nb][r] = (keep >> r) & 1u ? s_acc[nb][r] : 0.f;
-            }
-        }
-#pragma unroll
-        for (int t16 = 0; t16 < C::PT; t16++) {
-            const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
-            u32x4 pk;
-#pragma unroll
-            for (int e = 0; e < 4; e++) pk[e] = pack2<T>(s_acc[nb][r8 + 2 * e], s_acc[nb][r8 + 2 * e + 1]);
-            pf[t16] = __builtin_bit_cast(v8, pk);
         }
     };
 
