@@ -230,13 +230,13 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
                 product_rows<T, D, 1, C::KS, 4>(s_acc, kb + nb * 32 * C::ROWB, lo.r, qf);
                 product_rows<T, D, 1, C::KS, 4>(dp_acc, vb + nb * 32 * C::ROWB, lo.r, gf);
                 if (need_mask) mask_acc16(s_acc[0], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
-                uint32_t keep = 0xffffu;
-                if constexpr (DROPOUT) keep = drop_keep16_row(drop, row, n0 + nb * 32, hh);
+                uint32_t keep[8];
+                if constexpr (DROPOUT) drop_pairs_row(drop, row, n0 + nb * 32, hh, keep);
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const float pv = fast_exp2(s_acc[0][r] * sl2 - lse2);
                     float dpv = dp_acc[0][r];
-                    if constexpr (DROPOUT) dpv = drop_gate_bwd<D>(dpv * drop.rp, keep, r);   // gradient through the dropped P
+                    if constexpr (DROPOUT) dpv = drop_gate_half(dpv * drop.rp, keep[r >> 1], r & 1);   // gradient through the dropped P
                     s_acc[0][r] = pv * (dpv - dsum);
                 }
                 dsf[2 * nb] = pack_acc8<T>(s_acc[0], 0);
@@ -494,25 +494,30 @@ __global__ void __launch_bounds__(512, 1) bwd_dkv3_kernel(const BwdKParams kp) {
                     const int rel = key - ib - 4 * hh;
                     mask_acc16(s_acc[mb], 0, rel - rel_hi, rel - rel_lo);
                 }
-                uint32_t keep = 0xffffu;
-                if constexpr (DROPOUT) keep = drop_keep16_key(drop, key, ib, hh);
-                f32x16 xo;
+                uint32_t keep[8];
+                if constexpr (DROPOUT) drop_pairs_key(drop, key, ib, hh, keep);
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
                     const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + mb * 32 + 8 * q4 + 4 * hh);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int r = 4 * q4 + e;
-                        const float pv = fast_exp2(s_acc[mb][r] * sl2 - l4[e]);
-                        // sign bit = dropped (pv >= 0)
-                        xo[r] = DROPOUT ? __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, pv) | (~drop_word_bwd<D>(keep, r) & 0x80000000u)) : pv;
-                        s_acc[mb][r] = DROPOUT ? drop_gate_bwd<D>(pv, keep, r) : pv;
-                    }
+                    for (int e = 0; e < 4; e++) s_acc[mb][4 * q4 + e] = fast_exp2(s_acc[mb][4 * q4 + e] * sl2 - l4[e]);
                 }
-                *reinterpret_cast<f16x8*>(xw + ((mb * 2) * 64 + lane) * 16) = pack_acc8<_Float16>(xo, 0);
-                *reinterpret_cast<f16x8*>(xw + ((mb * 2 + 1) * 64 + lane) * 16) = pack_acc8<_Float16>(xo, 8);
-                pf[2 * mb] = pack_acc8<T>(s_acc[mb], 0);
-                pf[2 * mb + 1] = pack_acc8<T>(s_acc[mb], 8);
+                // hand-over copy in fp16 with the sign bit set where dropped (P >= 0), own copy with zeros there:
+                // both masked as packed pairs
+#pragma unroll
+                for (int h8 = 0; h8 < 2; h8++) {
+                    u32x4 xo = __builtin_bit_cast(u32x4, pack_acc8<_Float16>(s_acc[mb], 8 * h8));
+                    u32x4 pk = __builtin_bit_cast(u32x4, pack_acc8<T>(s_acc[mb], 8 * h8));
+                    if constexpr (DROPOUT) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            xo[e] |= ~keep[4 * h8 + e] & 0x80008000u;
+                            pk[e] &= keep[4 * h8 + e];
+                        }
+                    }
+                    *reinterpret_cast<u32x4*>(xw + ((mb * 2 + h8) * 64 + lane) * 16) = xo;
+                    pf[2 * mb + h8] = __builtin_bit_cast(v8, pk);
+                }
             }
             product_cols<T, D, C::PT, C::DB, 4>(acc, gb, lo.c, pf);
             }

@@ -187,77 +187,54 @@ FA_DEV bool drop_keep(const Drop& d, int i, int j) {          // one element (an
     const uint32_t w = drop_hash(d, (uint32_t)i >> 1, (uint32_t)j >> 1);
     return ((w >> (8 * ((i & 1) * 2 + (j & 1)))) & 0xffu) < d.thresh;
 }
-// The two kernels' geometries below give a lane one line of 2 x 2 blocks and its neighbour (lane ^ 1) the
-// other line of the SAME blocks, so the pair shares the hashes: each lane hashes half of the blocks, tests all
-// four bytes of every word it made, and hands the neighbour's flags over with one DPP move.  The four bytes of
-// a word are tested two at a time: byte + (256 - thresh) carries into bit 8 exactly when the byte is not
-// below thresh.  Both functions must be called by all 64 lanes together.
-FA_DEV uint32_t lane_xor1(uint32_t x) {    // x of lane ^ 1 (quad_perm [1, 0, 3, 2])
-    return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xf, 0xf, true);
+// Masks for the kernels, one 32-bit word per PAIR of accumulator registers (2 p, 2 p + 1) of a 32 x 32 block:
+// 0xffff in the half of a kept element, 0 in the half of a dropped one -- the form that masks a packed 16-bit
+// pair with one instruction.  Both register geometries give a lane one line of 2 x 2 blocks and its neighbour
+// (lane ^ 1) the other line of the SAME blocks, so the pair shares the hashes: each lane makes four, both take
+// the even lane's words for pairs 0..3 and the odd lane's for pairs 4..7 (DPP), pick their own two bytes of a
+// word into the two halves (byte permute) and compare both at once: byte - thresh is negative exactly when
+// the element is kept.  Must be called by all 64 lanes together; lanes l and l ^ 1 must own lines 2 m and
+// 2 m + 1 (rows or keys follow the lane number from an even base) with the same block origin and hh.
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+FA_DEV uint32_t drop_pair_mask(uint32_t w, uint32_t sel, uint32_t thresh2) {
+    const uint32_t x = __builtin_amdgcn_perm(w, w, sel);
+    const s16x2 t = __builtin_bit_cast(s16x2, x) - __builtin_bit_cast(s16x2, thresh2);
+    return __builtin_bit_cast(uint32_t, t >> 15);
 }
-// te: bit 8 / bit 24 set = byte 0 / byte 2 of w is dropped; to: the same for byte 1 / byte 3
-FA_DEV void drop_flags(const Drop& d, uint32_t w, uint32_t& te, uint32_t& to) {
-    const uint32_t add = (256u - d.thresh) * 0x00010001u;
-    te = ((w & 0x00ff00ffu) + add) & 0x01000100u;
-    to = (((w >> 8) & 0x00ff00ffu) + add) & 0x01000100u;
-}
-// Bit r of the result = keep for accumulator register r of a 32 x 32 block whose lane owns ROW `row`
-// and whose registers walk keys kb0 + 8 (r >> 2) + 4 hh + (r & 3)   (kb0 a multiple of 32).  Lanes l and
-// l ^ 1 must own rows 2 m and 2 m + 1 (rows follow the lane number from an even base) with the same kb0, hh.
-FA_DEV uint32_t drop_keep16_row(const Drop& d, int row, int kb0, int hh) {
-    const uint32_t odd = (uint32_t)row & 1u;          // this lane hashes the blocks of registers 8 odd .. 8 odd + 7
-    const uint32_t j2 = (uint32_t)(kb0 + 16 * (int)odd + 4 * hh) >> 1;
-    uint32_t acc = 0;      // bits 8..15: dropped flags of the even row for those 8 registers, bits 24..31: of the odd row
+FA_DEV void drop_pair_masks(const uint32_t (&w)[4], uint32_t sel, uint32_t thresh2, uint32_t (&m)[8]) {
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        uint32_t te, to;
-        drop_flags(d, drop_hash(d, (uint32_t)row >> 1, j2 + 4 * (k >> 1) + (k & 1)), te, to);
-        acc |= (te | (to << 1)) << (2 * k);
+        const uint32_t even = (uint32_t)__builtin_amdgcn_mov_dpp((int)w[k], 0xA0, 0xf, 0xf, true);   // quad_perm [0, 0, 2, 2]
+        const uint32_t odd = (uint32_t)__builtin_amdgcn_mov_dpp((int)w[k], 0xF5, 0xf, 0xf, true);    // quad_perm [1, 1, 3, 3]
+        m[k] = drop_pair_mask(even, sel, thresh2);
+        m[4 + k] = drop_pair_mask(odd, sel, thresh2);
     }
-    const uint32_t sh = 8u + 16u * odd;
-    const uint32_t mine = (acc >> sh) & 0xffu, theirs = (lane_xor1(acc) >> sh) & 0xffu;
-    return ~((mine << (8u * odd)) | (theirs << (8u - 8u * odd))) & 0xffffu;
 }
-// Same for a block whose lane owns KEY `key` and whose registers walk rows rb0 + 8 (r >> 2) + 4 hh + (r & 3);
-// lanes l and l ^ 1 must own keys 2 m and 2 m + 1 with the same rb0, hh.
-FA_DEV uint32_t drop_keep16_key(const Drop& d, int key, int rb0, int hh) {
+// lane owns ROW `row`, registers walk keys kb0 + 8 (r >> 2) + 4 hh + (r & 3)   (kb0 a multiple of 32)
+FA_DEV void drop_pairs_row(const Drop& d, int row, int kb0, int hh, uint32_t (&m)[8]) {
+    const uint32_t odd = (uint32_t)row & 1u;
+    const uint32_t j2 = (uint32_t)(kb0 + 16 * (int)odd + 4 * hh) >> 1;
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) w[k] = drop_hash(d, (uint32_t)row >> 1, j2 + 4 * (k >> 1) + (k & 1));
+    // bytes 2 odd (even key) and 2 odd + 1 (odd key) of a word; selector byte 0x0c gives zero
+    drop_pair_masks(w, 0x0c010c00u + odd * 0x00020002u, d.thresh * 0x00010001u, m);
+}
+// lane owns KEY `key`, registers walk rows rb0 + 8 (r >> 2) + 4 hh + (r & 3)   (rb0 a multiple of 32)
+FA_DEV void drop_pairs_key(const Drop& d, int key, int rb0, int hh, uint32_t (&m)[8]) {
     const uint32_t odd = (uint32_t)key & 1u;
     const uint32_t i2 = (uint32_t)(rb0 + 16 * (int)odd + 4 * hh) >> 1;
-    // bits 8 + 2 k / 24 + 2 k: dropped flags of rows 2 k / 2 k + 1 of this lane's 8 registers, for the even / odd key
-    uint32_t acc_e = 0, acc_o = 0;
+    uint32_t w[4];
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        uint32_t te, to;
-        drop_flags(d, drop_hash(d, i2 + 4 * (k >> 1) + (k & 1), (uint32_t)key >> 1), te, to);
-        acc_e |= te << (2 * k);
-        acc_o |= to << (2 * k);
-    }
-    const uint32_t mine = odd ? acc_o : acc_e, theirs = lane_xor1(odd ? acc_e : acc_o);
-    auto in_order = [](uint32_t x) { return ((x >> 8) & 0x55u) | ((x >> 23) & 0xaau); };
-    return ~((in_order(mine) << (8u * odd)) | (in_order(theirs) << (8u - 8u * odd))) & 0xffffu;
+    for (int k = 0; k < 4; k++) w[k] = drop_hash(d, i2 + 4 * (k >> 1) + (k & 1), (uint32_t)key >> 1);
+    // bytes odd (even row) and 2 + odd (odd row) of a word
+    drop_pair_masks(w, 0x0c020c00u + odd * 0x00010001u, d.thresh * 0x00010001u, m);
 }
 
-// x where bit r of `keep` is set, +0 otherwise: the bit is spread over a word (one bit-field extract) and
-// masks x, one instruction fewer than test + select
-// (as an instruction: written with shifts or the bit-field intrinsic, the compiler turns it back into test +
-// select and holds one 64-bit lane mask per element in scalar registers)
-FA_DEV uint32_t drop_word(uint32_t keep, int r) {
-    uint32_t m;
-    asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(m) : "v"(keep), "n"(r));
-    return m;
-}
-FA_DEV float drop_gate(float x, uint32_t keep, int r) {
-    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & drop_word(keep, r));
-}
-// For the backward kernels: at head dims above 64 the same in plain C++, where the compiler's own choice is the
-// faster one (the asm statement stands outside the instruction groups their schedules are built from:
-// -7 % at head dim 128, +4 % at 64).
-template <int D> FA_DEV uint32_t drop_word_bwd(uint32_t keep, int r) {
-    if constexpr (D <= 64) return drop_word(keep, r);
-    else return (uint32_t)((int32_t)(keep << (31 - r)) >> 31);
-}
-template <int D> FA_DEV float drop_gate_bwd(float x, uint32_t keep, int r) {
-    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & drop_word_bwd<D>(keep, r));
+// x where half `hi` of a pair mask is set, +0 otherwise (for values that are not packed yet)
+FA_DEV float drop_gate_half(float x, uint32_t pair, int hi) {
+    const uint32_t w = hi ? (uint32_t)((int32_t)pair >> 16) : (uint32_t)((int32_t)(pair << 16) >> 16);
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & w);
 }
 
 // Rotary embedding of 8 consecutive elements [d0, d0+8) of one row, fp32 math.

@@ -234,15 +234,12 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                     }
                 l_run[rb] = l_run[rb] * corr + sum;
                 m_run[rb] = m_new;
+                // the row sum above is of the undropped probabilities; dropped entries leave the
+                // second product only (masked after packing), and 1 / (1 - p) is applied once in the epilogue
+                uint32_t keep[C::NB][8];
                 if constexpr (DROPOUT) {
-                    // the row sum above is of the undropped probabilities; dropped entries leave the
-                    // second product only, and 1 / (1 - p) is applied once in the epilogue
 #pragma unroll
-                    for (int nb = 0; nb < C::NB; nb++) {
-                        const uint32_t keep = drop_keep16_row(drop, r0 + l32, n0 + nb * 32, hh);
-#pragma unroll
-                        for (int r = 0; r < 16; r++) s_acc[rb][nb][r] = drop_gate(s_acc[rb][nb][r], keep, r);
-                    }
+                    for (int nb = 0; nb < C::NB; nb++) drop_pairs_row(drop, r0 + l32, n0 + nb * 32, hh, keep[nb]);
                 }
                 if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
 #pragma unroll
@@ -255,8 +252,10 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                     const int nb = t16 >> 1, r8 = (t16 & 1) * 8;
                     u32x4 pk;
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
+                    for (int e = 0; e < 4; e++) {
                         pk[e] = pack2<T>(s_acc[rb][nb][r8 + 2 * e], s_acc[rb][nb][r8 + 2 * e + 1]);
+                        if constexpr (DROPOUT) pk[e] &= keep[nb][r8 / 2 + e];
+                    }
                     pf[rb][t16] = __builtin_bit_cast(v8, pk);
                 }
             }

@@ -309,9 +309,11 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
         }
     };
     auto probs = [&](int i, const f32x16 (&s)[C::NB], v8 (&pf)[C::PT], float& corr_out, bool& move_out, float sl2) __attribute__((always_inline)) {
-        uint32_t keep[C::NB];
+        uint32_t keep[C::NB][8];      // per pair of registers: 0xffff in the half of a kept element
+        if constexpr (DROPOUT) {
 #pragma unroll
-        for (int nb = 0; nb < C::NB; nb++) keep[nb] = DROPOUT ? drop_keep16_row(drop, row, tile_of(i) * C::BN + nb * 32, hh) : 0xffffu;
+            for (int nb = 0; nb < C::NB; nb++) drop_pairs_row(drop, row, tile_of(i) * C::BN + nb * 32, hh, keep[nb]);
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int nb = 0; nb < C::NB; nb++)
@@ -335,10 +337,8 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
                 const float e1 = fast_exp2(s[nb][r8 + 2 * e + 1] * sl2 - msc);
                 suma += e0;
                 sumb += e1;
-                if constexpr (DROPOUT)
-                    pk[e] = DROPOUT ? pack2<T>(drop_gate(e0, keep[nb], r8 + 2 * e), drop_gate(e1, keep[nb], r8 + 2 * e + 1)) : pack2<T>(e0, e1);
-                else
-                    pk[e] = pack2<T>(e0, e1);
+                pk[e] = pack2<T>(e0, e1);
+                if constexpr (DROPOUT) pk[e] &= keep[nb][r8 / 2 + e];
             }
             pf[t16] = __builtin_bit_cast(v8, pk);
         }
@@ -451,9 +451,11 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
         float mx = -INFINITY, msc = 0.f, corr = 1.f, suma = 0.f, sumb = 0.f;
         bool move = false;
         uint32_t pk[NP];
-        uint32_t keep[C::NB];
+        uint32_t keep[C::NB][8];      // per pair of registers: 0xffff in the half of a kept element
+        if constexpr (DROPOUT) {
 #pragma unroll
-        for (int nb = 0; nb < C::NB; nb++) keep[nb] = DROPOUT ? drop_keep16_row(drop, row, tile_of(i) * C::BN + nb * 32, hh) : 0xffffu;
+            for (int nb = 0; nb < C::NB; nb++) drop_pairs_row(drop, row, tile_of(i) * C::BN + nb * 32, hh, keep[nb]);
+        }
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             // ---- matrix instruction f and the read for f + LA
@@ -493,12 +495,8 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
                         const float e1 = fast_exp2(s_cur[(2 * pr + 1) / 16][(2 * pr + 1) % 16] * sc - msc);
                         suma += e0;
                         sumb += e1;
-                        if constexpr (DROPOUT)
-                            pk[pr] = DROPOUT ? pack2<T>(drop_gate(e0, keep[(2 * pr) / 16], (2 * pr) % 16),
-                                                        drop_gate(e1, keep[(2 * pr + 1) / 16], (2 * pr + 1) % 16))
-                                             : pack2<T>(e0, e1);
-                        else
-                            pk[pr] = pack2<T>(e0, e1);
+                        pk[pr] = pack2<T>(e0, e1);
+                        if constexpr (DROPOUT) pk[pr] &= keep[pr / 8][pr % 8];
                     }
                 }
             }

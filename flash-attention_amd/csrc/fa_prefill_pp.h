@@ -319,9 +319,11 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             // reference: -inf makes every exponent +inf or NaN) takes the rare branch, which forms the
             // exact row max from the untouched scores, moves the reference under the usual rule and
             // exponentiates again.
-            uint32_t keep[C::NB];
+            uint32_t keep[C::NB][8];
+            if constexpr (DROPOUT) {
 #pragma unroll
-            for (int nb = 0; nb < C::NB; nb++) keep[nb] = DROPOUT ? drop_keep16_row(drop, row, tt * BN + nb * 32, hh) : 0xffffu;
+                for (int nb = 0; nb < C::NB; nb++) drop_pairs_row(drop, row, tt * BN + nb * 32, hh, keep[nb]);
+            }
             auto exp_tile = [&](float msc) -> float {
                 float suma = 0.f, sumb = 0.f;
 #pragma unroll
@@ -336,8 +338,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
                         sumb += e1;
                         // the row sum is of the undropped probabilities; dropped entries leave the second
                         // product only, and 1 / (1 - p) is applied once in the epilogue
-                        pk[e] = DROPOUT ? pack2<T>(drop_gate(e0, keep[nb], r8 + 2 * e), drop_gate(e1, keep[nb], r8 + 2 * e + 1))
-                                        : pack2<T>(e0, e1);
+                        pk[e] = pack2<T>(e0, e1);
+                        if constexpr (DROPOUT) pk[e] &= keep[nb][r8 / 2 + e];
                     }
                     pf[t16] = __builtin_bit_cast(v8, pk);
                 }
