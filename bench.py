@@ -174,7 +174,9 @@ def bench_rotary(steps, warmup):
         "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "gb_per_s": gbs,
         "workload": "apply_rotary_emb bf16 (8, 8192, 32, 128) rotary_dim 128 in place",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                     "traffic": None, "kernel": "fa::rotary_kernel<bf16,bf16,u32>", "bytes_per_launch": algo_bytes},
+                     "traffic": _traffic("rotary_bf16_8x8192x32x128_inplace"),
+                     "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
+                     "kernel": "fa::rotary_kernel<bf16,bf16,u32,stream>", "bytes_per_launch": algo_bytes},
     }
 
 

@@ -180,6 +180,74 @@ def test_rotary_emb_varlen_func(inplace, interleaved, fraction, offsets_kind, dt
     _close(pad_input(leaf.grad, indices, b, s), gwant, "grad")
 
 
+@pytest.mark.parametrize("varlen", [False, True])
+@pytest.mark.parametrize("inplace", [False, True])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("h,d,rd", [(16, 128, 128), (32, 128, 64), (40, 64, 64), (24, 256, 96), (128, 32, 32)])
+def test_rotary_many_heads(h, d, rd, interleaved, inplace, varlen):
+    """With 128 or more 16-byte work items per token the kernel hands whole tokens to workgroups (one index
+    division per item instead of four); same results required, dense and packed, with per-sequence offsets
+    and positions that run past the table."""
+    from flash_attn.layers.rotary import apply_rotary_emb
+    _say("rotary many heads", h, d, rd, interleaved, inplace, varlen)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(h + d)
+    lens = [5, 1, 77, 130] if varlen else [61, 61, 61]
+    b, mx = len(lens), max(lens)
+    cos, sin = _table(mx + 20, rd, dtype, 3)
+    offsets = torch.tensor([0, 19, 3, 40][:b], dtype=torch.int32)       # the last packed sequence runs past the table
+    if varlen:
+        cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+        x_cpu = torch.randn(int(cu[-1]), h, d, generator=g).to(dtype)
+        x = x_cpu.to(DEV)
+        out = apply_rotary_emb(x, cos.to(DEV), sin.to(DEV), seqlen_offsets=offsets.to(DEV), cu_seqlens=cu.to(DEV),
+                               max_seqlen=mx, interleaved=interleaved, inplace=inplace)
+        pieces = [(x_cpu[int(cu[i]):int(cu[i + 1])][None], int(offsets[i]), lens[i]) for i in range(b)]
+    else:
+        x_cpu = torch.randn(b, mx, h, d, generator=g).to(dtype)
+        x = x_cpu.to(DEV)
+        out = apply_rotary_emb(x, cos.to(DEV), sin.to(DEV), seqlen_offsets=offsets.to(DEV), interleaved=interleaved,
+                               inplace=inplace)
+        pieces = [(x_cpu[i:i + 1], int(offsets[i]), mx) for i in range(b)]
+    if not inplace:
+        assert torch.equal(x.cpu(), x_cpu)
+    got = out.cpu()
+    row = 0
+    for i, (xi, off, n) in enumerate(pieces):
+        pos = (off + torch.arange(n))[None]
+        inside = pos[0] < cos.shape[0]
+        want = xi.clone()
+        if inside.any():
+            want[:, inside] = orc.rotary_apply(xi[:, inside], cos, sin, pos[:, inside], interleaved)
+        gi = got[row:row + n][None] if varlen else got[i:i + 1]
+        _close(gi, want, "sequence %d" % i)
+        row += n
+
+
+@pytest.mark.parametrize("interleaved,inplace", [(False, True), (True, False)])
+def test_rotary_half_gigabyte_tensor(interleaved, inplace):
+    """From 384 MiB on the kernel moves x and out with non-temporal accesses (another instantiation): the
+    benchmark shape (8, 8192, 32, 128), checked on sampled (batch, head) slices, and everything else of an
+    out-of-place result must be finite."""
+    from flash_attn.layers.rotary import apply_rotary_emb
+    _say("rotary 0.5 GB", interleaved, inplace)
+    b, s, h, d = 8, 8192, 32, 128
+    torch.manual_seed(5)
+    x = torch.randn(b, s, h, d, device=DEV, dtype=torch.bfloat16)
+    cos, sin = _table(s + 7, d, torch.bfloat16, 9)
+    sample = [(0, 0), (7, 31), (3, 17)]
+    before = {bh: x[bh[0], :, bh[1]].cpu() for bh in sample}
+    out = apply_rotary_emb(x, cos.to(DEV), sin.to(DEV), seqlen_offsets=7, interleaved=interleaved, inplace=inplace)
+    assert (out.data_ptr() == x.data_ptr()) == inplace
+    assert torch.isfinite(out).all()
+    pos = _positions(7, 1, s)
+    for (bi, hi) in sample:
+        want = orc.rotary_apply(before[(bi, hi)][None, :, None], cos, sin, pos, interleaved)
+        _close(out[bi, :, hi][None, :, None], want, "batch %d head %d" % (bi, hi))
+        if not inplace:
+            assert torch.equal(x[bi, :, hi].cpu(), before[(bi, hi)])
+
+
 @pytest.mark.parametrize("d,rd", [(64, 16), (96, 48), (256, 256), (40, 32)])
 @pytest.mark.parametrize("interleaved", [False, True])
 def test_rotary_fp32_tables_and_other_head_dims(d, rd, interleaved):
