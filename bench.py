@@ -304,7 +304,7 @@ def bench_decode(steps, warmup):
         "workload": "flash_attn_with_kvcache bf16 b64 cache(64,32768,8,128) hq64 append1+rotary128 causal",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": gbs / PEAK_HBM_GBS, "traffic": _traffic("decode_bf16_d128_b64_32k"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                     "kernel": "fa::decode_persistent_kernel<bf16,128,append> (step = that kernel, which also appends the new rows, + fa::combine_kernel)", "bytes_per_launch": algo_bytes},
+                     "kernel": "fa::decode_persistent_kernel<bf16,128,append,stream> (step = that kernel, which also appends the new rows, + fa::combine_kernel)", "bytes_per_launch": algo_bytes},
     }
 
 

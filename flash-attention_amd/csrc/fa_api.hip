@@ -165,6 +165,8 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = kp.dec_compact = 0;
     kp.work_counter = q.work_counter;
     kp.work_items = nullptr;
+    // K + V, 16-bit elements; seqlen_k is the cache capacity (or the longest packed sequence): an upper bound
+    kp.stream_kv = (int64_t)4 * q.b * q.seqlen_k * q.h_k * q.d >= kStreamKvBytes;
 }
 
 static int run_attention(KParams& kp, hipStream_t stream) {

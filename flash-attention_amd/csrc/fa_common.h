@@ -58,12 +58,16 @@ struct KParams {
     // dec_compact: the tickets cover only the slots that hold keys (the kernel counts them per batch entry
     // from the lengths); the merge then derives which slots were written from the lengths as well
     int32_t dec_persistent, dec_sa, dec_sb, dec_sub, dec_append, dec_compact;
+    // K and V together hold kStreamKvBytes or more (several times what the 256 MB memory-side cache keeps): the decode
+    // kernels, which read every row once, fetch them with non-temporal loads
+    int32_t stream_kv;
     int32_t* work_counter;
     // Packed batches: work list built on the device from cu_seqlens_q just before the launch (work_list_kernel,
     // fa_aux.hip), or NULL.  8 item counts, then for XCD x a list of (gridDim.x / 8) slots of two words:
     // batch index, (q head << 16) | row block.
     const int32_t* work_items;
 };
+constexpr int64_t kStreamKvBytes = (int64_t)1 << 30;
 constexpr int kDecCompactMaxBatch = 1024;    // batch entries whose slot counts the persistent decode kernel scans in LDS
 constexpr int kWorkListHeaderWords = 8;
 constexpr int kWorkListMaxBatch = 2048;      // sequences the list builder ranks (quadratic, in LDS)

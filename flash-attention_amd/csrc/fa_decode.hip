@@ -48,7 +48,12 @@ enum ItemMode { kChunk = 0, kMacro = 1, kSub = 2 };
 // as the final output (SPLIT = false) or as partial `slot` (SPLIT = true).
 // APPEND: rows [cache length, cache length + seqlen_knew) are not in the cache yet; the item whose key range
 // holds them writes them first.  Every key belongs to exactly one item, so each row has one writer.
-template <typename T, int D, bool SPLIT, bool APPEND = false>
+// STREAM: K and V rows are fetched with non-temporal loads.  Every row is read once, so nothing is gained by
+// keeping it in the caches, and past the size the memory-side cache holds the hint is worth 8-11 % (4.5 GB of
+// K/V: 0.747 -> 0.824 of 8 TB/s); caches of a few hundred MB that are read again step after step are up to 7 %
+// faster without it.  (A template parameter and not a run-time branch: the compiler merges the loads of the
+// two branches and drops the hint.)
+template <typename T, int D, bool SPLIT, bool APPEND = false, bool STREAM = false>
 FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b, const int slot,
                         const int mode, const int idx) {
     typedef DecodeCfg<T, D> C;
@@ -123,8 +128,15 @@ FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b
             const int f = lane + i * 64;
             const int row = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
             const int n = min(n0 + row, w_hi - 1);
-            kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
-            vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
+            const T* kp_ = kg + (int64_t)n * p.k_row_stride + c * 8;
+            const T* vp_ = vg + (int64_t)n * p.v_row_stride + c * 8;
+            if constexpr (STREAM) {
+                kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp_));
+                vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vp_));
+            } else {
+                kr[i] = ld_global16(kp_);
+                vr[i] = ld_global16(vp_);
+            }
         }
     };
     auto store_step = [&](int n0) {
@@ -347,12 +359,12 @@ FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b
     }
 }
 
-template <typename T, int D, bool SPLIT>
+template <typename T, int D, bool SPLIT, bool STREAM>
 __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     // kv heads vary fastest over the grid: the h_k workgroups that share the rows of one
     // (batch, chunk) of a (b, s, h_k, d) cache run together and consume whole cache rows.
-    decode_item<T, D, SPLIT>(kp, smem, blockIdx.x, blockIdx.z, blockIdx.y, kChunk, blockIdx.y);
+    decode_item<T, D, SPLIT, false, STREAM>(kp, smem, blockIdx.x, blockIdx.z, blockIdx.y, kChunk, blockIdx.y);
 }
 
 // Persistent form: a fixed number of resident workgroups draw items from a ticket counter, in the
@@ -368,7 +380,7 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 // L2, every stream completes in the remainder pass at the very end of the launch, and 512 latency-bound
 // merges there cost 2-3 x the stand-alone merge kernel; cache write-back / invalidation fences at device scope
 // around every item instead cost three times the whole kernel).
-template <typename T, int D, bool APPEND>
+template <typename T, int D, bool APPEND, bool STREAM>
 __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int s_ticket;
@@ -437,7 +449,7 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kern
             const int per_b = macro ? kp.dec_sa : kp.dec_sb;
             hk = t % p.h_k; idx = (t / p.h_k) % per_b; b = t / (p.h_k * per_b);
         }
-        decode_item<T, D, true, APPEND>(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
+        decode_item<T, D, true, APPEND, STREAM>(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
     }
     if (threadIdx.x == 0) {
         const int gone = __hip_atomic_fetch_add(kp.work_counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -448,41 +460,36 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kern
     }
 }
 
-template <typename T, int D>
-static int launch_decode_t(const KParams& kp, hipStream_t stream) {
+// (the kernel is a template argument, not a function argument: the once-per-device flag inside
+// FA_ALLOW_DYNAMIC_LDS is then one per kernel)
+template <auto KERN>
+static int launch_decode_kernel(dim3 grid, int smem, const KParams& kp, hipStream_t stream) {
+    const hipError_t e = FA_ALLOW_DYNAMIC_LDS(KERN, smem);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(KERN, grid, dim3(256), smem, stream, kp);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int D, bool STREAM>
+static int launch_decode_ts(const KParams& kp, hipStream_t stream) {
     typedef DecodeCfg<T, D> C;
-    const bool split = kp.num_splits > 1;
-    hipError_t e;
+    static_assert(C::kThreads == 256, "launch_decode_kernel launches 256 lanes");
     if (kp.dec_persistent) {
         const int total = kp.p.b * (kp.dec_sa + kp.dec_sb) * kp.p.h_k;
         const int resident = 256 * (D > 128 ? 1 : 2);          // workgroups the 256 CUs hold at once
-        dim3 grid(total < resident ? total : resident), block(C::kThreads);
-        if (kp.dec_append) {
-            auto kern = decode_persistent_kernel<T, D, true>;
-            e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
-            if (e != hipSuccess) return (int)e;
-            hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-        } else {
-            auto kern = decode_persistent_kernel<T, D, false>;
-            e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
-            if (e != hipSuccess) return (int)e;
-            hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-        }
-        return (int)hipGetLastError();
+        const dim3 grid(total < resident ? total : resident);
+        if (kp.dec_append) return launch_decode_kernel<decode_persistent_kernel<T, D, true, STREAM>>(grid, C::SMEM, kp, stream);
+        return launch_decode_kernel<decode_persistent_kernel<T, D, false, STREAM>>(grid, C::SMEM, kp, stream);
     }
-    dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b), block(C::kThreads);
-    if (split) {
-        auto kern = decode_kernel<T, D, true>;
-        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-    } else {
-        auto kern = decode_kernel<T, D, false>;
-        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-    }
-    return (int)hipGetLastError();
+    const bool split = kp.num_splits > 1;
+    const dim3 grid(kp.p.h_k, split ? kp.num_splits : 1, kp.p.b);
+    if (split) return launch_decode_kernel<decode_kernel<T, D, true, STREAM>>(grid, C::SMEM, kp, stream);
+    return launch_decode_kernel<decode_kernel<T, D, false, STREAM>>(grid, C::SMEM, kp, stream);
+}
+
+template <typename T, int D>
+static int launch_decode_t(const KParams& kp, hipStream_t stream) {
+    return kp.stream_kv ? launch_decode_ts<T, D, true>(kp, stream) : launch_decode_ts<T, D, false>(kp, stream);
 }
 
 int launch_decode(const KParams& kp, hipStream_t stream) {
