@@ -113,7 +113,8 @@ static SplitPlan plan(const fa_fwd_params& p, bool allow_split) {
                 int64_t len = rup(std::max<int64_t>(minlen, (int64_t)sk * streams / FA_DEC_SLOTS), 128);
                 if (counters_ok(p)) {
                     const int64_t lp = rup(std::max<int64_t>(256, (int64_t)sk * streams / FA_DEC_SLOTS_P), 128);
-                    if (lp >= 1024) len = lp;
+                    // (at least 2048 keys once persistent: batch 4 x 128k keys x 8 kv heads +9 % over 1024-key chunks)
+                    if (lp >= 1024) len = std::max<int64_t>(lp, 2048);
                 }
                 splits = (int)((sk + len - 1) / len);
             } else {
