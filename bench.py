@@ -157,6 +157,31 @@ def bench_mfma_peak(steps, warmup):
     return res
 
 
+def bench_hbm_peak(steps, warmup):
+    """What a kernel that only reads sustains from HBM (fa_hbm_read_peak in the library) over as many bytes as
+    the decode step moves, with ordinary and with non-temporal loads."""
+    import ctypes
+    import torch
+    from flash_attn import _native as nat
+    lib = nat.lib
+    lib.fa_hbm_read_peak.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]
+    lib.fa_hbm_read_peak.restype = ctypes.c_int
+    nbytes = 4544733184 // 16 * 16
+    src = torch.empty(nbytes // 2, dtype=torch.bfloat16, device="cuda").normal_()
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {"kernel": "fa::hbm_read_peak_kernel (16-byte loads, 8 in flight per lane, a contiguous share per workgroup, nothing written)", "bytes_per_launch": nbytes}
+    for name, nt in (("nontemporal", 1), ("ordinary", 0)):
+        def fn():
+            rc = lib.fa_hbm_read_peak(src.data_ptr(), nbytes, nt, sink.data_ptr(), stream)
+            if rc != 0:
+                raise RuntimeError("fa_hbm_read_peak failed: %d" % rc)
+        tm = time_steps(fn, max(3, steps // 3), max(2, warmup // 3))
+        gbs = nbytes / (tm[0] * 1e-3) / 1e9
+        res[name] = {"ms": tm[0], "ms_min": tm.ms_min, "gb_per_s": gbs, "frac_of_published_peak": gbs / PEAK_HBM_GBS}
+    return res
+
+
 def bench_rotary(steps, warmup):
     import torch
     from flash_attn.layers.rotary import apply_rotary
@@ -341,7 +366,7 @@ def main():
     ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default=None,
-                    choices=["prefill", "mfma_peak", "decode", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
+                    choices=["prefill", "mfma_peak", "hbm_peak", "decode", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
                     help="run one leg alone and print its record (for profiler runs: the trace then holds that leg's kernels only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
@@ -365,7 +390,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.only:
-        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "decode": bench_decode, "rotary": bench_rotary,
+        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "decode": bench_decode, "rotary": bench_rotary,
                "backward": bench_backward, "fwd_bwd": bench_fwd_bwd, "varlen": bench_varlen, "gqa_window": bench_gqa_window,
                "head_dims": bench_head_dims}[a.only]
         print(json.dumps({"only": a.only, "steps": a.steps, "warmup": a.warmup, a.only: leg(a.steps, a.warmup)}))
@@ -387,7 +412,11 @@ def main():
     }
     if not a.no_decode:
         dec = bench_decode(a.steps, a.warmup)
+        hbm = bench_hbm_peak(a.steps, a.warmup)
+        dec["roofline"]["measured_peak"] = hbm["nontemporal"]["gb_per_s"]
+        dec["roofline"]["frac_of_measured_peak"] = dec["gb_per_s"] / hbm["nontemporal"]["gb_per_s"]
         out["decode"] = dec
+        out["hbm_peak"] = hbm
     if not a.no_backward:
         out["rotary"] = bench_rotary(a.steps, a.warmup)
         out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))

@@ -293,6 +293,14 @@ int32_t fa_sizeof_bwd_params(void);
  */
 int fa_mfma_peak(float *sink, int32_t iters, int32_t random_operands, int64_t *flops, void *hip_stream);
 
+/*
+ * Memory microbenchmark (measurement aid; no counterpart in the reference): launches a kernel that reads
+ * `bytes` (a multiple of 16, at a 16-byte aligned device address) once, with non-temporal loads
+ * (nontemporal != 0) or ordinary ones, and writes nothing.  The caller times the launch on `hip_stream`.
+ * `sink` is 4 bytes of device memory (never written in practice).
+ */
+int fa_hbm_read_peak(const void *src, int64_t bytes, int32_t nontemporal, void *sink, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif
