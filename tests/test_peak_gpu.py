@@ -1,0 +1,49 @@
+"""The two measurement kernels of the library (fa_mfma_peak, fa_hbm_read_peak) launch, finish and report what
+they did; sizes are small, the rates are bench.py's business."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _lib():
+    from flash_attn import _native as nat
+    lib = nat.lib
+    lib.fa_hbm_read_peak.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p]
+    lib.fa_hbm_read_peak.restype = ctypes.c_int
+    lib.fa_mfma_peak.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p]
+    lib.fa_mfma_peak.restype = ctypes.c_int
+    return lib
+
+
+@pytest.mark.parametrize("nbytes", [16, 4096 * 16 + 16, 64 << 20, (64 << 20) + 16 * 12345])
+@pytest.mark.parametrize("nontemporal", [0, 1])
+def test_hbm_read_peak_reads_any_multiple_of_16_bytes(nbytes, nontemporal):
+    print("hbm read peak", nbytes, nontemporal, flush=True)
+    lib = _lib()
+    src = torch.full((nbytes,), 7, dtype=torch.uint8, device=DEV)
+    guard = torch.full((4096,), 9, dtype=torch.uint8, device=DEV)
+    sink = torch.zeros(1, dtype=torch.int32, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.fa_hbm_read_peak(src.data_ptr(), nbytes, nontemporal, sink.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0 and bool((src == 7).all()) and bool((guard == 9).all())     # nothing written
+    # argument errors: no launch
+    assert lib.fa_hbm_read_peak(None, nbytes, nontemporal, sink.data_ptr(), stream) != 0
+    assert lib.fa_hbm_read_peak(src.data_ptr() + 8, 16, nontemporal, sink.data_ptr(), stream) != 0
+    assert lib.fa_hbm_read_peak(src.data_ptr(), 8, nontemporal, sink.data_ptr(), stream) != 0
+
+
+@pytest.mark.parametrize("random_operands", [0, 1])
+def test_mfma_peak_counts_its_operations(random_operands):
+    print("mfma peak", random_operands, flush=True)
+    lib = _lib()
+    sink = torch.zeros(1, dtype=torch.float32, device=DEV)
+    flops = ctypes.c_int64(0)
+    assert lib.fa_mfma_peak(sink.data_ptr(), 10, random_operands, ctypes.byref(flops), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert flops.value == 1024 * 4 * 10 * 16 * 2 * 32 * 32 * 16 and float(sink.item()) == 0.0
+    assert lib.fa_mfma_peak(sink.data_ptr(), 0, random_operands, ctypes.byref(flops), None) != 0
