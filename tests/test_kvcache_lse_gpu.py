@@ -55,7 +55,7 @@ def _run(q, kc, vc, lens, kn=None, vn=None, cos=None, sin=None, causal=False, wi
 @pytest.mark.parametrize("with_new", [False, True])
 def test_lse_persistent_decode_and_merge(with_new):
     """One decode step over caches large enough for the ticket-scheduled kernel (it takes over from
-    about 4 million cached key rows per launch: 8 x 32768 x 16 here, chunks of 1024 keys): sequences
+    about 4 million cached key rows per launch: 8 x 32768 x 16 here, chunks of 2048 keys): sequences
     with many complete chunks plus a ragged remainder, one chunk plus a few keys, less than one chunk,
     and an empty cache.  Every batch entry is checked against the oracle on its own slice."""
     _say("kvcache_lse persistent", with_new)
@@ -65,7 +65,7 @@ def test_lse_persistent_decode_and_merge(with_new):
     kc = torch.randn(b, cap, h, d, device=DEV, dtype=dtype)
     vc = torch.randn(b, cap, h, d, device=DEV, dtype=dtype)
     q = torch.randn(b, 1, h, d, device=DEV, dtype=dtype)
-    lens = torch.tensor([cap - 1, 1100, 3000, 5, 0, 20000, 1024, 2047], dtype=torch.int32)
+    lens = torch.tensor([cap - 1, 1100, 3000, 5, 0, 20000, 2048, 2051], dtype=torch.int32)
     kn = vn = cos = sin = None
     if with_new:
         kn = torch.randn(b, 1, h, d, device=DEV, dtype=dtype)
@@ -84,7 +84,7 @@ def test_lse_persistent_decode_and_merge(with_new):
     import ctypes
     n = ctypes.c_int32(0)
     assert nat.lib.fa_plan_splits(ctypes.byref(p), 2, ctypes.byref(n)) == 0
-    assert n.value == cap // 1024 + 2, n.value      # 32 complete-chunk slots + 2 remainder slots of 512 keys
+    assert n.value == cap // 2048 + 4, n.value      # 16 complete-chunk slots + 4 remainder slots of 512 keys
     dev = lambda t: None if t is None else t.to(DEV)
     out, lse = nat.fwd_kvcache(q, kc, vc, kn, vn, lens.to(DEV), dev(cos), dev(sin), None, None, d ** -0.5, True, -1, -1,
                                True, 0)
