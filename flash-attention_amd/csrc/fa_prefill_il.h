@@ -33,7 +33,9 @@ namespace fa {
 #define FA_IL_LA 4
 #endif
 
-// One query-row group of 32 rows per wave, the whole head dimension in that wave (d <= 128).
+// One query-row group of 32 rows per wave, the whole head dimension in that wave.  Up to head dim 128 two
+// (three at 64) workgroups share a CU; at head dim 256 O (128 accumulator registers) and the Q fragments (64)
+// leave room for one wave per SIMD only, which then has all 512 registers and 160 KB of LDS to itself.
 // DV_: head dims the products run over (a multiple of 32, d <= DV_ <= D_); tiles keep the LDS layout of the
 // bucket D_ (head dim 96 runs on the 128 bucket with 6 of 8 k-steps and 3 of 4 output column blocks).
 template <typename T, int D_, int BN_, int DV_ = D_>
@@ -56,12 +58,14 @@ struct ILCfg {
     static constexpr int ROWS_PER_PASS = kThreads / CPR;
     static constexpr int PASSB = kThreads * 16;             // LDS bytes filled by one pass of the workgroup
     static constexpr int XCH = 0;
-    static constexpr int SMEM = 2 * NS * TILE;              // K ring, then V ring
+    static constexpr int OUT_LANES = DH / 8 <= 8 ? 8 : DH / 8 <= 16 ? 16 : 32;      // lanes per output row in the epilogue
+    static constexpr int STAGE = kWaves * 32 * (OUT_LANES * 16 + 16);              // output staging of the epilogue
+    static constexpr int SMEM = 2 * NS * TILE > STAGE ? 2 * NS * TILE : STAGE;      // K ring, then V ring
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
-// Head dim 256: O (128 accumulator registers for 32 rows) plus Q fragments (64) do not leave room
-// for two waves per SIMD, so two waves share each group of 32 query rows and split the head
+// Head dim 256 with two waves per SIMD (the form that runs with dropout, whose mask arithmetic needs a second
+// wave to hide behind): two waves share each group of 32 query rows and split the head
 // dimension between them.  Each computes the partial scores over its 128 columns of Q and K,
 // the two partial S tiles are exchanged through LDS and added (both waves then hold the same S
 // and run the same softmax), and each accumulates its own 128 columns of O.  8 waves, 128 rows
@@ -93,9 +97,10 @@ struct ILCfgPair {
 // Occupancy: two workgroups per CU at head dim 128 (about 250 registers); at head dim 64, where the
 // vector work per matrix instruction doubles and a third wave per SIMD adds the issue slots it needs,
 // three workgroups in 168 registers each (measured +3..10 %); the dropout variant, whose mask arithmetic
-// does not fit 168 registers without spilling, stays at two.
+// does not fit 168 registers without spilling, stays at two; one wave per SIMD (all 512 registers) for the
+// whole-head-dim form at 256.
 template <typename T, typename C, bool DROPOUT = false>
-__global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROPOUT) ? 3 : 2) prefill_il_kernel(const KParams kp) {
+__global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 256) ? 1 : (!C::kPair && C::D == 64 && !DROPOUT) ? 3 : 2) prefill_il_kernel(const KParams kp) {
     constexpr int D = C::D, BN = C::BN;
     typedef typename Elem<T>::v8 v8;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -108,7 +113,7 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
     const int G = p.h / p.h_k;
     int g, mb, hk, b;
     if (!xcd_work_item(kp, (uint32_t)kp.num_m_blocks,
-                       !(kp.has_left || kp.has_right) ? 0u : C::kPair ? 32u : ((C::D == 64 && !DROPOUT) ? 96u : 64u), g, mb, hk, b)) return;
+                       !(kp.has_left || kp.has_right) ? 0u : (C::kPair || C::D == 256) ? 32u : ((C::D == 64 && !DROPOUT) ? 96u : 64u), g, mb, hk, b)) return;
     const int head = hk * G + g;
 
     const SeqInfo si = seq_info(p, b);
@@ -167,6 +172,11 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
     const int frow = (wave * 64 + lane) / C::CPR;
     const int fch = lane % C::CPR;
     const int kch = min(swz_k<D>(fch, frow), p.d / 8 - 1);
+    // (a pass of fewer than 16 rows -- 256 lanes at head dim 256 cover 8 -- alternates between two row
+    // phases of the K swizzle: odd passes take their own chunk)
+    constexpr bool kTwoPhases = (C::ROWS_PER_PASS % 16) != 0;
+    static_assert(!kTwoPhases || C::ROWS_PER_PASS == 8, "K swizzle phase per pass");
+    const int kch1 = kTwoPhases ? min(swz_k<D>(fch, frow + C::ROWS_PER_PASS), p.d / 8 - 1) : kch;
     const int vch = min(swz_v<D>(fch, frow), p.d / 8 - 1);
     const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
     const uint32_t fill_base = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(wave * 1024));
@@ -178,6 +188,7 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
     const T* ktile = kg + (int64_t)(t_hi - 1) * BN * p.k_row_stride;     // uniform
     const T* vtile = vg + (int64_t)(t_hi - 1) * BN * p.v_row_stride;
     const uint32_t koff = (uint32_t)(((int64_t)frow * p.k_row_stride + kch * 8) * 2);
+    const uint32_t koff1 = (uint32_t)(((int64_t)frow * p.k_row_stride + kch1 * 8) * 2);
     const uint32_t voff = (uint32_t)(((int64_t)frow * p.v_row_stride + vch * 8) * 2);
     const bool tail_clamp = t_hi * BN > si.sk;    // only visit 0 can reach past seqlen_k
     auto fill_s = [&](const T* base, uint32_t off, uint32_t dst) { async_fill16(base, off, dst); };
@@ -187,11 +198,11 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) {
                 const int n = min(frow + j * C::ROWS_PER_PASS, si.sk - 1 - (t_hi - 1) * BN);
-                fill_s(ktile, (uint32_t)(((int64_t)n * p.k_row_stride + kch * 8) * 2), dst + j * C::PASSB);
+                fill_s(ktile, (uint32_t)(((int64_t)n * p.k_row_stride + ((j & 1) ? kch1 : kch) * 8) * 2), dst + j * C::PASSB);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < C::LOADS; j++) fill_s(ktile + j * kpass, koff, dst + j * C::PASSB);
+            for (int j = 0; j < C::LOADS; j++) fill_s(ktile + j * kpass, (j & 1) ? koff1 : koff, dst + j * C::PASSB);
         }
         ktile -= kstep;
     };
@@ -574,7 +585,7 @@ __global__ void __launch_bounds__(C::kThreads, (!C::kPair && C::D == 64 && !DROP
     // behind the barrier that follows the last product and each wave uses its own region
     {
         constexpr int OCPR = C::DH / 8;                 // 16 B chunks per output row of the wave
-        constexpr int OCPP = OCPR <= 8 ? 8 : 16;        // lanes per row in a store instruction (a power of two)
+        constexpr int OCPP = OCPR <= 8 ? 8 : OCPR <= 16 ? 16 : 32;   // lanes per row in a store instruction (a power of two)
         constexpr int PITCH = OCPP * 16 + 16;
         static_assert(C::kWaves * 32 * PITCH <= C::SMEM, "staging region");
         char* stage = smem + wave * (32 * PITCH);
@@ -626,10 +637,16 @@ int launch_prefill_il(const KParams& kp, hipStream_t stream) {
     }
     return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream);
 }
+// Head dims 129..256.  Without dropout: the whole head dimension in one wave, 32-key tiles, one wave per SIMD
+// (ILCfg<T, 256, 32>; head dims up to 192 run 12 of 16 k-steps and 6 of 8 output column blocks).  Measured
+// against the pair form on the same shapes: +9 % causal 8k, +15 % full, +10 % at head dim 192, +7 % on packed
+// batches.  64-key tiles do not work there: the step then holds 64 matrix instructions and the compiler no
+// longer unrolls it (the S tiles end up in scratch memory, 14 x slower).  With dropout: the pair form.
 template <typename T>
-int launch_prefill_il_pair(const KParams& kp, hipStream_t stream) {
-    if (kp.p.d <= 192 && !(kp.p.p_dropout > 0.f)) return launch_prefill_il_one<T, ILCfgPair<T, 192>, false>(kp, stream);
-    return launch_prefill_il_cfg<T, ILCfgPair<T>>(kp, stream);
+int launch_prefill_il_256(const KParams& kp, hipStream_t stream) {
+    if (kp.p.p_dropout > 0.f) return launch_prefill_il_one<T, ILCfgPair<T>, true>(kp, stream);
+    if (kp.p.d <= 192) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 192>, false>(kp, stream);
+    return launch_prefill_il_one<T, ILCfg<T, 256, 32>, false>(kp, stream);
 }
 
 }  // namespace fa

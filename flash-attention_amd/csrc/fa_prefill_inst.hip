@@ -35,8 +35,9 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
         return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }
 #else
-    // head dim 129..256: pairs of waves split the head dimension (fa_prefill_il.h)
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) return launch_prefill_il_pair<InstT>(kp, stream);
+    // head dim 129..256: one wave per SIMD with the whole head dimension, or pairs of waves that split it
+    // (with dropout); fa_prefill_il.h
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) return launch_prefill_il_256<InstT>(kp, stream);
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }
