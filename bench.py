@@ -182,6 +182,33 @@ def bench_hbm_peak(steps, warmup):
     return res
 
 
+def bench_lds_peak(steps, warmup):
+    """What the LDS of a CU delivers to 16-byte-per-lane reads (fa_lds_read_peak in the library), with one and
+    with two waves per SIMD, in bytes per shader clock; at the full matrix rate the operand fragments of the
+    attention kernels need 128."""
+    import ctypes
+    import torch
+    from flash_attn import _native as nat
+    lib = nat.lib
+    lib.fa_lds_read_peak.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64),
+                                     ctypes.c_void_p, ctypes.c_void_p]
+    lib.fa_lds_read_peak.restype = ctypes.c_int
+    wgs = 256
+    cycles = torch.zeros(wgs, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {"kernel": "fa::lds_read_peak_kernel (ds_read_b128, 1 KB per wave instruction, no bank conflicts, one workgroup per CU)"}
+    for waves in (4, 8):
+        nbytes = ctypes.c_int64(0)
+        for _ in range(3):
+            rc = lib.fa_lds_read_peak(cycles.data_ptr(), wgs, waves, 5000, ctypes.byref(nbytes), sink.data_ptr(), stream)
+            if rc != 0:
+                raise RuntimeError("fa_lds_read_peak failed: %d" % rc)
+        torch.cuda.synchronize()
+        res["waves_per_simd_%d" % (waves // 4)] = {"bytes_per_clock_per_cu": nbytes.value / cycles.double().mean().item()}
+    return res
+
+
 def bench_rotary(steps, warmup):
     import torch
     from flash_attn.layers.rotary import apply_rotary
@@ -366,7 +393,7 @@ def main():
     ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default=None,
-                    choices=["prefill", "mfma_peak", "hbm_peak", "decode", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
+                    choices=["prefill", "mfma_peak", "hbm_peak", "lds_peak", "decode", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
                     help="run one leg alone and print its record (for profiler runs: the trace then holds that leg's kernels only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
@@ -390,7 +417,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.only:
-        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "decode": bench_decode, "rotary": bench_rotary,
+        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "lds_peak": bench_lds_peak, "decode": bench_decode, "rotary": bench_rotary,
                "backward": bench_backward, "fwd_bwd": bench_fwd_bwd, "varlen": bench_varlen, "gqa_window": bench_gqa_window,
                "head_dims": bench_head_dims}[a.only]
         print(json.dumps({"only": a.only, "steps": a.steps, "warmup": a.warmup, a.only: leg(a.steps, a.warmup)}))
@@ -399,6 +426,7 @@ def main():
     peak = bench_mfma_peak(a.steps, a.warmup)
     pre["roofline"]["measured_peak"] = peak["random_bf16"]["tflops"]
     pre["roofline"]["frac_of_measured_peak"] = pre["tflops"] / peak["random_bf16"]["tflops"]
+    lds = bench_lds_peak(a.steps, a.warmup)
     out = {
         "metric": "fwd TFLOP/s (bf16, hdim128, causal, 8k)",
         "value": pre["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -409,6 +437,7 @@ def main():
         "tokens_per_s": pre["tokens_per_s"],
         "roofline": pre["roofline"],
         "mfma_peak": peak,
+        "lds_peak": lds,
     }
     if not a.no_decode:
         dec = bench_decode(a.steps, a.warmup)

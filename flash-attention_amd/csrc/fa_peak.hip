@@ -5,7 +5,8 @@
 // of the operands, so the sustained rate depends on the DATA.  This kernel runs nothing but independent
 // MFMAs (one wave per SIMD, four accumulators in rotation, operands resident in registers) on operands
 // that are either random bf16 values (sign, three exponents around 1, random mantissa) or zeros, and the
-// benchmark reports both next to the attention kernels' rates.  Beside it: the same for HBM reads.
+// benchmark reports both next to the attention kernels' rates.  Beside it: the same for HBM reads and for
+// LDS reads.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "fa_mi355x.h"
@@ -83,7 +84,38 @@ __global__ void __launch_bounds__(256) hbm_read_peak_kernel(const peak_u32x4* __
     if (r == 0x9e3779b9u && n16 < 0) *sink = r;      // keeps the loads alive; never true
 }
 
+// LDS microbenchmark: what the LDS of a CU delivers to ds_read_b128 (one 1 KB operand fragment per wave
+// instruction, the access the attention kernels feed their matrix instructions with).  One workgroup per CU,
+// `waves` waves each reading its own conflict-free 16 KB window over and over; cycles[workgroup] receives the
+// shader-clock cycles the workgroup's loop took.
+__global__ void __launch_bounds__(1024) lds_read_peak_kernel(uint64_t* cycles, uint32_t* sink, int iters) {
+    __shared__ __attribute__((aligned(16))) char window[65536];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < 65536 / 4; i += blockDim.x) reinterpret_cast<uint32_t*>(window)[i] = (uint32_t)i * 2654435761u;
+    __syncthreads();
+    const char* base = window + (wave & 3) * 16384 + lane * 16;
+    peak_u32x4 acc = {0, 0, 0, 0};
+    const uint64_t t0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int u = 0; u < 16; u++) acc ^= *reinterpret_cast<const peak_u32x4*>(base + u * 1024);
+        asm volatile("" : "+v"(acc));
+    }
+    const uint64_t t1 = __builtin_readcyclecounter();
+    if (tid == 0) cycles[blockIdx.x] = t1 - t0;
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u && iters < 0) *sink = acc[0];     // never true
+}
+
 }  // namespace fa
+
+extern "C" int fa_lds_read_peak(uint64_t* cycles, int32_t workgroups, int32_t waves, int32_t iters, int64_t* bytes_per_workgroup,
+                                void* sink, void* hip_stream) {
+    if (!cycles || !sink || !bytes_per_workgroup || workgroups <= 0 || waves <= 0 || waves > 16 || iters <= 0) return 1;
+    hipLaunchKernelGGL(fa::lds_read_peak_kernel, dim3(workgroups), dim3(64 * waves), 0, (hipStream_t)hip_stream, cycles,
+                       reinterpret_cast<uint32_t*>(sink), iters);
+    *bytes_per_workgroup = (int64_t)waves * iters * 16 * 1024;
+    return (int)hipGetLastError();
+}
 
 extern "C" int fa_hbm_read_peak(const void* src, int64_t bytes, int32_t nontemporal, void* sink, void* hip_stream) {
     if (!src || !sink || bytes < 16 || ((uintptr_t)src & 15) != 0) return 1;

@@ -301,6 +301,16 @@ int fa_mfma_peak(float *sink, int32_t iters, int32_t random_operands, int64_t *f
  */
 int fa_hbm_read_peak(const void *src, int64_t bytes, int32_t nontemporal, void *sink, void *hip_stream);
 
+/*
+ * LDS microbenchmark (measurement aid; no counterpart in the reference): `workgroups` workgroups of `waves`
+ * waves (1..16) each issue iters x 16 conflict-free ds_read_b128 instructions (1 KB per wave instruction) and
+ * write the shader-clock cycles of that loop to cycles[workgroup] (device memory, `workgroups` x 8 bytes);
+ * *bytes_per_workgroup receives the LDS bytes one workgroup read.  bytes / cycles is the LDS read rate of a
+ * CU in bytes per clock when one workgroup runs per CU.  `sink` is 4 bytes of device memory (never written).
+ */
+int fa_lds_read_peak(uint64_t *cycles, int32_t workgroups, int32_t waves, int32_t iters, int64_t *bytes_per_workgroup,
+                     void *sink, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif
