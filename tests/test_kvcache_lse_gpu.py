@@ -22,6 +22,11 @@ def _say(*a):
     sys.stdout.flush()
 
 
+def _fa_func():
+    import flash_attn
+    return flash_attn.flash_attn_func
+
+
 def _nat():
     import flash_attn._native as nat
     return nat
@@ -126,3 +131,49 @@ def test_lse_tiled_split_kernel():
     lse, l_ref = _run(q, kc, vc, lens, causal=True, num_splits=3)
     assert torch.isposinf(l_ref[1, :, :30]).all() and torch.isposinf(lse[1, :, :30]).all()
     _run(q, kc, vc, lens, causal=True, window=(100, 0), num_splits=0)
+
+
+@pytest.mark.parametrize("mode", ["plain", "causal", "append_rotary", "window_right", "window_left"])
+@pytest.mark.parametrize("h,hk,d", [(32, 1, 128), (64, 2, 64), (40, 2, 128), (24, 1, 256), (17, 1, 96)])
+def test_single_query_with_more_than_16_grouped_heads(h, hk, d, mode):
+    """One query position and more grouped q heads per kv head than the decode kernel packs (16): the library
+    reads q and out with the grouped heads as rows (the reference's seqlen_q <-> ngroups swap,
+    csrc/flash_attn/flash_api.cpp:1096-1104), so K/V are fetched once per kv head.  Output, log-sum-exp and the
+    appended rows must be those of the plain problem; a left window bound keeps the plain form."""
+    _say("single query, many grouped heads", h, hk, d, mode)
+    nat = _nat()
+    dtype, cap, b = torch.bfloat16, 5000, 3
+    torch.manual_seed(h + d)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, 1, h, d, dtype=dtype)
+    lens = torch.tensor([4096, 37, 2500], dtype=torch.int32)
+    kn = vn = cos = sin = None
+    causal, wl, wr = mode == "causal", -1, -1
+    if mode == "append_rotary":
+        kn = torch.randn(b, 1, hk, d, dtype=dtype)
+        vn = torch.randn(b, 1, hk, d, dtype=dtype)
+        cos, sin = orc.rotary_table(cap, d, dtype=dtype)
+        causal = True
+    if mode == "window_right":
+        wr = 7
+    if mode == "window_left":
+        wl = 300
+    dev = lambda t: None if t is None else t.to(DEV)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    out, lse = nat.fwd_kvcache(q.to(DEV), kc_d, vc_d, dev(kn), dev(vn), lens.to(DEV), dev(cos), dev(sin), None, None, d ** -0.5,
+                               causal, wl, wr, True, 0)
+    kw = dict(causal=causal, window_size=(wl, wr))
+    o_ref, l_ref, k_ref, v_ref = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, **kw)
+    o_pt, _, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, upcast=False, reorder_ops=True, **kw)
+    ok, err, bound = orc.tolerance_ok(out.cpu(), o_ref, o_pt, 3.0, 1e-5)
+    _say("   out err %.3e bound %.3e" % (err, bound))
+    assert ok
+    assert lse.shape == (b, h, 1) and orc.lse_ok(lse.cpu(), l_ref, 1e-3)[0]
+    assert torch.equal(vc_d.cpu(), v_ref)
+    assert torch.allclose(kc_d.cpu().float(), k_ref.float(), rtol=1e-3, atol=1e-3)
+    # the same through the public call without a cache argument (mha_fwd path), one batch entry at its length
+    if mode in ("plain", "causal"):
+        L = int(lens[2])
+        o2 = _fa_func()(q[2:3].to(DEV), kc[2:3, :L].to(DEV), vc[2:3, :L].to(DEV), causal=causal)
+        assert orc.tolerance_ok(o2.cpu(), o_ref[2:3], o_pt[2:3], 3.0, 1e-5)[0]
