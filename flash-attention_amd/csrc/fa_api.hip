@@ -67,6 +67,25 @@ static bool groups_as_rows(fa_fwd_params& q) {
     return true;
 }
 
+// A few query positions (speculative or chunked decoding) with grouped q heads: seqlen_q x G rows would be
+// G separate row blocks of the tiled kernel, each streaming the kv head's K/V for a handful of rows.  Here the
+// (position, grouped head) pairs of a kv head become the rows of one problem with h_k heads (KParams::pack_g):
+// row = position * G + head within the group, so a workgroup serves up to 128 of them and K/V are fetched once
+// (batch 64 x 16k keys, 64 q heads on 8 kv heads, 4 positions: 4.0 -> 0.8 ms).  Up to 16 rows the decode kernel
+// packs them itself; from 128 positions on a row block is full without packing.  Returns G when it applies.
+static int positions_and_groups_as_rows(fa_fwd_params& q, int64_t* q_head_stride, int64_t* o_head_stride) {
+    const int G = q.h_k > 0 ? q.h / q.h_k : 0;
+    if (q.seqlen_q <= 1 || q.seqlen_q >= 128 || G < 2 || (int64_t)q.seqlen_q * G <= 16 || q.cu_seqlens_q || q.p_dropout != 0.f || q.s_dmask)
+        return 0;
+    if (q_head_stride) *q_head_stride = q.q_head_stride;
+    if (o_head_stride) *o_head_stride = q.o_head_stride;
+    q.seqlen_q *= G;
+    q.h = q.h_k;
+    q.q_head_stride *= G;
+    q.o_head_stride *= G;
+    return G;
+}
+
 static int check_common(const fa_fwd_params* p) {
     if (!p) return fail("params is NULL");
     if (!p->q || !p->k || !p->v || !p->o || !p->softmax_lse) return fail("q, k, v, o and softmax_lse must be set");
@@ -110,7 +129,8 @@ struct SplitPlan {
 static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     SplitPlan r;
     fa_fwd_params p = p_in;
-    groups_as_rows(p);         // what runs is the problem with the grouped heads as rows (no change when it already is)
+    // what runs is the problem with the grouped heads as rows (no change when it already is)
+    if (!groups_as_rows(p)) positions_and_groups_as_rows(p, nullptr, nullptr);
     const int sk = p.seqlen_k;
     const int db = bucket(p.d);
     const bool dec = use_decode_kernel(p);
@@ -190,6 +210,8 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = kp.dec_compact = 0;
     kp.work_counter = q.work_counter;
     kp.work_items = nullptr;
+    kp.pack_g = 0;
+    kp.pack_q_hs = kp.pack_o_hs = 0;
     // K + V, 16-bit elements; seqlen_k is the cache capacity (or the longest packed sequence): an upper bound
     kp.stream_kv = (int64_t)4 * q.b * q.seqlen_k * q.h_k * q.d >= kStreamKvBytes;
 }
@@ -367,6 +389,7 @@ int fa_fwd(const fa_fwd_params* p, void* hip_stream) {
     kp.p.seqlen_knew = 0;
     kp.p.rotary_dim = 0;
     if (groups_as_rows(kp.p)) kp.has_right = 0;
+    else kp.pack_g = positions_and_groups_as_rows(kp.p, &kp.pack_q_hs, &kp.pack_o_hs);
     if (int r = resolve_splits(kp, kp.p, true)) return r;
     return run_attention(kp, (hipStream_t)hip_stream);
 }
@@ -416,6 +439,7 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
     kp.rotary_q = kp.p.rotary_dim > 0;
     // (q rotary: without a mask every row is rotated to the position of the first new token, as the one row was)
     if (groups_as_rows(kp.p)) kp.has_right = 0;
+    else kp.pack_g = positions_and_groups_as_rows(kp.p, &kp.pack_q_hs, &kp.pack_o_hs);
     if (int r = resolve_splits(kp, kp.p, true)) return r;
     hipStream_t stream = (hipStream_t)hip_stream;
     // The persistent decode kernel appends the new rows itself: the item that reaches them writes them.

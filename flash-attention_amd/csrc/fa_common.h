@@ -61,6 +61,13 @@ struct KParams {
     // K and V together hold kStreamKvBytes or more (several times what the 256 MB memory-side cache keeps): the decode
     // kernels, which read every row once, fetch them with non-temporal loads
     int32_t stream_kv;
+    // Few query positions with grouped q heads (pack_g > 1): the rows of the tiled kernel's problem are the
+    // (position, grouped head) pairs of one kv head, row = position * pack_g + head within the group; p.h is
+    // then the number of kv heads, p.seqlen_q the number of such rows, p.q_head_stride / p.o_head_stride step
+    // over a whole group and pack_q_hs / pack_o_hs over one q head.  Masks, rotary positions and softmax_lse
+    // follow the position, row / pack_g.
+    int32_t pack_g;
+    int64_t pack_q_hs, pack_o_hs;
     int32_t* work_counter;
     // Packed batches: work list built on the device from cu_seqlens_q just before the launch (work_list_kernel,
     // fa_aux.hip), or NULL.  8 item counts, then for XCD x a list of (gridDim.x / 8) slots of two words:
@@ -520,7 +527,10 @@ FA_DEV void combine_row(const KParams& kp, const int64_t row, const int lane) {
     const int i = (int)(row % p.seqlen_q);
     const int h = (int)((row / p.seqlen_q) % p.h);
     const int b = (int)(row / ((int64_t)p.seqlen_q * p.h));
-    if (lane == 0) p.softmax_lse[row] = lse;
+    // rows that stand for (position, grouped head) pairs: see KParams::pack_g
+    const int pg = kp.pack_g > 1 ? kp.pack_g : 1;
+    const int qi = i / pg, gg = i - qi * pg;
+    if (lane == 0) p.softmax_lse[(((int64_t)b * p.h + h) * pg + gg) * (p.seqlen_q / pg) + qi] = lse;
 
     // each lane owns 4 consecutive output dims (64 lanes x 4 = 256 dims max)
     const int d0 = lane * 4;
@@ -551,7 +561,8 @@ FA_DEV void combine_row(const KParams& kp, const int64_t row, const int lane) {
             if (w[j] != 0.f) acc += v[j] * w[j];
     }
     if (d0 < p.d) {
-        int64_t off = (int64_t)i * p.o_row_stride + (int64_t)h * p.o_head_stride + (int64_t)b * p.o_batch_stride;
+        int64_t off = (int64_t)qi * p.o_row_stride + (int64_t)h * p.o_head_stride + (int64_t)b * p.o_batch_stride;
+        if (pg > 1) off += (int64_t)gg * kp.pack_o_hs;
         u32x2 v = {pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3])};
         st_global8(reinterpret_cast<T*>(p.o) + off + d0, v);
     }

@@ -67,13 +67,15 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     const int m0 = mb * C::BM;
     if (m0 >= si.sq) return;
 
-    const int shift = si.sk - si.sq;
+    // rows may stand for (query position, grouped head) pairs (KParams::pack_g): the position of row r is r / pg
+    const int pg = kp.pack_g > 1 ? kp.pack_g : 1;
+    const int shift = si.sk - si.sq / pg;
     const int wl = p.window_left, wr = p.window_right;
     const bool has_left = kp.has_left, has_right = kp.has_right;
     int n_hi = si.sk;
-    if (has_right) n_hi = min(n_hi, min(m0 + C::BM, si.sq) + shift + wr);
+    if (has_right) n_hi = min(n_hi, (min(m0 + C::BM, si.sq) - 1) / pg + 1 + shift + wr);
     int n_lo = 0;
-    if (has_left) n_lo = max(0, m0 + shift - wl);
+    if (has_left) n_lo = max(0, m0 / pg + shift - wl);
     int t_lo = n_lo / BN;
     int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
     if (SPLIT) {
@@ -92,7 +94,8 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     for (int rb = 0; rb < RB; rb++) {
         const int row = m0 + (wave * RB + rb) * 32 + l32;
         const bool valid = row < si.sq;
-        const T* qrow = qg + (int64_t)row * p.q_row_stride;
+        const int qi = row / pg;
+        const T* qrow = qg + (int64_t)qi * p.q_row_stride + (pg > 1 ? (int64_t)(row - qi * pg) * kp.pack_q_hs : (int64_t)0);
 #pragma unroll
         for (int dk = 0; dk < C::KS; dk++) {
             const int d0 = dk * 16 + 8 * hh;
@@ -102,7 +105,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                 if (kp.rotary_q && d0 < p.rotary_dim) {
                     // (a full cache puts cache length + row past the cache: the table is only known to cover the
                     // cache capacity, so the position stops at its last row)
-                    const int pos = min(si.sk_cache + ((p.is_causal || has_left || has_right) ? row : 0), p.seqlen_k - 1);
+                    const int pos = min(si.sk_cache + ((p.is_causal || has_left || has_right) ? qi : 0), p.seqlen_k - 1);
                     const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
                     const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
                     float x[8];
@@ -186,8 +189,8 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             const int r0 = m0 + (wave * RB + rb) * 32;
-            skip[rb] = (has_right && n0 > r0 + 31 + shift + wr) ||
-                       (has_left && n0 + BN - 1 < r0 + shift - wl) || (r0 >= si.sq);
+            skip[rb] = (has_right && n0 > (r0 + 31) / pg + shift + wr) ||
+                       (has_left && n0 + BN - 1 < r0 / pg + shift - wl) || (r0 >= si.sq);
             any_work |= !skip[rb];
         }
 
@@ -202,10 +205,10 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
             for (int rb = 0; rb < RB; rb++) {
                 if (skip[rb]) continue;
                 const int r0 = m0 + (wave * RB + rb) * 32;
-                const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0 + shift + wr) ||
-                                       (has_left && n0 < r0 + 31 + shift - wl);
+                const bool need_mask = (n0 + BN > si.sk) || (has_right && n0 + BN - 1 > r0 / pg + shift + wr) ||
+                                       (has_left && n0 < (r0 + 31) / pg + shift - wl);
                 if (need_mask) {
-                    const int row = r0 + l32;
+                    const int row = (r0 + l32) / pg;       // the query position the masks follow
                     int lim_hi = si.sk - 1;
                     if (has_right) lim_hi = min(lim_hi, row + shift + wr);
                     const int lim_lo = has_left ? row + shift - wl : 0;
@@ -279,6 +282,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
         const float inv = dead ? 1.f : drop.rp / l_tot;
         const float lse = dead ? (SPLIT ? -INFINITY : INFINITY) : m_run[rb] * p.softmax_scale + __logf(l_tot);
         if (row >= si.sq) continue;
+        const int qi = row / pg, gg = row - qi * pg;
         if (SPLIT) {
             const int64_t ridx = (((int64_t)split * p.b + b) * p.h + head) * p.seqlen_q + row;
             if (hh == 0) p.lse_accum[ridx] = lse;
@@ -295,8 +299,9 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
                     }
                 }
         } else {
-            if (hh == 0) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
-            T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)row * p.o_row_stride + (int64_t)head * p.o_head_stride;
+            if (hh == 0) p.softmax_lse[(((int64_t)b * p.h + head) * pg + gg) * (p.seqlen_q / pg) + qi] = lse;
+            T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)qi * p.o_row_stride + (int64_t)head * p.o_head_stride +
+                      (pg > 1 ? (int64_t)gg * kp.pack_o_hs : (int64_t)0);
 #pragma unroll
             for (int db = 0; db < C::DB; db++)
 #pragma unroll

@@ -22,8 +22,9 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     //    kernel, 256 rows per workgroup, each K/V tile fetched once per 256 rows;
     //  * otherwise from 512 query rows on: the software-pipelined kernel, two independent
     //    128-row workgroups per CU, whose start-up and output phases overlap.
-    // Shorter sequences, split key ranges and q rotary take the general 4-wave kernel.
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) {
+    // Shorter sequences, split key ranges, q rotary and rows that stand for (position, grouped head) pairs take
+    // the general 4-wave kernel.
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512 && kp.pack_g <= 1) {
         const bool masked = kp.has_right || kp.has_left;
         const bool long_keys = kp.p.seqlen_k >= (masked ? 2048 : 769);
         // When the 256-row blocks of the ping-pong kernel would occupy no more than half of the 256
@@ -37,7 +38,7 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
 #else
     // head dim 129..256: one wave per SIMD with the whole head dimension, or pairs of waves that split it
     // (with dropout); fa_prefill_il.h
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512) return launch_prefill_il_256<InstT>(kp, stream);
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= 512 && kp.pack_g <= 1) return launch_prefill_il_256<InstT>(kp, stream);
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }

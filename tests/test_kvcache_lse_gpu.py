@@ -177,3 +177,55 @@ def test_single_query_with_more_than_16_grouped_heads(h, hk, d, mode):
         L = int(lens[2])
         o2 = _fa_func()(q[2:3].to(DEV), kc[2:3, :L].to(DEV), vc[2:3, :L].to(DEV), causal=causal)
         assert orc.tolerance_ok(o2.cpu(), o_ref[2:3], o_pt[2:3], 3.0, 1e-5)[0]
+
+
+@pytest.mark.parametrize("num_splits", [0, 1])
+@pytest.mark.parametrize("mode", ["plain", "causal", "append_rotary", "window_right", "window_left", "local"])
+@pytest.mark.parametrize("sq,h,hk,d", [(4, 64, 8, 128), (2, 32, 2, 64), (5, 12, 3, 128), (16, 8, 4, 96), (33, 6, 2, 128),
+                                        (100, 4, 2, 64), (3, 48, 1, 256), (127, 2, 1, 128)])
+def test_few_query_positions_with_grouped_heads(sq, h, hk, d, mode, num_splits):
+    """2..127 query positions with grouped q heads and more than 16 (position, head) rows per kv head (a draft of
+    several tokens checked at once, a short chunk of a prompt): the library lays those rows out as the rows of
+    one problem per kv head, so K/V are fetched once and not once per q head.  Masks and rotary positions follow
+    the position of a row, softmax_lse keeps its (batch, head, position) layout."""
+    _say("few positions, grouped heads", sq, h, hk, d, mode, num_splits)
+    nat = _nat()
+    dtype, cap, b = torch.bfloat16, 3000, 3
+    torch.manual_seed(sq * 7 + h)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, sq, h, d, dtype=dtype)
+    lens = torch.tensor([2500, max(sq, 37), 1203], dtype=torch.int32)
+    kn = vn = cos = sin = None
+    causal, wl, wr = mode in ("causal", "append_rotary"), -1, -1
+    if mode == "append_rotary":
+        kn = torch.randn(b, sq, hk, d, dtype=dtype)
+        vn = torch.randn(b, sq, hk, d, dtype=dtype)
+        cos, sin = orc.rotary_table(cap, d - d % 16, dtype=dtype)
+        lens = lens - sq                   # the cache holds the older tokens, the call appends these
+    if mode == "window_right":
+        wr = 2
+    if mode == "window_left":
+        wl = 300
+    if mode == "local":
+        wl, wr = 150, 1
+    dev = lambda t: None if t is None else t.to(DEV)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    out, lse = nat.fwd_kvcache(q.to(DEV), kc_d, vc_d, dev(kn), dev(vn), lens.to(DEV), dev(cos), dev(sin), None, None, d ** -0.5,
+                               causal, wl, wr, True, num_splits)
+    kw = dict(causal=causal, window_size=(wl, wr))
+    o_ref, l_ref, k_ref, v_ref = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, **kw)
+    o_pt, _, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, upcast=False, reorder_ops=True, **kw)
+    ok, err, bound = orc.tolerance_ok(out.cpu(), o_ref, o_pt, 3.0, 1e-5)
+    _say("   out err %.3e bound %.3e" % (err, bound))
+    assert ok
+    assert lse.shape == (b, h, sq) and orc.lse_ok(lse.cpu(), l_ref, 1e-3)[0]
+    assert torch.equal(vc_d.cpu(), v_ref)
+    assert torch.allclose(kc_d.cpu().float(), k_ref.float(), rtol=1e-3, atol=1e-3)
+    if mode in ("plain", "causal", "local") and num_splits == 0:
+        # the same problem through flash_attn_func on one batch entry (q as a strided view of a wider tensor)
+        L = int(lens[0])
+        wide = torch.zeros(1, sq, h + 2, d, dtype=dtype)
+        wide[:, :, 1:h + 1] = q[0:1]
+        o2 = _fa_func()(wide.to(DEV)[:, :, 1:h + 1], kc[0:1, :L].to(DEV), vc[0:1, :L].to(DEV), causal=causal, window_size=(wl, wr))
+        assert orc.tolerance_ok(o2.cpu(), o_ref[0:1], o_pt[0:1], 3.0, 1e-5)[0]
