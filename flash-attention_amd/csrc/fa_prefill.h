@@ -39,7 +39,10 @@ struct PrefillCfg {
     static_assert(RB == 1, "one 32-row block per wave");
 };
 
-template <typename T, int D, int RB, int BN, int MINW, bool SPLIT, bool DROPOUT = false>
+// STREAM: K and V tiles are fetched with non-temporal loads -- for launches in which every K/V row is read by
+// exactly one workgroup (one row block per kv head, all of its q heads in it) and the caches are too large to
+// stay in the memory-side cache anyway (+5-8 % there; see decode_item in fa_decode.hip).
+template <typename T, int D, int RB, int BN, int MINW, bool SPLIT, bool DROPOUT = false, bool STREAM = false>
 __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     typedef PrefillCfg<T, D, RB, BN> C;
     typedef typename Elem<T>::v8 v8;
@@ -143,8 +146,13 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
             const int f = tid + i * C::kThreads;
             const int row = f / C::CPR, c = min(f % C::CPR, d_last_chunk);
             const int n = min(n0 + row, si.sk - 1);
-            kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
-            vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
+            if constexpr (STREAM) {
+                kr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kg + (int64_t)n * p.k_row_stride + c * 8));
+                vr[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vg + (int64_t)n * p.v_row_stride + c * 8));
+            } else {
+                kr[i] = ld_global16(kg + (int64_t)n * p.k_row_stride + c * 8);
+                vr[i] = ld_global16(vg + (int64_t)n * p.v_row_stride + c * 8);
+            }
         }
     };
     auto store_tile = [&](int buf, int t) {
@@ -329,7 +337,18 @@ int launch_prefill(KParams kp, hipStream_t stream) {
     if (nblocks == 0) return -2;
     dim3 grid((unsigned)nblocks), block(C::kThreads);
     hipError_t e;
-    if (split) {
+    const bool one_reader = kp.stream_kv && kp.num_m_blocks == 1 && kp.p.h == kp.p.h_k && !(kp.p.p_dropout > 0.f);
+    if (split && one_reader) {
+        auto kern = prefill_kernel<T, D, RB, BN, MINW, true, false, true>;
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    } else if (one_reader) {
+        auto kern = prefill_kernel<T, D, RB, BN, MINW, false, false, true>;
+        e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
+    } else if (split) {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, true>;
         e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
         if (e != hipSuccess) return (int)e;
