@@ -29,9 +29,12 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
         const bool long_keys = kp.p.seqlen_k >= (masked ? 2048 : 769);
         // When the 256-row blocks of the ping-pong kernel would occupy no more than half of the 256
         // CUs (a chunk of 1024 queries of one sequence with 32 heads: 128 blocks), the 128-row blocks
-        // of the pipelined kernel fill them: measured +12..25 % at 128 blocks, -11 % at 192.
+        // of the pipelined kernel fill them: measured +12..25 % at 128 blocks, -11 % at 192.  Under a mask up to
+        // 256 blocks: one 256-row block per CU leaves every CU waiting for the one with the heaviest block
+        // (causal 2k-8k at exactly 256 blocks: +4..12 %; 384 blocks: -2 %; without a mask the ping-pong kernel
+        // stays 10-14 % ahead at 256).
         const int64_t pp_wgs = (int64_t)((kp.p.seqlen_q + 255) / 256) * kp.p.h * kp.p.b;
-        if (FA_D >= 128 && long_keys && pp_wgs <= 128) return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
+        if (FA_D >= 128 && long_keys && pp_wgs <= (masked ? 256 : 128)) return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
         if (FA_D >= 128 && long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
         return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }
