@@ -360,6 +360,34 @@ def bench_decode(steps, warmup):
     }
 
 
+def bench_decode_variants(steps, warmup):
+    """Decoding shapes beside config 5 that take other paths of the library: four query positions at once on the
+    config 5 caches (a draft of four tokens: 32 (position, head) rows per kv head, laid out as the rows of one
+    tiled problem per kv head) and one position on a multi-query cache (32 q heads on 1 kv head: the grouped
+    heads become the rows).  Bytes: the cached K/V rows the masks let the queries see, once."""
+    import torch
+    import flash_attn
+    res = {}
+    for name, (b, cap, hk, h, d, sq, lo) in (("four_positions_gqa8", (64, 32768, 8, 64, 128, 4, 1024)),
+                                                ("one_position_mqa32", (16, 65536, 1, 32, 128, 1, 30000))):
+        torch.manual_seed(0)
+        k_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
+        v_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
+        q = torch.randn(b, sq, h, d, device="cuda", dtype=torch.bfloat16)
+        cache_seqlens = torch.randint(lo, cap - sq, (b,), dtype=torch.int32).cuda()
+        fn = lambda: flash_attn.flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=cache_seqlens, causal=True)
+        tm = time_steps(fn, steps, warmup)
+        ms = tm[0]
+        algo_bytes = int(cache_seqlens.long().sum().item()) * hk * d * 2 * 2 + 2 * b * sq * h * d * 2
+        gbs = algo_bytes / (ms * 1e-3) / 1e9
+        res[name] = {"ms": ms, "ms_min": tm.ms_min, "gb_per_s": gbs,
+                     "workload": "flash_attn_with_kvcache bf16 b%d cache(%d,%d,%d,%d) hq%d seqlen_q %d causal" % (b, b, cap, hk, d, h, sq),
+                     "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                                  "traffic": None, "kernel": "fa::prefill_kernel<bf16,128,split> + fa::combine_kernel", "bytes_per_launch": algo_bytes}}
+        del k_cache, v_cache
+    return res
+
+
 def cpu_baseline():
     """Oracle on the host cores: 1 batch entry x 4 heads of the prefill workload (1/32 of the
     (batch, head) pairs, which are independent), repeated for about 12 s."""
@@ -393,7 +421,7 @@ def main():
     ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default=None,
-                    choices=["prefill", "mfma_peak", "hbm_peak", "lds_peak", "decode", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
+                    choices=["prefill", "mfma_peak", "hbm_peak", "lds_peak", "decode", "decode_variants", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
                     help="run one leg alone and print its record (for profiler runs: the trace then holds that leg's kernels only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
@@ -417,7 +445,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.only:
-        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "lds_peak": bench_lds_peak, "decode": bench_decode, "rotary": bench_rotary,
+        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "lds_peak": bench_lds_peak, "decode": bench_decode, "decode_variants": bench_decode_variants, "rotary": bench_rotary,
                "backward": bench_backward, "fwd_bwd": bench_fwd_bwd, "varlen": bench_varlen, "gqa_window": bench_gqa_window,
                "head_dims": bench_head_dims}[a.only]
         print(json.dumps({"only": a.only, "steps": a.steps, "warmup": a.warmup, a.only: leg(a.steps, a.warmup)}))
@@ -446,6 +474,7 @@ def main():
         dec["roofline"]["frac_of_measured_peak"] = dec["gb_per_s"] / hbm["nontemporal"]["gb_per_s"]
         out["decode"] = dec
         out["hbm_peak"] = hbm
+        out["decode_variants"] = bench_decode_variants(a.steps, a.warmup)
     if not a.no_backward:
         out["rotary"] = bench_rotary(a.steps, a.warmup)
         out["backward"] = bench_backward(max(1, a.steps // 2), max(1, a.warmup // 2))
