@@ -36,9 +36,6 @@ static const int kNumCU = 256;   // MI355X
 #ifndef FA_DEC_SB
 #define FA_DEC_SB 8
 #endif
-#ifndef FA_ONEBLK_SLOTS
-#define FA_ONEBLK_SLOTS 4096    // work items per launch of the tiled kernel when every (batch, head) is one row block
-#endif
 #ifndef FA_DEC_MINLEN
 #define FA_DEC_MINLEN 512       // shortest chunk of the decode kernel (keys) once the launch fills the CUs
 #endif
@@ -137,7 +134,19 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     const int sk = p.seqlen_k;
     const int db = bucket(p.d);
     const bool dec = use_decode_kernel(p);
-    const int gran = dec ? 128 : prefill_block_n(db);
+    // The tiled kernel under the persistent schedule of the decode kernel (prefill_persistent_kernel): one row
+    // block per (batch, kv head) with every q head of the kv head in it, over a cache whose lengths are on the
+    // device.  Chunks of 2048 keys or more (about FA_DEC_SLOTS_P per launch), their remainders in pieces of 512+.
+    const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;
+    int64_t tile_chunk = 0;
+    if (!dec && allow_split && p.num_splits == 0 && p.p_dropout == 0.f && counters_ok(p) && !p.cu_seqlens_q && p.cu_seqlens_k &&
+        !p.is_seqlens_k_cumulative && p.seqlen_q <= prefill_block_m(db) && p.h == p.h_k) {
+        const int64_t len = (std::max<int64_t>(2048, (int64_t)sk * wgs / FA_DEC_SLOTS_P) + 511) / 512 * 512;
+        // (launches that fill the CUs without a split keep the plain form up to 8192 keys: two or three chunks per
+        // sequence do not pay for the merge)
+        if (sk >= 2 * len && (wgs < kNumCU || sk >= 8192)) tile_chunk = len;
+    }
+    const int gran = dec ? 128 : tile_chunk ? 512 : prefill_block_n(db);
     auto rup = [](int64_t x, int64_t m) { return (int)((x + m - 1) / m * m); };
     int splits = 1;
     bool automatic = false;
@@ -164,21 +173,17 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
                     if (lp >= 1024) len = std::max<int64_t>(lp, 2048);
                 }
                 splits = (int)((sk + len - 1) / len);
+            } else if (tile_chunk) {
+                splits = (int)((sk + tile_chunk - 1) / tile_chunk);
             } else {
-                const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;
                 if (wgs < kNumCU) {
                     const int64_t want = (2 * kNumCU + wgs - 1) / wgs;
                     splits = (int)std::min<int64_t>(want, (sk + 255) / 256);
                 }
-                // One row block per (batch, head) and enough of them to fill the CUs, over long keys: each
-                // workgroup streams its whole sequence alone, bound by its own requests in flight (about
-                // 16 GB/s), and sequences of unequal length leave the early finishers idle.  Chunks of 4096
-                // keys or more, about FA_ONEBLK_SLOTS work items per launch (batch 64 x 1-32k keys, 4 positions
-                // on 8 kv heads: +9 %).  Shorter keys and smaller launches lose to the extra merge.
-                else if (p.seqlen_q <= prefill_block_m(db) && sk >= 16384) {
-                    const int64_t len = rup(std::max<int64_t>(4096, (int64_t)sk * wgs / FA_ONEBLK_SLOTS), gran);
-                    splits = (int)((sk + len - 1) / len);
-                }
+                // From 256 row blocks on nothing is split here, also where every (batch, head) is one row block
+                // over long keys: the plan sees the capacity of a cache, not the lengths in it, and chunks cut for
+                // the capacity are mostly empty workgroups when the sequences are short (batch 64, 4096 keys in
+                // caches of 32768, 4 positions on 8 kv heads: 0.28 ms split against 0.19).
             }
         }
         splits = std::max(1, std::min(splits, FA_MAX_SPLITS));
@@ -195,8 +200,11 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     // The pieces of a remainder stay at 512 keys or more (halves of a 1024-key chunk, quarters of a
     // 2048-key one, eighths from 4096 on): shorter pieces are mostly start-up and merge (measured
     // +6 % at batch 256 x 4k and at batch 64 x 8k with 16 grouped heads, nothing lost at config 5).
-    const int sb = len < 2048 ? 2 : len < 4096 ? 4 : FA_DEC_SB;
-    if (dec && automatic && splits > 1 && counters_ok(p) && len >= 1024 && splits + sb <= FA_MAX_SPLITS) {
+    // (The tiled kernel pays more per item -- its Q rows, a first tile nothing overlaps, up to 128 partial rows to
+    // write: about what 160 keys take -- and its pieces stay at 1024 keys or more.)
+    // Halves, quarters or eighths of a multiple of 512: whole tiles.
+    const int sb = tile_chunk ? (len < 4096 ? 2 : len < 8192 ? 4 : FA_DEC_SB) : len < 2048 ? 2 : len < 4096 ? 4 : FA_DEC_SB;
+    if ((dec || tile_chunk) && automatic && splits > 1 && counters_ok(p) && len >= 1024 && splits + sb <= FA_MAX_SPLITS) {
         r.persistent = 1;
         r.sa = splits;
         r.sb = sb;

@@ -620,6 +620,108 @@ FA_DEV void dec_slot_counts(const KParams& kp, int b, int& n_macro, int& n_sub) 
     n_sub = min(kp.dec_sb, (hi - whole * kp.split_len + kp.dec_sub - 1) / kp.dec_sub);
 }
 
+// Key range of one work item.  kChunk: chunk `idx` of kp.split_len keys.  kMacro / kSub are the two
+// passes of the persistent schedule: first every COMPLETE chunk of kp.split_len keys, then the
+// ragged remainder of each sequence in pieces of kp.dec_sub keys, so that the last items handed out
+// are small and the workgroups finish together.
+enum ItemMode { kChunk = 0, kMacro = 1, kSub = 2 };
+// keys [c_lo, c_hi) of work item (mode, idx) of a sequence whose visible keys end at hi
+FA_DEV void item_key_range(const KParams& kp, int mode, int idx, int hi, int& c_lo, int& c_hi) {
+    if (mode == kSub) {
+        const int base = hi / kp.split_len * kp.split_len;     // start of the incomplete chunk
+        c_lo = base + idx * kp.dec_sub;
+        c_hi = (base == hi) ? c_lo : c_lo + kp.dec_sub;
+    } else {
+        c_lo = idx * kp.split_len;
+        c_hi = c_lo + kp.split_len;
+        if (mode == kMacro && c_hi > hi) c_hi = c_lo;          // incomplete: left to the kSub pass
+    }
+}
+
+// The persistent schedule itself, for a grid of resident workgroups: calls item(kv head, batch entry, partial
+// slot, mode, idx) for this workgroup's block id and then for every ticket it draws from kp.work_counter[0]
+// until the items are used up; the last workgroup to finish puts the two counter words back to zero.  All
+// lanes of the workgroup must call it together and return from every item (it synchronises the workgroup
+// between items, so an item may use all of LDS).
+template <class F>
+FA_DEV void for_each_ticket(const KParams& kp, F&& item) {
+    __shared__ int s_ticket;
+    // compact schedule: s_pm[b] / s_ps[b] = slots with keys (complete chunks / remainder pieces) of the batch
+    // entries before b; tickets then number only those slots, batch entry by batch entry, kv heads fastest
+    __shared__ int s_pm[kDecCompactMaxBatch + 1], s_ps[kDecCompactMaxBatch + 1];
+    const fa_fwd_params& p = kp.p;
+    int n_macro = p.b * kp.dec_sa * p.h_k;
+    int total = n_macro + p.b * kp.dec_sb * p.h_k;
+    if (kp.dec_compact) {
+        for (int bb = threadIdx.x; bb < p.b; bb += blockDim.x) {
+            int nm, ns;
+            dec_slot_counts(kp, bb, nm, ns);
+            s_pm[bb + 1] = nm;
+            s_ps[bb + 1] = ns;
+        }
+        __syncthreads();
+        if (threadIdx.x < 64) {        // one wave turns the counts into running sums, 64 entries at a time
+            const int lane = threadIdx.x;
+            int carry_m = 0, carry_s = 0;
+            for (int base = 0; base < p.b; base += 64) {
+                const int i = base + lane;
+                int vm = i < p.b ? s_pm[i + 1] : 0, vs = i < p.b ? s_ps[i + 1] : 0;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) {
+                    const int um = __shfl_up(vm, o), us = __shfl_up(vs, o);
+                    if (lane >= o) { vm += um; vs += us; }
+                }
+                if (i < p.b) { s_pm[i + 1] = carry_m + vm; s_ps[i + 1] = carry_s + vs; }
+                carry_m += __shfl(vm, 63);
+                carry_s += __shfl(vs, 63);
+            }
+            if (lane == 0) { s_pm[0] = 0; s_ps[0] = 0; }
+        }
+        __syncthreads();
+        n_macro = s_pm[p.b] * p.h_k;
+        total = n_macro + s_ps[p.b] * p.h_k;
+    }
+    int32_t* const ticket = kp.work_counter;
+    // the first item of a workgroup is the one its block id names (no round trip to the counter before any
+    // work starts); the tickets drawn afterwards continue behind the grid
+    for (bool first = true;; first = false) {
+        int t = (int)blockIdx.x;
+        if (!first) {
+            __syncthreads();          // previous item is done with LDS and with s_ticket
+            if (threadIdx.x == 0) s_ticket = (int)gridDim.x + __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            t = s_ticket;
+        }
+        if (t >= total) break;
+        const bool macro = t < n_macro;
+        if (!macro) t -= n_macro;
+        int hk, idx, b;
+        if (kp.dec_compact) {
+            const int* pre = macro ? s_pm : s_ps;
+            hk = t % p.h_k;
+            const int q = t / p.h_k;            // q-th slot with keys of its pass: the batch entry is the last b with pre[b] <= q
+            int lo_b = 0, hi_b = p.b;           // invariant: pre[lo_b] <= q < pre[hi_b]
+            while (hi_b - lo_b > 1) {
+                const int mid = (lo_b + hi_b) >> 1;
+                if (pre[mid] <= q) lo_b = mid; else hi_b = mid;
+            }
+            b = lo_b;
+            idx = q - pre[b];
+        } else {
+            const int per_b = macro ? kp.dec_sa : kp.dec_sb;
+            hk = t % p.h_k; idx = (t / p.h_k) % per_b; b = t / (p.h_k * per_b);
+        }
+        item(hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
+    }
+    if (threadIdx.x == 0) {
+        const int gone = __hip_atomic_fetch_add(kp.work_counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (gone == (int)gridDim.x - 1) {     // every workgroup has drawn its last ticket
+            __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(kp.work_counter + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // Which work item a workgroup of the tiled forward and backward kernels takes.  Block ids are dealt round-robin
 // over the 8 XCDs by hardware, each XCD has its own L2, and all row blocks of a (batch, kv head)
 // stream should meet in one L2 (heavy blocks first; grouped q heads adjacent).

@@ -38,12 +38,6 @@ struct DecodeCfg {
     static constexpr int SMEM = STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES;
 };
 
-// Key range of one work item.  kChunk: chunk `idx` of kp.split_len keys.  kMacro / kSub are the two
-// passes of the persistent schedule: first every COMPLETE chunk of kp.split_len keys, then the
-// ragged remainder of each sequence in pieces of kp.dec_sub keys, so that the last items handed out
-// are small and the workgroups finish together.
-enum ItemMode { kChunk = 0, kMacro = 1, kSub = 2 };
-
 // One (batch, kv head, key range) item: attention of the packed query rows over the range, written
 // as the final output (SPLIT = false) or as partial `slot` (SPLIT = true).
 // APPEND: rows [cache length, cache length + seqlen_knew) are not in the cache yet; the item whose key range
@@ -76,15 +70,7 @@ FA_DEV void decode_item(const KParams& kp, char* smem, const int hk, const int b
     if (has_left) lo = max(0, shift - wl);
     if (SPLIT) {
         int c_lo, c_hi;
-        if (mode == kSub) {
-            const int base = hi / kp.split_len * kp.split_len;     // start of the incomplete chunk
-            c_lo = base + idx * kp.dec_sub;
-            c_hi = (base == hi) ? c_lo : c_lo + kp.dec_sub;
-        } else {
-            c_lo = idx * kp.split_len;
-            c_hi = c_lo + kp.split_len;
-            if (mode == kMacro && c_hi > hi) c_hi = c_lo;          // incomplete: left to the kSub pass
-        }
+        item_key_range(kp, mode, idx, hi, c_lo, c_hi);
         lo = max(lo, c_lo);
         hi = min(hi, c_hi);
     }
@@ -383,81 +369,9 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 template <typename T, int D, bool APPEND, bool STREAM>
 __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    __shared__ int s_ticket;
-    // compact schedule: s_pm[b] / s_ps[b] = slots with keys (complete chunks / remainder pieces) of the batch
-    // entries before b; tickets then number only those slots, batch entry by batch entry, kv heads fastest
-    __shared__ int s_pm[kDecCompactMaxBatch + 1], s_ps[kDecCompactMaxBatch + 1];
-    const fa_fwd_params& p = kp.p;
-    int n_macro = p.b * kp.dec_sa * p.h_k;
-    int total = n_macro + p.b * kp.dec_sb * p.h_k;
-    if (kp.dec_compact) {
-        for (int bb = threadIdx.x; bb < p.b; bb += blockDim.x) {
-            int nm, ns;
-            dec_slot_counts(kp, bb, nm, ns);
-            s_pm[bb + 1] = nm;
-            s_ps[bb + 1] = ns;
-        }
-        __syncthreads();
-        if (threadIdx.x < 64) {        // one wave turns the counts into running sums, 64 entries at a time
-            const int lane = threadIdx.x;
-            int carry_m = 0, carry_s = 0;
-            for (int base = 0; base < p.b; base += 64) {
-                const int i = base + lane;
-                int vm = i < p.b ? s_pm[i + 1] : 0, vs = i < p.b ? s_ps[i + 1] : 0;
-#pragma unroll
-                for (int o = 1; o < 64; o <<= 1) {
-                    const int um = __shfl_up(vm, o), us = __shfl_up(vs, o);
-                    if (lane >= o) { vm += um; vs += us; }
-                }
-                if (i < p.b) { s_pm[i + 1] = carry_m + vm; s_ps[i + 1] = carry_s + vs; }
-                carry_m += __shfl(vm, 63);
-                carry_s += __shfl(vs, 63);
-            }
-            if (lane == 0) { s_pm[0] = 0; s_ps[0] = 0; }
-        }
-        __syncthreads();
-        n_macro = s_pm[p.b] * p.h_k;
-        total = n_macro + s_ps[p.b] * p.h_k;
-    }
-    int32_t* const ticket = kp.work_counter;
-    // the first item of a workgroup is the one its block id names (no round trip to the counter before any
-    // work starts); the tickets drawn afterwards continue behind the grid
-    for (bool first = true;; first = false) {
-        int t = (int)blockIdx.x;
-        if (!first) {
-            __syncthreads();          // previous item is done with LDS and with s_ticket
-            if (threadIdx.x == 0) s_ticket = (int)gridDim.x + __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-            t = s_ticket;
-        }
-        if (t >= total) break;
-        const bool macro = t < n_macro;
-        if (!macro) t -= n_macro;
-        int hk, idx, b;
-        if (kp.dec_compact) {
-            const int* pre = macro ? s_pm : s_ps;
-            hk = t % p.h_k;
-            const int q = t / p.h_k;            // q-th slot with keys of its pass: the batch entry is the last b with pre[b] <= q
-            int lo_b = 0, hi_b = p.b;           // invariant: pre[lo_b] <= q < pre[hi_b]
-            while (hi_b - lo_b > 1) {
-                const int mid = (lo_b + hi_b) >> 1;
-                if (pre[mid] <= q) lo_b = mid; else hi_b = mid;
-            }
-            b = lo_b;
-            idx = q - pre[b];
-        } else {
-            const int per_b = macro ? kp.dec_sa : kp.dec_sb;
-            hk = t % p.h_k; idx = (t / p.h_k) % per_b; b = t / (p.h_k * per_b);
-        }
-        decode_item<T, D, true, APPEND, STREAM>(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
-    }
-    if (threadIdx.x == 0) {
-        const int gone = __hip_atomic_fetch_add(kp.work_counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (gone == (int)gridDim.x - 1) {     // every workgroup has drawn its last ticket
-            __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(kp.work_counter + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    for_each_ticket(kp, [&](int hk, int b, int slot, int mode, int idx) {
+        decode_item<T, D, true, APPEND, STREAM>(kp, smem, hk, b, slot, mode, idx);
+    });
 }
 
 // (the kernel is a template argument, not a function argument: the once-per-device flag inside

@@ -39,31 +39,19 @@ struct PrefillCfg {
     static_assert(RB == 1, "one 32-row block per wave");
 };
 
-// STREAM: K and V tiles are fetched with non-temporal loads -- for launches in which every K/V row is read by
-// exactly one workgroup (one row block per kv head, all of its q heads in it) and the caches are too large to
-// stay in the memory-side cache anyway (+5-8 % there; see decode_item in fa_decode.hip).
-template <typename T, int D, int RB, int BN, int MINW, bool SPLIT, bool DROPOUT = false, bool STREAM = false>
-__global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
+// One work item: the row block mb of q head hk * G + g of batch entry b over a key range -- all visible keys
+// (SPLIT = false), or those of item (mode, idx) of the split schedule, written as partial `split` (item_key_range).
+template <typename T, int D, int RB, int BN, bool SPLIT, bool DROPOUT, bool STREAM>
+FA_DEV void prefill_item(const KParams& kp, char* smem, const int hk, const int b, const int g, const int mb,
+                         const int split, const int mode, const int idx) {
     typedef PrefillCfg<T, D, RB, BN> C;
     typedef typename Elem<T>::v8 v8;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
     const fa_fwd_params& p = kp.p;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int l32 = lane & 31, hh = lane >> 5;
-
-    // ---- work decode: whole (batch, kv head) streams go to one XCD (block ids are dealt round-robin
-    // over the 8 XCDs), so that workgroups sharing a K/V stream share an L2; see xcd_stream_unit.
     const int G = p.h / p.h_k;
-    const int S = SPLIT ? kp.num_splits : 1;
-    uint32_t unit;
-    int hk, b;
-    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
-                         (uint32_t)(S * G * kp.num_m_blocks), (kp.has_left || kp.has_right) ? 32u * MINW : 0u, (uint32_t)(S * G), unit, hk, b)) return;
-    const int split = (int)(unit % (uint32_t)S); unit /= (uint32_t)S;
-    const int g = (int)(unit % (uint32_t)G);
-    const int mb = kp.num_m_blocks - 1 - (int)(unit / (uint32_t)G);
     const int head = hk * G + g;
 
     const SeqInfo si = seq_info(p, b);
@@ -82,9 +70,10 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     int t_lo = n_lo / BN;
     int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
     if (SPLIT) {
-        const int s_lo = split * (kp.split_len / BN);
-        t_lo = max(t_lo, s_lo);
-        t_hi = min(t_hi, s_lo + kp.split_len / BN);
+        int c_lo, c_hi;      // multiples of BN (the planner's chunk and piece lengths are)
+        item_key_range(kp, mode, idx, si.sk, c_lo, c_hi);
+        t_lo = max(t_lo, c_lo / BN);
+        t_hi = min(t_hi, c_hi / BN);
     }
 
     const T* __restrict__ qg = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)head * p.q_head_stride;
@@ -325,6 +314,40 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     }
 }
 
+// STREAM: K and V tiles are fetched with non-temporal loads -- for launches in which every K/V row is read by
+// exactly one workgroup (one row block per kv head, all of its q heads in it) and the caches are too large to
+// stay in the memory-side cache anyway (+5-8 % there; see decode_item in fa_decode.hip).
+template <typename T, int D, int RB, int BN, int MINW, bool SPLIT, bool DROPOUT = false, bool STREAM = false>
+__global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const fa_fwd_params& p = kp.p;
+    // ---- work decode: whole (batch, kv head) streams go to one XCD (block ids are dealt round-robin
+    // over the 8 XCDs), so that workgroups sharing a K/V stream share an L2; see xcd_stream_unit.
+    const int G = p.h / p.h_k;
+    const int S = SPLIT ? kp.num_splits : 1;
+    uint32_t unit;
+    int hk, b;
+    if (!xcd_stream_unit(xcd_strided(p.cu_seqlens_q != nullptr, p.b, p.h_k), (uint32_t)p.b, (uint32_t)p.h_k,
+                         (uint32_t)(S * G * kp.num_m_blocks), (kp.has_left || kp.has_right) ? 32u * MINW : 0u, (uint32_t)(S * G), unit, hk, b)) return;
+    const int split = (int)(unit % (uint32_t)S); unit /= (uint32_t)S;
+    const int g = (int)(unit % (uint32_t)G);
+    const int mb = kp.num_m_blocks - 1 - (int)(unit / (uint32_t)G);
+    prefill_item<T, D, RB, BN, SPLIT, DROPOUT, STREAM>(kp, smem, hk, b, g, mb, split, kChunk, split);
+}
+
+// One row block per (batch, kv head) -- a few query positions, the grouped q heads of a kv head as rows -- over
+// a cache whose lengths only the device knows: the persistent two-pass schedule of the decode kernel
+// (for_each_ticket), here with this kernel's tiles.  A plan cut for the capacity of the cache leaves the
+// workgroups of short sequences empty and those of the longest ones alone at the end; the tickets hand out
+// only chunks that hold keys, the ragged remainders last and in small pieces.
+template <typename T, int D, int RB, int BN, int MINW, bool STREAM>
+__global__ void __launch_bounds__(256, MINW) prefill_persistent_kernel(const KParams kp) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    for_each_ticket(kp, [&](int hk, int b, int slot, int mode, int idx) {
+        prefill_item<T, D, RB, BN, true, false, STREAM>(kp, smem, hk, b, 0, 0, slot, mode, idx);
+    });
+}
+
 template <typename T, int D, int RB, int BN, int MINW>
 int launch_prefill(KParams kp, hipStream_t stream) {
     typedef PrefillCfg<T, D, RB, BN> C;
@@ -337,6 +360,25 @@ int launch_prefill(KParams kp, hipStream_t stream) {
     if (nblocks == 0) return -2;
     dim3 grid((unsigned)nblocks), block(C::kThreads);
     hipError_t e;
+    if (kp.dec_persistent) {
+        // (the planner asks for this only with one row block per kv head, no grouped heads left and no dropout)
+        if (kp.num_m_blocks != 1 || kp.p.h != kp.p.h_k || !split || kp.p.p_dropout > 0.f) return -3;
+        const int64_t items = (int64_t)kp.p.b * (kp.dec_sa + kp.dec_sb) * kp.p.h_k;
+        const int64_t resident = 256 * MINW;                     // workgroups the 256 CUs hold at once
+        const dim3 pgrid((unsigned)std::min(items, resident));
+        if (kp.stream_kv) {
+            auto kern = prefill_persistent_kernel<T, D, RB, BN, MINW, true>;
+            e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
+            if (e != hipSuccess) return (int)e;
+            hipLaunchKernelGGL(kern, pgrid, block, C::SMEM, stream, kp);
+        } else {
+            auto kern = prefill_persistent_kernel<T, D, RB, BN, MINW, false>;
+            e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
+            if (e != hipSuccess) return (int)e;
+            hipLaunchKernelGGL(kern, pgrid, block, C::SMEM, stream, kp);
+        }
+        return (int)hipGetLastError();
+    }
     const bool one_reader = kp.stream_kv && kp.num_m_blocks == 1 && kp.p.h == kp.p.h_k && !(kp.p.p_dropout > 0.f);
     if (split && one_reader) {
         auto kern = prefill_kernel<T, D, RB, BN, MINW, true, false, true>;

@@ -179,23 +179,44 @@ def test_single_query_with_more_than_16_grouped_heads(h, hk, d, mode):
         assert orc.tolerance_ok(o2.cpu(), o_ref[2:3], o_pt[2:3], 3.0, 1e-5)[0]
 
 
-@pytest.mark.parametrize("num_splits", [0, 1])
+def _planned_splits(nat, b, h, hk, sq, cap, d):
+    """partial slots the library plans for a kv-cache call with per-batch cache lengths and automatic splits"""
+    import ctypes
+    p = nat.FaFwdParams()
+    p.b, p.h, p.h_k, p.seqlen_q, p.seqlen_k, p.d, p.dtype = b, h, hk, sq, cap, d, 1
+    p.is_seqlens_k_cumulative = 0
+    p.softmax_scale = d ** -0.5
+    p.window_left = p.window_right = -1
+    for name in ("q", "k", "v", "o", "softmax_lse", "work_counter", "cu_seqlens_k"):
+        setattr(p, name, 256)          # non-null placeholders: planning reads no memory
+    p.q_head_stride = p.o_head_stride = d
+    p.work_counter_len = 2
+    n = ctypes.c_int32(0)
+    assert nat.lib.fa_plan_splits(ctypes.byref(p), 2, ctypes.byref(n)) == 0
+    return n.value
+
+
+@pytest.mark.parametrize("num_splits,cap", [(0, 3000), (1, 3000), (0, 9000)])
 @pytest.mark.parametrize("mode", ["plain", "causal", "append_rotary", "window_right", "window_left", "local"])
 @pytest.mark.parametrize("sq,h,hk,d", [(4, 64, 8, 128), (2, 32, 2, 64), (5, 12, 3, 128), (16, 8, 4, 96), (33, 6, 2, 128),
                                         (100, 4, 2, 64), (3, 48, 1, 256), (127, 2, 1, 128)])
-def test_few_query_positions_with_grouped_heads(sq, h, hk, d, mode, num_splits):
+def test_few_query_positions_with_grouped_heads(sq, h, hk, d, mode, num_splits, cap):
     """2..127 query positions with grouped q heads and more than 16 (position, head) rows per kv head (a draft of
     several tokens checked at once, a short chunk of a prompt): the library lays those rows out as the rows of
     one problem per kv head, so K/V are fetched once and not once per q head.  Masks and rotary positions follow
-    the position of a row, softmax_lse keeps its (batch, head, position) layout."""
-    _say("few positions, grouped heads", sq, h, hk, d, mode, num_splits)
+    the position of a row, softmax_lse keeps its (batch, head, position) layout.  Caches of 9000 rows take the
+    ticket-scheduled form of the tiled kernel (chunks of 2048 keys, remainders in pieces of 1024: lengths with
+    complete chunks and a remainder, less than a chunk, a whole number of chunks)."""
+    _say("few positions, grouped heads", sq, h, hk, d, mode, num_splits, cap)
     nat = _nat()
-    dtype, cap, b = torch.bfloat16, 3000, 3
+    dtype, b = torch.bfloat16, 3
+    if cap == 9000 and sq * (h // hk) <= 128:      # (more rows than one row block holds: the plain split form)
+        assert _planned_splits(nat, b, h, hk, sq, cap, d) == 5 + 2     # 5 chunk slots + 2 remainder slots
     torch.manual_seed(sq * 7 + h)
     kc = torch.randn(b, cap, hk, d, dtype=dtype)
     vc = torch.randn(b, cap, hk, d, dtype=dtype)
     q = torch.randn(b, sq, h, d, dtype=dtype)
-    lens = torch.tensor([2500, max(sq, 37), 1203], dtype=torch.int32)
+    lens = torch.tensor([2500, max(sq, 37), 1203] if cap == 3000 else [8700, max(sq, 37), 4096 + sq], dtype=torch.int32)
     kn = vn = cos = sin = None
     causal, wl, wr = mode in ("causal", "append_rotary"), -1, -1
     if mode == "append_rotary":
@@ -229,3 +250,36 @@ def test_few_query_positions_with_grouped_heads(sq, h, hk, d, mode, num_splits):
         wide[:, :, 1:h + 1] = q[0:1]
         o2 = _fa_func()(wide.to(DEV)[:, :, 1:h + 1], kc[0:1, :L].to(DEV), vc[0:1, :L].to(DEV), causal=causal, window_size=(wl, wr))
         assert orc.tolerance_ok(o2.cpu(), o_ref[0:1], o_pt[0:1], 3.0, 1e-5)[0]
+
+
+@pytest.mark.parametrize("num_splits", [0, 1])
+@pytest.mark.parametrize("sq,h,hk,b,cap", [(4, 64, 8, 16, 16384), (1, 24, 1, 64, 32768), (40, 2, 2, 16, 65536)])
+def test_caches_of_a_gibibyte_take_the_streaming_tile_loop(sq, h, hk, b, cap, num_splits):
+    """K/V caches of 1 GiB and more whose rows one workgroup reads (one row block per kv head) are fetched with
+    non-temporal loads, requested two tiles ahead: the key loop of that variant has its own prologue and runs
+    two tiles per trip.  Lengths of 1, 2, 3 and 4 tiles, an odd and an even long one, and an empty entry; a few
+    batch entries are checked against the oracle, out and softmax_lse, with and without split keys."""
+    _say("gibibyte caches", sq, h, hk, b, cap, num_splits)
+    nat = _nat()
+    dtype, d = torch.bfloat16, 128
+    assert 4 * b * cap * hk * d >= 1 << 30
+    torch.manual_seed(sq + 11 * num_splits)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, sq, h, d, dtype=dtype)
+    lens = torch.randint(cap // 4, cap - sq, (b,), dtype=torch.int32)
+    picks = [0, 1, 2, 3, 4, 5, 6, b - 1]
+    lens[:7] = torch.tensor([max(sq, 40), 100, 130, 250, cap - 1, cap - 64 - 7, 0 if sq == 1 else sq], dtype=torch.int32)
+    out, lse = nat.fwd_kvcache(q.to(DEV), kc.to(DEV), vc.to(DEV), None, None, lens.to(DEV), None, None, None, None, d ** -0.5,
+                               True, -1, -1, True, num_splits)
+    out, lse = out.cpu(), lse.cpu()
+    assert torch.isfinite(out.float()).all()
+    for i in picks:
+        sl = slice(i, i + 1)
+        o_ref, l_ref, _, _ = orc.kvcache_forward(q[sl], kc[sl], vc[sl], None, None, None, None, lens[sl], causal=True)
+        o_pt, _, _, _ = orc.kvcache_forward(q[sl], kc[sl], vc[sl], None, None, None, None, lens[sl], causal=True,
+                                            upcast=False, reorder_ops=True)
+        ok, err, bound = orc.tolerance_ok(out[sl], o_ref, o_pt, 3.0, 1e-5)
+        _say("   entry %d length %d: out err %.3e bound %.3e" % (i, int(lens[i]), err, bound))
+        assert ok
+        assert orc.lse_ok(lse[sl], l_ref, 1e-3)[0]
