@@ -364,12 +364,14 @@ def bench_decode_variants(steps, warmup):
     """Decoding shapes beside config 5 that take other paths of the library: four query positions at once on the
     config 5 caches (a draft of four tokens: 32 (position, head) rows per kv head, laid out as the rows of one
     tiled problem per kv head) and one position on a multi-query cache (32 q heads on 1 kv head: the grouped
-    heads become the rows).  Bytes: the cached K/V rows the masks let the queries see, once."""
+    heads become the rows).  Both run the tiled kernel under the ticket schedule (chunks that hold keys, drawn
+    from a counter).  Bytes: the cached K/V rows the masks let the queries see, once."""
     import torch
     import flash_attn
     res = {}
-    for name, (b, cap, hk, h, d, sq, lo) in (("four_positions_gqa8", (64, 32768, 8, 64, 128, 4, 1024)),
-                                                ("one_position_mqa32", (16, 65536, 1, 32, 128, 1, 30000))):
+    for name, (b, cap, hk, h, d, sq, lo, kern) in (
+            ("four_positions_gqa8", (64, 32768, 8, 64, 128, 4, 1024, "fa::prefill_persistent_kernel<bf16,128,stream>")),
+            ("one_position_mqa32", (16, 65536, 1, 32, 128, 1, 30000, "fa::prefill_persistent_kernel<bf16,128>"))):
         torch.manual_seed(0)
         k_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
         v_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
@@ -383,7 +385,7 @@ def bench_decode_variants(steps, warmup):
         res[name] = {"ms": ms, "ms_min": tm.ms_min, "gb_per_s": gbs,
                      "workload": "flash_attn_with_kvcache bf16 b%d cache(%d,%d,%d,%d) hq%d seqlen_q %d causal" % (b, b, cap, hk, d, h, sq),
                      "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                                  "traffic": None, "kernel": "fa::prefill_kernel<bf16,128,split> + fa::combine_kernel", "bytes_per_launch": algo_bytes}}
+                                  "traffic": None, "kernel": kern + " + fa::combine_kernel", "bytes_per_launch": algo_bytes}}
         del k_cache, v_cache
     return res
 

@@ -42,13 +42,12 @@ struct PrefillCfg {
 // One work item: the row block mb of q head hk * G + g of batch entry b over a key range -- all visible keys
 // (SPLIT = false), or those of item (mode, idx) of the split schedule, written as partial `split` (item_key_range).
 template <typename T, int D, int RB, int BN, bool SPLIT, bool DROPOUT, bool STREAM>
-FA_DEV void prefill_item(const KParams& kp, char* smem, const int hk, const int b, const int g, const int mb,
+FA_DEV void prefill_item(const KParams& kp, char* smem, const int tid, const int hk, const int b, const int g, const int mb,
                          const int split, const int mode, const int idx) {
     typedef PrefillCfg<T, D, RB, BN> C;
     typedef typename Elem<T>::v8 v8;
     const fa_fwd_params& p = kp.p;
 
-    const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int l32 = lane & 31, hh = lane >> 5;
     const int G = p.h / p.h_k;
@@ -332,7 +331,7 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
     const int split = (int)(unit % (uint32_t)S); unit /= (uint32_t)S;
     const int g = (int)(unit % (uint32_t)G);
     const int mb = kp.num_m_blocks - 1 - (int)(unit / (uint32_t)G);
-    prefill_item<T, D, RB, BN, SPLIT, DROPOUT, STREAM>(kp, smem, hk, b, g, mb, split, kChunk, split);
+    prefill_item<T, D, RB, BN, SPLIT, DROPOUT, STREAM>(kp, smem, (int)threadIdx.x, hk, b, g, mb, split, kChunk, split);
 }
 
 // One row block per (batch, kv head) -- a few query positions, the grouped q heads of a kv head as rows -- over
@@ -344,7 +343,13 @@ template <typename T, int D, int RB, int BN, int MINW, bool STREAM>
 __global__ void __launch_bounds__(256, MINW) prefill_persistent_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     for_each_ticket(kp, [&](int hk, int b, int slot, int mode, int idx) {
-        prefill_item<T, D, RB, BN, true, false, STREAM>(kp, smem, hk, b, 0, 0, slot, mode, idx);
+        // The lane index is made opaque per item: what an item derives from it (row and column offsets of the
+        // tile movers, LDS offsets, Q row addresses) would otherwise be computed once before the ticket loop and
+        // kept in registers across it, which do not exist: the spills landed between the loads of the Q rows,
+        // each reload waiting for every load before it (15 us per item).
+        int tid = (int)threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        prefill_item<T, D, RB, BN, true, false, STREAM>(kp, smem, tid, hk, b, 0, 0, slot, mode, idx);
     });
 }
 
