@@ -638,13 +638,13 @@ FA_DEV void item_key_range(const KParams& kp, int mode, int idx, int hi, int& c_
     }
 }
 
-// The persistent schedule itself, for a grid of resident workgroups: calls item(kv head, batch entry, partial
-// slot, mode, idx) for this workgroup's block id and then for every ticket it draws from kp.work_counter[0]
-// until the items are used up; the last workgroup to finish puts the two counter words back to zero.  All
-// lanes of the workgroup must call it together and return from every item (it synchronises the workgroup
-// between items, so an item may use all of LDS).
-template <class F>
-FA_DEV void for_each_ticket(const KParams& kp, F&& item) {
+// The persistent schedule itself, for a grid of resident workgroups: calls Item::run(kp, smem, kv head, batch
+// entry, partial slot, mode, idx) for this workgroup's block id and then for every ticket it draws from
+// kp.work_counter[0] until the items are used up; the last workgroup to finish puts the two counter words back
+// to zero.  All lanes of the workgroup must call it together and return from every item (it synchronises the
+// workgroup between items, so an item may use all of the dynamic LDS, `smem`).
+template <class Item>
+FA_DEV void for_each_ticket(const KParams& kp, char* smem) {
     __shared__ int s_ticket;
     // compact schedule: s_pm[b] / s_ps[b] = slots with keys (complete chunks / remainder pieces) of the batch
     // entries before b; tickets then number only those slots, batch entry by batch entry, kv heads fastest
@@ -711,7 +711,7 @@ FA_DEV void for_each_ticket(const KParams& kp, F&& item) {
             const int per_b = macro ? kp.dec_sa : kp.dec_sb;
             hk = t % p.h_k; idx = (t / p.h_k) % per_b; b = t / (p.h_k * per_b);
         }
-        item(hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
+        Item::run(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
     }
     if (threadIdx.x == 0) {
         const int gone = __hip_atomic_fetch_add(kp.work_counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -366,12 +366,17 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 // L2, every stream completes in the remainder pass at the very end of the launch, and 512 latency-bound
 // merges there cost 2-3 x the stand-alone merge kernel; cache write-back / invalidation fences at device scope
 // around every item instead cost three times the whole kernel).
+// (what for_each_ticket calls per ticket)
+template <typename T, int D, bool APPEND, bool STREAM>
+struct DecodeTicketItem {
+    static FA_DEV void run(const KParams& kp, char* smem, int hk, int b, int slot, int mode, int idx) {
+        decode_item<T, D, true, APPEND, STREAM>(kp, smem, hk, b, slot, mode, idx);
+    }
+};
 template <typename T, int D, bool APPEND, bool STREAM>
 __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_persistent_kernel(const KParams kp) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    for_each_ticket(kp, [&](int hk, int b, int slot, int mode, int idx) {
-        decode_item<T, D, true, APPEND, STREAM>(kp, smem, hk, b, slot, mode, idx);
-    });
+    for_each_ticket<DecodeTicketItem<T, D, APPEND, STREAM>>(kp, smem);
 }
 
 // (the kernel is a template argument, not a function argument: the once-per-device flag inside

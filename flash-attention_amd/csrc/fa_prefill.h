@@ -339,10 +339,10 @@ __global__ void __launch_bounds__(256, MINW) prefill_kernel(const KParams kp) {
 // (for_each_ticket), here with this kernel's tiles.  A plan cut for the capacity of the cache leaves the
 // workgroups of short sequences empty and those of the longest ones alone at the end; the tickets hand out
 // only chunks that hold keys, the ragged remainders last and in small pieces.
-template <typename T, int D, int RB, int BN, int MINW, bool STREAM>
-__global__ void __launch_bounds__(256, MINW) prefill_persistent_kernel(const KParams kp) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    for_each_ticket(kp, [&](int hk, int b, int slot, int mode, int idx) {
+// (PrefillTicketItem: what for_each_ticket calls per ticket)
+template <typename T, int D, int RB, int BN, bool STREAM>
+struct PrefillTicketItem {
+    static FA_DEV void run(const KParams& kp, char* smem, int hk, int b, int slot, int mode, int idx) {
         // The lane index is made opaque per item: what an item derives from it (row and column offsets of the
         // tile movers, LDS offsets, Q row addresses) would otherwise be computed once before the ticket loop and
         // kept in registers across it, which do not exist: the spills landed between the loads of the Q rows,
@@ -350,7 +350,12 @@ __global__ void __launch_bounds__(256, MINW) prefill_persistent_kernel(const KPa
         int tid = (int)threadIdx.x;
         asm volatile("" : "+v"(tid));
         prefill_item<T, D, RB, BN, true, false, STREAM>(kp, smem, tid, hk, b, 0, 0, slot, mode, idx);
-    });
+    }
+};
+template <typename T, int D, int RB, int BN, int MINW, bool STREAM>
+__global__ void __launch_bounds__(256, MINW) prefill_persistent_kernel(const KParams kp) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    for_each_ticket<PrefillTicketItem<T, D, RB, BN, STREAM>>(kp, smem);
 }
 
 template <typename T, int D, int RB, int BN, int MINW>
