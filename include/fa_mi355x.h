@@ -65,8 +65,11 @@ typedef struct fa_fwd_params {
                                        When set, split-KV decode launches run as a persistent kernel whose
                                        workgroups draw (batch, kv head, key chunk) items from a ticket and
                                        whose item that reaches the new rows appends them to the cache (no
-                                       append launch).  Words past the first FA_WORK_COUNTER_WORDS are
-                                       scratch with no required contents: when there are at least
+                                       append launch); fa_fwd_kvcache launches of a few query positions (or one
+                                       position on more than 16 grouped heads) over per-batch cache lengths run
+                                       the tiled kernel under the same ticket schedule.  Words past the first
+                                       FA_WORK_COUNTER_WORDS are scratch with no required contents: when there
+                                       are at least
                                        fa_work_list_words(p) words, fa_varlen_fwd first builds its work
                                        list there on the device (sequences by falling length, no empty
                                        workgroups between working ones).  Must not be shared by calls
@@ -113,7 +116,7 @@ typedef struct fa_fwd_params {
     int32_t reserved0;
 } fa_fwd_params;
 
-/* words the persistent decode kernel needs behind work_counter: ticket, exit count */
+/* words the ticket-scheduled kernels need behind work_counter: ticket, exit count */
 #define FA_WORK_COUNTER_WORDS 2
 
 /*
