@@ -36,6 +36,12 @@ static const int kNumCU = 256;   // MI355X
 #ifndef FA_DEC_SB
 #define FA_DEC_SB 8
 #endif
+#ifndef FA_TILE_SLOTS
+#define FA_TILE_SLOTS 4096      // chunk slots per launch of the ticket-scheduled tiled kernel
+#endif
+#ifndef FA_TILE_MINLEN
+#define FA_TILE_MINLEN 2048     // its shortest chunk (keys)
+#endif
 #ifndef FA_DEC_MINLEN
 #define FA_DEC_MINLEN 512       // shortest chunk of the decode kernel (keys) once the launch fills the CUs
 #endif
@@ -141,7 +147,7 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     int64_t tile_chunk = 0;
     if (!dec && allow_split && p.num_splits == 0 && p.p_dropout == 0.f && counters_ok(p) && !p.cu_seqlens_q && p.cu_seqlens_k &&
         !p.is_seqlens_k_cumulative && p.seqlen_q <= prefill_block_m(db) && p.h == p.h_k) {
-        const int64_t len = (std::max<int64_t>(2048, (int64_t)sk * wgs / FA_DEC_SLOTS_P) + 511) / 512 * 512;
+        const int64_t len = (std::max<int64_t>(FA_TILE_MINLEN, (int64_t)sk * wgs / FA_TILE_SLOTS) + 511) / 512 * 512;
         // (launches that fill the CUs without a split keep the plain form up to 8192 keys: two or three chunks per
         // sequence do not pay for the merge)
         if (sk >= 2 * len && (wgs < kNumCU || sk >= 8192)) tile_chunk = len;
