@@ -54,6 +54,8 @@ def test_no_alloc_entry_matches_kvcache_entry_twice():
     _case(nat, 3, 5000, 16, 2, 128, [4999, 0, 1234], seed=2)
     _say("no_alloc third call: 2 query rows, unsplit")
     _case(nat, 2, 300, 4, 2, 64, [100, 299 - 2], seqlen_q=2, seed=3)
+    _say("no_alloc fourth call: 4 query positions x 8 grouped heads (tiled kernel under the ticket schedule + merge)")
+    _case(nat, 3, 9000, 32, 4, 128, [8700, 40, 4100], seqlen_q=4, seed=4)
 
 
 def test_no_alloc_entry_rejects_what_does_not_fit():
