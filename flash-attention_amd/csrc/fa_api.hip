@@ -36,6 +36,9 @@ static const int kNumCU = 256;   // MI355X
 #ifndef FA_DEC_SB
 #define FA_DEC_SB 8
 #endif
+#ifndef FA_SPLIT_BELOW
+#define FA_SPLIT_BELOW 256      // row blocks x heads x batch below which the tiled kernel's keys are split
+#endif
 #ifndef FA_TILE_SLOTS
 #define FA_TILE_SLOTS 4096      // chunk slots per launch of the ticket-scheduled tiled kernel
 #endif
@@ -136,7 +139,7 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     SplitPlan r;
     fa_fwd_params p = p_in;
     // what runs is the problem with the grouped heads as rows (no change when it already is)
-    if (!groups_as_rows(p)) positions_and_groups_as_rows(p, nullptr, nullptr);
+    const bool packed = !groups_as_rows(p) && positions_and_groups_as_rows(p, nullptr, nullptr) > 0;
     const int sk = p.seqlen_k;
     const int db = bucket(p.d);
     const bool dec = use_decode_kernel(p);
@@ -182,7 +185,18 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
             } else if (tile_chunk) {
                 splits = (int)((sk + tile_chunk - 1) / tile_chunk);
             } else {
-                if (wgs < kNumCU) {
+                // Launches that take the pipelined / ping-pong kernels when left whole (fa_prefill_inst.hip) are split
+                // later than the others: those kernels are 1.3-1.5 x (head dim 256: 2 x) as fast per workgroup as
+                // the general kernel the split form runs, and the split adds the merge.  Measured, 128-511 rows,
+                // 16-192 row blocks, 512-32768 keys: whole wins from 64 row blocks on up to 1024 keys (2048 at head dim 64; +17-58 %),
+                // from 96 up to 2048 (+26-63 %), from 192 on longer keys (+2-150 %; at 128: -17..-36 %); head dim
+                // 256 from 64 up to 2048 keys and from 96 beyond (+7-28 %; at 64: -28..-43 %).
+                int64_t split_below = FA_SPLIT_BELOW;
+                if (!packed && !p.rotary_cos && p.seqlen_q >= prefill_long_rows(db)) {
+                    if (db > 128) split_below = sk <= 2048 ? 64 : 96;
+                    else split_below = sk <= (db <= 64 ? 2048 : 1024) ? 64 : sk <= 2048 ? 96 : 192;
+                }
+                if (wgs < split_below) {
                     const int64_t want = (2 * kNumCU + wgs - 1) / wgs;
                     splits = (int)std::min<int64_t>(want, (sk + 255) / 256);
                 }

@@ -15,6 +15,11 @@ FA_DECL_PREFILL(launch_prefill_fp16_256)
 
 int prefill_block_n(int d_bucket);   // key-tile length of the prefill kernel for a bucket
 int prefill_block_m(int d_bucket);
+// Query rows from which an unsplit launch without q rotary takes the pipelined / ping-pong kernels instead of
+// the general tiled kernel (measured on 32..511 rows x 128..16384 keys, bf16, with and without a causal mask:
+// head dims 64 and 128 +15-45 % from 128 rows on, 0..+28 % at 100-127 rows, -9..+14 % at 64 rows; head dim 256
+// +25-57 % from 32 rows on, +50-100 % from 128).
+inline int prefill_long_rows(int d_bucket) { return d_bucket > 128 ? 32 : 96; }
 
 int launch_decode(const KParams& kp, hipStream_t stream);      // small-q split-KV kernel
 int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials

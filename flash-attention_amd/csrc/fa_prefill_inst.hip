@@ -4,10 +4,6 @@
 #include "fa_prefill_il.h"
 #include "fa_launch.h"
 
-#ifndef FA_LONG_ROWS
-#define FA_LONG_ROWS 128     // query rows from which the long-sequence kernels take over
-#endif
-
 namespace fa {
 #if FA_T_BF16
 typedef __bf16 InstT;
@@ -24,11 +20,11 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     // Long query sequences (measured cross-overs on MI355X):
     //  * head dim 128, from 2048 keys on (causal / windowed) or beyond 768 (full): the 8-wave ping-pong
     //    kernel, 256 rows per workgroup, each K/V tile fetched once per 256 rows;
-    //  * otherwise from 512 query rows on: the software-pipelined kernel, two independent
+    //  * otherwise (from prefill_long_rows query rows on): the software-pipelined kernel, two independent
     //    128-row workgroups per CU, whose start-up and output phases overlap.
     // Shorter sequences, split key ranges, q rotary and rows that stand for (position, grouped head) pairs take
     // the general 4-wave kernel.
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= FA_LONG_ROWS && kp.pack_g <= 1) {
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= prefill_long_rows(FA_D) && kp.pack_g <= 1) {
         const bool masked = kp.has_right || kp.has_left;
         const bool long_keys = kp.p.seqlen_k >= (masked ? 2048 : 769);
         // When the 256-row blocks of the ping-pong kernel would occupy no more than half of the 256
@@ -45,7 +41,7 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
 #else
     // head dim 129..256: one wave per SIMD with the whole head dimension, or pairs of waves that split it
     // (with dropout); fa_prefill_il.h
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= FA_LONG_ROWS && kp.pack_g <= 1) return launch_prefill_il_256<InstT>(kp, stream);
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= prefill_long_rows(FA_D) && kp.pack_g <= 1) return launch_prefill_il_256<InstT>(kp, stream);
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }
