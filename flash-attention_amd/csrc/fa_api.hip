@@ -150,7 +150,11 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     int64_t tile_chunk = 0;
     if (!dec && allow_split && p.num_splits == 0 && p.p_dropout == 0.f && counters_ok(p) && !p.cu_seqlens_q && p.cu_seqlens_k &&
         !p.is_seqlens_k_cumulative && p.seqlen_q <= prefill_block_m(db) && p.h == p.h_k) {
-        const int64_t len = (std::max<int64_t>(FA_TILE_MINLEN, (int64_t)sk * wgs / FA_TILE_SLOTS) + 511) / 512 * 512;
+        // (launches too small to give every resident workgroup a chunk of FA_TILE_MINLEN keys take shorter ones,
+        // down to 512: one sequence of 16k keys on 8 kv heads is 64 chunks of 2048 keys, a quarter of the CUs)
+        const int64_t fill = ((int64_t)sk * wgs / (2 * kNumCU) + 511) / 512 * 512;
+        const int64_t minlen = std::min<int64_t>(FA_TILE_MINLEN, std::max<int64_t>(512, fill));
+        const int64_t len = (std::max<int64_t>(minlen, (int64_t)sk * wgs / FA_TILE_SLOTS) + 511) / 512 * 512;
         // (launches that fill the CUs without a split keep the plain form up to 8192 keys: two or three chunks per
         // sequence do not pay for the merge)
         if (sk >= 2 * len && (wgs < kNumCU || sk >= 8192)) tile_chunk = len;
@@ -224,7 +228,7 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     // write: about what 160 keys take -- and its pieces stay at 1024 keys or more.)
     // Halves, quarters or eighths of a multiple of 512: whole tiles.
     const int sb = tile_chunk ? (len < 4096 ? 2 : len < 8192 ? 4 : FA_DEC_SB) : len < 2048 ? 2 : len < 4096 ? 4 : FA_DEC_SB;
-    if ((dec || tile_chunk) && automatic && splits > 1 && counters_ok(p) && len >= 1024 && splits + sb <= FA_MAX_SPLITS) {
+    if ((dec || tile_chunk) && automatic && splits > 1 && counters_ok(p) && len >= (dec ? 1024 : 512) && splits + sb <= FA_MAX_SPLITS) {
         r.persistent = 1;
         r.sa = splits;
         r.sb = sb;

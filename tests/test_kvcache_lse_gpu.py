@@ -205,13 +205,13 @@ def test_few_query_positions_with_grouped_heads(sq, h, hk, d, mode, num_splits, 
     several tokens checked at once, a short chunk of a prompt): the library lays those rows out as the rows of
     one problem per kv head, so K/V are fetched once and not once per q head.  Masks and rotary positions follow
     the position of a row, softmax_lse keeps its (batch, head, position) layout.  Caches of 9000 rows take the
-    ticket-scheduled form of the tiled kernel (chunks of 2048 keys, remainders in pieces of 1024: lengths with
+    ticket-scheduled form of the tiled kernel (a launch this small: chunks of 512 keys, remainders in pieces of 256; lengths with
     complete chunks and a remainder, less than a chunk, a whole number of chunks)."""
     _say("few positions, grouped heads", sq, h, hk, d, mode, num_splits, cap)
     nat = _nat()
     dtype, b = torch.bfloat16, 3
     if cap == 9000 and sq * (h // hk) <= 128:      # (more rows than one row block holds: the plain split form)
-        assert _planned_splits(nat, b, h, hk, sq, cap, d) == 5 + 2     # 5 chunk slots + 2 remainder slots
+        assert _planned_splits(nat, b, h, hk, sq, cap, d) == 18 + 2     # 18 chunk slots + 2 remainder slots
     torch.manual_seed(sq * 7 + h)
     kc = torch.randn(b, cap, hk, d, dtype=dtype)
     vc = torch.randn(b, cap, hk, d, dtype=dtype)
