@@ -182,6 +182,51 @@ int launch_append_kv(const KParams& kp, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// q rows of a kv-cache call rotated to their positions and written to the rows of the output tensor -- what the
+// general tiled kernel does while it loads its Q fragments (prefill_item, fa_prefill.h; same arithmetic: fp32,
+// rounded once; the position stops at the last row the table is known to cover), as a pass of its own for the
+// launches that then take the pipelined / ping-pong kernels, which read Q without rotating it.  The attention
+// kernel afterwards reads its Q rows from `o` and writes its results over them: a workgroup reads only the rows
+// it writes, and all of them before it writes any.
+template <typename T>
+__global__ void __launch_bounds__(256) rotate_q_kernel(const KParams kp) {
+    const fa_fwd_params& p = kp.p;
+    const int cpr = p.d / 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.b * p.seqlen_q * p.h * cpr) return;
+    const int c = (int)(idx % cpr);
+    int64_t r = idx / cpr;
+    const int head = (int)(r % p.h); r /= p.h;
+    const int i = (int)(r % p.seqlen_q);
+    const int b = (int)(r / p.seqlen_q);
+    const SeqInfo si = seq_info(p, b);
+    const T* qrow = reinterpret_cast<const T*>(p.q) + si.q_off + (int64_t)i * p.q_row_stride + (int64_t)head * p.q_head_stride;
+    T* orow = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)i * p.o_row_stride + (int64_t)head * p.o_head_stride;
+    const int d0 = c * 8;
+    u32x4 raw = ld_global16(qrow + d0);
+    if (d0 < p.rotary_dim) {
+        // (without a mask every row is rotated to the position of the first new token)
+        const int pos = min(si.sk_cache + ((kp.has_left || kp.has_right) ? i : 0), p.seqlen_k - 1);
+        const T* cr = reinterpret_cast<const T*>(p.rotary_cos) + (int64_t)pos * (p.rotary_dim / 2);
+        const T* sr = reinterpret_cast<const T*>(p.rotary_sin) + (int64_t)pos * (p.rotary_dim / 2);
+        float x[8];
+        unpack8<T>(raw, x);
+        rotary8<T>(x, qrow, cr, sr, d0, p.rotary_dim, p.is_rotary_interleaved != 0);
+        raw = pack8<T>(x);
+    }
+    st_global16(orow + d0, raw);
+}
+
+int launch_rotate_q(const KParams& kp, hipStream_t stream) {
+    const fa_fwd_params& p = kp.p;
+    const int64_t total = (int64_t)p.b * p.seqlen_q * p.h * (p.d / 8);
+    if (total == 0) return 0;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (p.dtype == FA_DTYPE_BF16) hipLaunchKernelGGL(rotate_q_kernel<__bf16>, grid, block, 0, stream, kp);
+    else hipLaunchKernelGGL(rotate_q_kernel<_Float16>, grid, block, 0, stream, kp);
+    return (int)hipGetLastError();
+}
+
 // Testing aid behind return_softmax (the reference's S_dmask, csrc/flash_attn/flash_api.cpp:351-357):
 // s_dmask[b, h, i, j] = exp(scale q_i . k_j - lse_i), negated where dropout removed the entry, 0 where
 // the mask hides it or outside (seqlen_q, seqlen_k).  Runs after the attention kernel, so lse is

@@ -25,6 +25,7 @@ int launch_decode(const KParams& kp, hipStream_t stream);      // small-q split-
 int launch_combine(const KParams& kp, hipStream_t stream);     // merge of split partials
 // k_new/v_new (+rotary) -> cache
 int launch_append_kv(const KParams& kp, hipStream_t stream);
+int launch_rotate_q(const KParams& kp, hipStream_t stream);     // q rows rotated to their positions -> rows of o
 int launch_attn_probs(const KParams& kp, hipStream_t stream);  // s_dmask: signed softmax probabilities (testing)
 int launch_rotary(const fa_rotary_params& p, hipStream_t stream);   // standalone rotary embedding
 // Packed batches: builds the work list of a forward launch of `nblocks` workgroups with row blocks of

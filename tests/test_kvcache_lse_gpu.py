@@ -283,3 +283,40 @@ def test_caches_of_a_gibibyte_take_the_streaming_tile_loop(sq, h, hk, b, cap, nu
         _say("   entry %d length %d: out err %.3e bound %.3e" % (i, int(lens[i]), err, bound))
         assert ok
         assert orc.lse_ok(lse[sl], l_ref, 1e-3)[0]
+
+
+@pytest.mark.parametrize("mode", ["causal", "full", "local"])
+@pytest.mark.parametrize("inter", [False, True])
+@pytest.mark.parametrize("sq,h,hk,d,rot", [(128, 64, 8, 128, 128), (300, 32, 32, 64, 32), (97, 72, 8, 96, 64), (200, 32, 4, 256, 256)])
+def test_appended_chunk_with_rotary_on_the_long_sequence_kernels(sq, h, hk, d, rot, inter, mode):
+    """A chunk of 97..300 tokens appended with rotary to caches, in a launch that is not split (256+ row blocks):
+    the q rows are rotated into the output tensor by a pass of their own and the long-sequence kernels read them
+    from there.  Out, softmax_lse and the cache contents against the oracle; q must come back untouched."""
+    _say("appended chunk with rotary", sq, h, hk, d, rot, inter, mode)
+    nat = _nat()
+    dtype, cap, b = torch.bfloat16, 1500, 4
+    assert (sq + 127) // 128 * h * b >= 256
+    torch.manual_seed(sq + d)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, sq, h, d, dtype=dtype)
+    kn = torch.randn(b, sq, hk, d, dtype=dtype)
+    vn = torch.randn(b, sq, hk, d, dtype=dtype)
+    lens = torch.tensor([cap - sq, 0, 700, 1], dtype=torch.int32)
+    cos, sin = orc.rotary_table(cap, rot, dtype=dtype)
+    causal, wl, wr = mode == "causal", -1, -1
+    if mode == "local":
+        wl, wr = 200, 30
+    q_d, kc_d, vc_d = q.to(DEV), kc.to(DEV), vc.to(DEV)
+    out, lse = nat.fwd_kvcache(q_d, kc_d, vc_d, kn.to(DEV), vn.to(DEV), lens.to(DEV), cos.to(DEV), sin.to(DEV), None, None, d ** -0.5,
+                               causal, wl, wr, inter, 0)
+    assert torch.equal(q_d.cpu(), q)
+    kw = dict(causal=causal, window_size=(wl, wr), rotary_interleaved=inter)
+    o_ref, l_ref, k_ref, v_ref = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, **kw)
+    o_pt, _, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, upcast=False, reorder_ops=True, **kw)
+    ok, err, bound = orc.tolerance_ok(out.cpu(), o_ref, o_pt, 3.0, 1e-5)
+    _say("   out err %.3e bound %.3e" % (err, bound))
+    assert ok
+    assert orc.lse_ok(lse.cpu(), l_ref, 1e-3)[0]
+    assert torch.equal(vc_d.cpu(), v_ref)
+    assert torch.allclose(kc_d.cpu().float(), k_ref.float(), rtol=1e-3, atol=1e-3)
