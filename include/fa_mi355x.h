@@ -145,7 +145,9 @@ int fa_varlen_fwd(const fa_fwd_params *p, void *hip_stream);
  * KV-cache forward.  Replaces mha_fwd_kvcache (flash_api.cpp:1038-1279): optional append of
  * k_new/v_new at rows cache_seqlens[b] .. of cache row cache_batch_idx[b] (new keys rotated when
  * rotary tables are given, :763-852 of flash_fwd_kernel.h), q rotated on load (:854-891), then
- * attention over cache_seqlens[b] + seqlen_knew keys.  Mutates k and v in place.
+ * attention over cache_seqlens[b] + seqlen_knew keys.  Mutates k and v in place.  With rotary tables and 96 or
+ * more query rows, o may hold the rotated q rows before the results land in it: o must not overlap q partially
+ * (o == q is recognised).
  */
 int fa_fwd_kvcache(const fa_fwd_params *p, void *hip_stream);
 
