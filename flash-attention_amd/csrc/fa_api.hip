@@ -196,7 +196,7 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
                 // from 96 up to 2048 (+26-63 %), from 192 on longer keys (+2-150 %; at 128: -17..-36 %); head dim
                 // 256 from 64 up to 2048 keys and from 96 beyond (+7-28 %; at 64: -28..-43 %).
                 int64_t split_below = FA_SPLIT_BELOW;
-                if (!packed && !p.rotary_cos && p.seqlen_q >= prefill_long_rows(db)) {
+                if (!packed && p.seqlen_q >= prefill_long_rows(db)) {     // (with q rotary too: see fa_fwd_kvcache)
                     if (db > 128) split_below = sk <= 2048 ? 64 : 96;
                     else split_below = sk <= (db <= 64 ? 2048 : 1024) ? 64 : sk <= 2048 ? 96 : 192;
                 }
