@@ -138,7 +138,7 @@ def test_random_kvcache(block):
         g = torch.Generator().manual_seed(3000 + block * 100 + it)
         gen = lambda shape, dtype: torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype)
         d = rnd.choice([32, 64, 80, 96, 128, 160, 256])
-        seqlen_q = rnd.choice([1, 1, 1, 2, 3, 5, 16, 17, 64, 100])
+        seqlen_q = rnd.choice([1, 1, 1, 2, 3, 5, 16, 17, 64, 100, 130, 260])
         seqlen_k = max(rnd.choice([1, 17, 128, 129, 255, 256, 339, 1000, 1024, 3000, 5000, 8200, 12000]), seqlen_q + 3)
         b = rnd.choice([1, 2, 3, 7])
         hk = rnd.choice([1, 2, 3]); h = hk * rnd.choice([1, 2, 4, 8, 8, 17, 32])
