@@ -145,7 +145,8 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     const bool dec = use_decode_kernel(p);
     // The tiled kernel under the persistent schedule of the decode kernel (prefill_persistent_kernel): one row
     // block per (batch, kv head) with every q head of the kv head in it, over a cache whose lengths are on the
-    // device.  Chunks of 2048 keys or more (about FA_DEC_SLOTS_P per launch), their remainders in pieces of 512+.
+    // device.  Chunks of FA_TILE_MINLEN keys or more (about FA_TILE_SLOTS per launch), their remainders in halves,
+    // quarters or eighths of a chunk (1024 keys or more; see sb below).
     const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;
     int64_t tile_chunk = 0;
     if (!dec && allow_split && p.num_splits == 0 && p.p_dropout == 0.f && counters_ok(p) && !p.cu_seqlens_q && p.cu_seqlens_k &&
