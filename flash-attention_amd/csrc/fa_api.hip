@@ -158,7 +158,12 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
         const int64_t len = (std::max<int64_t>(minlen, (int64_t)sk * wgs / FA_TILE_SLOTS) + 511) / 512 * 512;
         // (launches that fill the CUs without a split keep the plain form up to 8192 keys: two or three chunks per
         // sequence do not pay for the merge)
-        if (sk >= 2 * len && (wgs < kNumCU || sk >= 8192)) tile_chunk = len;
+        // (Rows that are plain query positions, enough of them for the pipelined kernels, in a launch that fills the
+        // CUs: left whole, on those kernels -- 96-128 rows, 256-2048 row blocks, caches of 8k-32k: +5-57 % at head
+        // dims 64 / 128 and +30-85 % at 256 on equal and on short lengths, -6..-11 % on lengths drawn from the
+        // whole range at 512 row blocks; with 64 row blocks the ticket schedule is 2-4 x as fast.)
+        const bool whole_is_fast = !packed && p.seqlen_q >= prefill_long_rows(db) && wgs >= kNumCU;
+        if (sk >= 2 * len && (wgs < kNumCU || sk >= 8192) && !whole_is_fast) tile_chunk = len;
     }
     const int gran = dec ? 128 : tile_chunk ? 512 : prefill_block_n(db);
     auto rup = [](int64_t x, int64_t m) { return (int)((x + m - 1) / m * m); };
