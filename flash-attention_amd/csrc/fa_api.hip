@@ -16,6 +16,7 @@
 namespace fa {
 
 static thread_local std::string g_err;
+thread_local int32_t g_last_kernel = FA_KERNEL_NONE;
 static int fail(const char* msg) { g_err = msg; return 1; }
 static int fail_hip(int e, const char* where) {
     g_err = std::string(where) + ": " + hipGetErrorString((hipError_t)e);
@@ -122,9 +123,26 @@ static int check_common(const fa_fwd_params* p) {
     return 0;
 }
 
+// elements from the first to one past the last element of a (b, s, h, d) tensor with non-negative strides
+static int64_t span_elems(int64_t b, int64_t s, int64_t h, int64_t d, int64_t bs, int64_t rs, int64_t hs) {
+    return (b - 1) * bs + (s - 1) * rs + (h - 1) * hs + d;
+}
+static bool spans_overlap(const void* a, int64_t a_elems, const void* b, int64_t b_elems) {
+    const uintptr_t a0 = (uintptr_t)a, a1 = a0 + (uintptr_t)a_elems * 2, b0 = (uintptr_t)b, b1 = b0 + (uintptr_t)b_elems * 2;
+    return a0 < b1 && b0 < a1;
+}
+
 // the caller lent enough zeroed words for the persistent decode kernel
 static bool counters_ok(const fa_fwd_params& p) {
-    return p.work_counter != nullptr && p.work_counter_len >= FA_WORK_COUNTER_WORDS;
+    return p.work_counter != nullptr && p.work_counter_len >= FA_WORK_COUNTER_WORDS && (uintptr_t)p.work_counter % 8 == 0;
+}
+// epoch of the next launch's ticket counters (epoch_counter_next, fa_common.h): never zero, never the same twice
+// in a row within a process
+static uint32_t next_epoch() {
+    static std::atomic<uint32_t> g_epoch{0};
+    uint32_t e = g_epoch.fetch_add(1, std::memory_order_relaxed) + 1;
+    if (e == 0) e = g_epoch.fetch_add(1, std::memory_order_relaxed) + 1;
+    return e;
 }
 
 // Split planning for 256 CUs.
@@ -259,6 +277,7 @@ static void fill_kparams(KParams& kp, const fa_fwd_params& p) {
     kp.rotary_q = 0;
     kp.dec_persistent = kp.dec_sa = kp.dec_sb = kp.dec_sub = kp.dec_append = kp.dec_compact = 0;
     kp.work_counter = q.work_counter;
+    kp.epoch = next_epoch();
     kp.work_items = nullptr;
     kp.pack_g = 0;
     kp.pack_q_hs = kp.pack_o_hs = 0;
@@ -292,6 +311,8 @@ static int run_attention(KParams& kp, hipStream_t stream) {
     return 0;
 }
 
+// `p` is the problem as the caller described it (before grouped heads become rows): plan() applies those
+// transforms itself, so what it answers here is what fa_plan_splits answered for the same params.
 static int resolve_splits(KParams& kp, const fa_fwd_params& p, bool allow_split) {
     const SplitPlan r = plan(p, allow_split);
     const int s = r.splits;
@@ -393,6 +414,7 @@ extern "C" {
 
 const char* fa_last_error(void) { return g_err.c_str(); }
 int32_t fa_version(void) { return (0 << 16) | 1; }
+int32_t fa_last_kernel(void) { return g_last_kernel; }
 int32_t fa_sizeof_params(void) { return (int32_t)sizeof(fa_fwd_params); }
 
 int fa_num_splits_heuristic_reference(int32_t batch_nheads_mblocks, int32_t num_sms, int32_t num_n_blocks, int32_t max_splits) {
@@ -440,7 +462,7 @@ int fa_fwd(const fa_fwd_params* p, void* hip_stream) {
     kp.p.rotary_dim = 0;
     if (groups_as_rows(kp.p)) kp.has_right = 0;
     else kp.pack_g = positions_and_groups_as_rows(kp.p, &kp.pack_q_hs, &kp.pack_o_hs);
-    if (int r = resolve_splits(kp, kp.p, true)) return r;
+    if (int r = resolve_splits(kp, *p, true)) return r;
     return run_attention(kp, (hipStream_t)hip_stream);
 }
 
@@ -490,7 +512,7 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
     // (q rotary: without a mask every row is rotated to the position of the first new token, as the one row was)
     if (groups_as_rows(kp.p)) kp.has_right = 0;
     else kp.pack_g = positions_and_groups_as_rows(kp.p, &kp.pack_q_hs, &kp.pack_o_hs);
-    if (int r = resolve_splits(kp, kp.p, true)) return r;
+    if (int r = resolve_splits(kp, *p, true)) return r;
     hipStream_t stream = (hipStream_t)hip_stream;
     // The persistent decode kernel appends the new rows itself: the item that reaches them writes them.
     // With a left window bound some new rows may lie outside every query's window and would not be
@@ -503,8 +525,13 @@ int fa_fwd_kvcache(const fa_fwd_params* p, void* hip_stream) {
     // pass of their own and the attention kernel reads them from there, so that the launch takes the pipelined /
     // ping-pong kernels like one without rotary (a chunk of 512 tokens appended to caches of 16k, batch 64:
     // 8.7 -> 6.0 ms; the general kernel, which rotates while it loads Q, runs at two thirds of their rate).
-    // (Not when the caller's o is q itself: the rotation of a row reads both halves of it.)
-    if (kp.rotary_q && kp.num_splits <= 1 && kp.pack_g <= 1 && !use_decode_kernel(kp.p) && kp.p.q != kp.p.o &&
+    // (o holds the rotated q rows before the results land in it, so o must not share memory with q: when their
+    // address ranges meet -- the same tensor, or views of one tensor -- the general kernel runs, which rotates
+    // while it loads and writes nothing but results)
+    const bool disjoint = !spans_overlap(
+        kp.p.q, span_elems(kp.p.b, kp.p.seqlen_q, kp.p.h, kp.p.d, kp.p.q_batch_stride, kp.p.q_row_stride, kp.p.q_head_stride),
+        kp.p.o, span_elems(kp.p.b, kp.p.seqlen_q, kp.p.h, kp.p.d, kp.p.o_batch_stride, kp.p.o_row_stride, kp.p.o_head_stride));
+    if (kp.rotary_q && kp.num_splits <= 1 && kp.pack_g <= 1 && !use_decode_kernel(kp.p) && disjoint &&
         kp.p.seqlen_q >= prefill_long_rows(bucket(kp.p.d))) {
         if (int e = launch_rotate_q(kp, stream)) return fail_hip(e, "q rotary kernel launch");
         kp.p.q = kp.p.o;

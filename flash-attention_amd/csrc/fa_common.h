@@ -52,8 +52,8 @@ struct KParams {
     int32_t has_left, has_right;  // window bounds active (after causal normalisation)
     int32_t rotary_q;      // rotate q on load
     // persistent decode schedule (see fa_decode.hip): dec_sa slots of split_len keys, then dec_sb
-    // slots of dec_sub keys for each sequence's ragged remainder; tickets from work_counter[0], workgroups
-    // that have left counted in [1].
+    // slots of dec_sub keys for each sequence's ragged remainder; tickets from work_counter[0..1], workgroups
+    // that have left counted in [2..3] (64-bit epoch counters, epoch_counter_next).
     // dec_append: the item that reaches rows [cache length, cache length + seqlen_knew) writes them
     // dec_compact: the tickets cover only the slots that hold keys (the kernel counts them per batch entry
     // from the lengths); the merge then derives which slots were written from the lengths as well
@@ -69,6 +69,7 @@ struct KParams {
     int32_t pack_g;
     int64_t pack_q_hs, pack_o_hs;
     int32_t* work_counter;
+    uint32_t epoch;        // non-zero, drawn anew by the host for every call: tags the counters of this launch
     // Packed batches: work list built on the device from cu_seqlens_q just before the launch (work_list_kernel,
     // fa_aux.hip), or NULL.  8 item counts, then for XCD x a list of (gridDim.x / 8) slots of two words:
     // batch index, (q head << 16) | row block.
@@ -638,11 +639,36 @@ FA_DEV void item_key_range(const KParams& kp, int mode, int idx, int hi, int& c_
     }
 }
 
+// A counter that needs no set-up launch and survives a launch that never finished.  The 64-bit word (two of the
+// caller's int32 words, 8-byte aligned) holds (epoch << 32) | count; `epoch` is a non-zero number the host draws
+// anew for every launch.  A word whose upper half is not this launch's epoch -- zero as every finished launch
+// leaves it, or whatever a launch that was torn down mid-way, or a caller that did not clear the words, left
+// behind -- counts as zero: the first draw that finds it so installs (epoch, 1) with a compare-and-swap and takes
+// value 0, draws that lose that race see the epoch and count on.  Returns the value before the increment.  The
+// usual draw is one atomic add; only the first draws of a launch take the second path, and every path ends after
+// at most one failed compare-and-swap per other lane drawing at that moment (nothing waits for another workgroup).
+FA_DEV uint32_t epoch_counter_next(int32_t* words, uint32_t epoch) {
+    uint64_t* w = reinterpret_cast<uint64_t*>(words);
+    uint64_t old = __hip_atomic_fetch_add(w, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((uint32_t)(old >> 32) == epoch) return (uint32_t)old;
+    const uint64_t fresh = ((uint64_t)epoch << 32) | 1u;
+    for (;;) {
+        uint64_t cur = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((uint32_t)(cur >> 32) == epoch) {
+            old = __hip_atomic_fetch_add(w, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return (uint32_t)old;
+        }
+        if (__hip_atomic_compare_exchange_strong(w, &cur, fresh, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            return 0u;
+    }
+}
+
 // The persistent schedule itself, for a grid of resident workgroups: calls Item::run(kp, smem, kv head, batch
 // entry, partial slot, mode, idx) for this workgroup's block id and then for every ticket it draws from
-// kp.work_counter[0] until the items are used up; the last workgroup to finish puts the two counter words back
-// to zero.  All lanes of the workgroup must call it together and return from every item (it synchronises the
-// workgroup between items, so an item may use all of the dynamic LDS, `smem`).
+// the counter in kp.work_counter[0..1] until the items are used up; workgroups that have left are counted in
+// kp.work_counter[2..3] and the last one puts all four words back to zero (epoch_counter_next).  All lanes of
+// the workgroup must call it together and return from every item (it synchronises the workgroup between items,
+// so an item may use all of the dynamic LDS, `smem`).
 template <class Item>
 FA_DEV void for_each_ticket(const KParams& kp, char* smem) {
     __shared__ int s_ticket;
@@ -681,14 +707,13 @@ FA_DEV void for_each_ticket(const KParams& kp, char* smem) {
         n_macro = s_pm[p.b] * p.h_k;
         total = n_macro + s_ps[p.b] * p.h_k;
     }
-    int32_t* const ticket = kp.work_counter;
     // the first item of a workgroup is the one its block id names (no round trip to the counter before any
     // work starts); the tickets drawn afterwards continue behind the grid
     for (bool first = true;; first = false) {
         int t = (int)blockIdx.x;
         if (!first) {
             __syncthreads();          // previous item is done with LDS and with s_ticket
-            if (threadIdx.x == 0) s_ticket = (int)gridDim.x + __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (threadIdx.x == 0) s_ticket = (int)gridDim.x + (int)epoch_counter_next(kp.work_counter, kp.epoch);
             __syncthreads();
             t = s_ticket;
         }
@@ -714,10 +739,11 @@ FA_DEV void for_each_ticket(const KParams& kp, char* smem) {
         Item::run(kp, smem, hk, b, macro ? idx : kp.dec_sa + idx, macro ? kMacro : kSub, idx);
     }
     if (threadIdx.x == 0) {
-        const int gone = __hip_atomic_fetch_add(kp.work_counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (gone == (int)gridDim.x - 1) {     // every workgroup has drawn its last ticket
-            __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(kp.work_counter + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t gone = epoch_counter_next(kp.work_counter + 2, kp.epoch);
+        if (gone == gridDim.x - 1u) {     // every workgroup has drawn its last ticket: leave both counters fresh
+            uint64_t* w = reinterpret_cast<uint64_t*>(kp.work_counter);
+            __hip_atomic_store(w, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(w + 1, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

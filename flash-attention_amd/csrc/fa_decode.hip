@@ -356,8 +356,9 @@ __global__ void __launch_bounds__(256, (D > 128 ? 1 : 2)) decode_kernel(const KP
 // Persistent form: a fixed number of resident workgroups draw items from a ticket counter, in the
 // same cache-row-friendly order (kv head fastest), first the kMacro pass then the kSub pass.
 //  * The item whose key range reaches the new rows appends them (APPEND, see decode_item): no append launch.
-//  * work_counter[0] is the ticket, work_counter[1] counts the workgroups that have left; the last one puts
-//    both back to zero, so the words are zero again when the kernel ends and no launch has to reset them.
+//  * work_counter[0..1] is the ticket counter, work_counter[2..3] counts the workgroups that have left; the last
+//    one puts both back to zero, and both are tagged with the call's epoch (epoch_counter_next, fa_common.h), so
+//    no launch has to reset them, not even after a launch that never finished.
 // Measured and not adopted: drawing the next ticket when an item's key loop ends, so that the counter's round
 // trip runs under the merge and the output stores (+1 % on the step); drawing it early (before the item: the returning atomic sits in front
 // of the item's first K/V loads in the wave's in-order memory queue, +7 % time; after the item's last load:
@@ -386,7 +387,8 @@ static int launch_decode_kernel(dim3 grid, int smem, const KParams& kp, hipStrea
     const hipError_t e = FA_ALLOW_DYNAMIC_LDS(KERN, smem);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(KERN, grid, dim3(256), smem, stream, kp);
-    return (int)hipGetLastError();
+    return note_kernel((int)hipGetLastError(), kp.dec_persistent ? FA_KERNEL_DECODE_TICKETS : FA_KERNEL_DECODE, false, kp.num_splits > 1,
+                       kp.p.d <= 64 ? 64 : kp.p.d <= 128 ? 128 : 256);
 }
 
 template <typename T, int D, bool STREAM>

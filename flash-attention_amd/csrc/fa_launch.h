@@ -4,6 +4,13 @@
 
 namespace fa {
 struct BwdKParams;
+// What fa_last_kernel() reports: every attention launcher notes the kernel it enqueued (FA_KERNEL_* | flags |
+// computed head dims << 16) for the calling thread.  Host-side only.
+extern thread_local int32_t g_last_kernel;
+inline int note_kernel(int launch_error, int id, bool dropout, bool split, int head_dims) {
+    if (launch_error == 0) g_last_kernel = id | (dropout ? FA_KERNEL_FLAG_DROPOUT : 0) | (split ? FA_KERNEL_FLAG_SPLIT : 0) | (head_dims << 16);
+    return launch_error;
+}
 #define FA_DECL_PREFILL(name) int name(const KParams& kp, hipStream_t stream);
 FA_DECL_PREFILL(launch_prefill_bf16_64)
 FA_DECL_PREFILL(launch_prefill_bf16_128)

@@ -18,6 +18,7 @@
 //  * Key tiles that a wave's rows cannot see (causal / sliding window) are skipped per wave.
 #pragma once
 #include "fa_common.h"
+#include "fa_launch.h"
 
 namespace fa {
 
@@ -387,7 +388,7 @@ int launch_prefill(KParams kp, hipStream_t stream) {
             if (e != hipSuccess) return (int)e;
             hipLaunchKernelGGL(kern, pgrid, block, C::SMEM, stream, kp);
         }
-        return (int)hipGetLastError();
+        return note_kernel((int)hipGetLastError(), FA_KERNEL_TILED_TICKETS, false, true, D);
     }
     const bool one_reader = kp.stream_kv && kp.num_m_blocks == 1 && kp.p.h == kp.p.h_k && !(kp.p.p_dropout > 0.f);
     if (split && one_reader) {
@@ -416,7 +417,7 @@ int launch_prefill(KParams kp, hipStream_t stream) {
         if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     }
-    return (int)hipGetLastError();
+    return note_kernel((int)hipGetLastError(), FA_KERNEL_TILED, kp.p.p_dropout > 0.f, split, D);
 }
 
 // key-tile length used by launch_prefill for a head-dim bucket (the split planner needs it)

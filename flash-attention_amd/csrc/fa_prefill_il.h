@@ -42,6 +42,7 @@ template <typename T, int D_, int BN_, int DV_ = D_>
 struct ILCfg {
     static constexpr int D = D_, BN = BN_;
     static constexpr bool kPair = false;
+    static constexpr int kKernelId = D_ > 128 ? FA_KERNEL_WIDE : FA_KERNEL_PIPELINED, kHeadDims = DV_;   // for fa_last_kernel
     static constexpr int kThreads = 256;
     static constexpr int kWaves = 4;
     static constexpr int BM = kWaves * 32;
@@ -74,6 +75,7 @@ template <typename T, int DV_ = 256>
 struct ILCfgPair {
     static constexpr int D = 256, BN = 32;
     static constexpr bool kPair = true;
+    static constexpr int kKernelId = FA_KERNEL_WIDE_PAIR, kHeadDims = DV_;
     static constexpr int kThreads = 512;
     static constexpr int kWaves = 8;
     static constexpr int BM = (kWaves / 2) * 32;
@@ -623,7 +625,7 @@ int launch_prefill_il_one(KParams kp, hipStream_t stream) {
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-    return (int)hipGetLastError();
+    return note_kernel((int)hipGetLastError(), C::kKernelId, DROPOUT, false, C::kHeadDims);
 }
 
 template <typename T, typename C>

@@ -50,7 +50,3 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }
 }  // namespace fa
-#if defined(FA_PP_TIMING) && FA_T_BF16 && FA_D == 128
-// measurement builds only: copies the stage stamps of fa::prefill_pp_kernel<bf16, 128> to the host
-extern "C" int fa_pp_debug_read(void* host, size_t bytes) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fa::fa_pp_dbg), bytes); }
-#endif

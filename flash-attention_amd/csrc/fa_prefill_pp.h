@@ -54,19 +54,6 @@ struct PPCfg {
     static_assert((BN * CPR) % kThreads == 0 && 64 % CPR == 0, "tile shape");
 };
 
-// -DFA_PP_TIMING: every workgroup records when it passes the stages of the kernel (shader-clock counter,
-// slots 0-5; constant 100 MHz counter at entry and exit, slots 6-7) for waves 0 and 4, into fa_pp_dbg, which
-// fa_pp_debug_read (fa_prefill_inst.hip) copies out.  Measurement builds only.
-#ifdef FA_PP_TIMING
-#define FA_PP_DBG_BLOCKS 32768      // workgroups with a record; launches with more blocks record only these
-__device__ long long fa_pp_dbg[FA_PP_DBG_BLOCKS * 2 * 16];
-#define FA_PP_STAMP(i) do { if (lane == 0 && (wave & 3) == 0 && blockIdx.x < FA_PP_DBG_BLOCKS) fa_pp_dbg[(blockIdx.x * 2 + group) * 16 + (i)] = __builtin_readcyclecounter(); } while (0)
-#define FA_PP_REALTIME(i) do { if (lane == 0 && (wave & 3) == 0 && blockIdx.x < FA_PP_DBG_BLOCKS) fa_pp_dbg[(blockIdx.x * 2 + group) * 16 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define FA_PP_STAMP(i) do {} while (0)
-#define FA_PP_REALTIME(i) do {} while (0)
-#endif
-
 // DV: head dims the products run over (a multiple of 32, p.d <= DV <= D).  Tiles keep the LDS layout of the
 // bucket D; with DV < D the k-steps and output column blocks past DV are not computed (head dim 96 on the
 // 128 bucket: 6 of 8 k-steps of S, 3 of 4 column blocks of O).
@@ -83,24 +70,16 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const int wave = tid >> 6, lane = tid & 63;
     const int l32 = lane & 31, hh = lane >> 5;
     const int group = wave >> 2;
-    FA_PP_STAMP(0);
-    FA_PP_REALTIME(6);
-#ifdef FA_PP_TIMING
-    if (lane == 0 && wave == 0 && blockIdx.x < FA_PP_DBG_BLOCKS)      // HW_ID: which CU runs this workgroup
-        fa_pp_dbg[(blockIdx.x * 2) * 16 + 12] = (long long)__builtin_amdgcn_s_getreg((31 << 11) | 4);
-#endif
 
     // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
     const uint32_t G = (uint32_t)(p.h / p.h_k);
     int g, mb, hk, b;
     if (!xcd_work_item(kp, (uint32_t)kp.num_m_blocks, (kp.has_left || kp.has_right) ? 32u : 0u, g, mb, hk, b)) return;
     const int head = hk * (int)G + g;
-    FA_PP_STAMP(8);       // work item known
 
     const SeqInfo si = seq_info(p, b);
     const int m0 = mb * C::BM;
     if (m0 >= si.sq) return;
-    FA_PP_STAMP(9);       // sequence bounds known
 
     const int shift = si.sk - si.sq;
     const int wl = p.window_left, wr = p.window_right;
@@ -121,13 +100,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     const int row = r0 + l32;
 
     // visit i of the key loop handles key tile tile_of(i) and uses ring slot i % NS
-#ifdef FA_PP_ASCENDING
-    constexpr int kDir = 1;
-    auto tile_of = [&](int i) { return t_lo + i; };
-#else
-    constexpr int kDir = -1;
+    // (from the last tile down: the masked tiles of a causal row block come first)
     auto tile_of = [&](int i) { return t_hi - 1 - i; };
-#endif
 
     // ---- asynchronous tile fills.  Pass j of wave w fills LDS positions [(w + 8j) * 64, +64) of the
     // tile (16 B each); position p is tile row p / CPR, stored chunk p % CPR, and holds global chunk
@@ -142,13 +116,13 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
     // 32-bit per-lane byte offset, so stepping to the next tile is scalar arithmetic.
     const int64_t kstep = (int64_t)BN * p.k_row_stride, vstep = (int64_t)BN * p.v_row_stride;
     const int64_t kpass = (int64_t)C::ROWS_PER_PASS * p.k_row_stride, vpass = (int64_t)C::ROWS_PER_PASS * p.v_row_stride;
-    const int t_first = kDir > 0 ? t_lo : t_hi - 1;
+    const int t_first = t_hi - 1;
     const T* ktile = kg + (int64_t)t_first * BN * p.k_row_stride;       // tile next to be requested
     const T* vtile = vg + (int64_t)t_first * BN * p.v_row_stride;
     const uint32_t koff = (uint32_t)(((int64_t)frow * p.k_row_stride + kch * 8) * 2);
     const uint32_t voff = (uint32_t)(((int64_t)frow * p.v_row_stride + vch * 8) * 2);
     // only key tile t_hi - 1 can reach past seqlen_k: its rows are clamped
-    const int i_tail = (t_hi * BN > si.sk) ? (kDir > 0 ? nt - 1 : 0) : -1;
+    const int i_tail = (t_hi * BN > si.sk) ? 0 : -1;
     auto fill_k = [&](int i) {
         const uint32_t dst = fill_base + (uint32_t)((i & (C::NS - 1)) * C::TILE);
         if (i == i_tail) {
@@ -161,7 +135,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) async_fill16(ktile + j * kpass, koff, dst + j * 8192);
         }
-        ktile += kDir * kstep;
+        ktile -= kstep;
     };
     auto fill_v = [&](int i) {
         const uint32_t dst = fill_base + (uint32_t)((C::NS + (i & (C::NS - 1))) * C::TILE);
@@ -175,7 +149,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) async_fill16(vtile + j * vpass, voff, dst + j * 8192);
         }
-        vtile += kDir * vstep;
+        vtile -= vstep;
     };
 
     // The first tiles are requested before anything else is set up: the q rows, the accumulators and the
@@ -186,7 +160,6 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         if (nt > 1) { fill_k(1); fill_v(1); }
         if (nt > 2) fill_k(2);
     }
-    FA_PP_STAMP(1);
 
     v8 qf[KSV];
     {
@@ -200,8 +173,6 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             qf[dk] = __builtin_bit_cast(v8, raw);
         }
     }
-
-    FA_PP_STAMP(10);      // q loads issued
     f32x16 o_acc[DBV];
 #pragma unroll
     for (int db = 0; db < DBV; db++)
@@ -378,10 +349,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
         // ---- prologue: K(0), V(0), K(1), V(1), K(2) were requested above; S = K(0) Q
         wait_vmcnt<0>();
         __syncthreads();
-        FA_PP_STAMP(2);
         if (active(0)) qk(0);
         if (group == 1) __syncthreads();   // group 1 runs one phase behind group 0
-        FA_PP_STAMP(3);
 
         for (int i = 0; i < nt; i++) {
             // ---- Y(i): VALU phase (and requests for the tiles needed 3 iterations ahead)
@@ -401,7 +370,6 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             __syncthreads();
         }
         if (group == 0) __syncthreads();
-        FA_PP_STAMP(4);
     }
 
     // ---- epilogue
@@ -436,11 +404,6 @@ __global__ void __launch_bounds__(512, 2) prefill_pp_kernel(const KParams kp) {
             if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
         }
     }
-    FA_PP_STAMP(5);
-    FA_PP_REALTIME(7);
-#ifdef FA_PP_TIMING
-    if (lane == 0 && wave == 0 && blockIdx.x < FA_PP_DBG_BLOCKS) fa_pp_dbg[(blockIdx.x * 2) * 16 + 11] = nt;
-#endif
 }
 
 template <typename T, int D, int BN, bool DROPOUT, int DV = D>
@@ -457,7 +420,7 @@ int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-    return (int)hipGetLastError();
+    return note_kernel((int)hipGetLastError(), FA_KERNEL_PINGPONG, DROPOUT, false, DV);
 }
 template <typename T, int D, int BN>
 int launch_prefill_pp(const KParams& kp, hipStream_t stream) {

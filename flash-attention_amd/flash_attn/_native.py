@@ -100,6 +100,8 @@ def _load():
     lib.fa_last_error.restype = ctypes.c_char_p
     lib.fa_version.argtypes = []
     lib.fa_version.restype = ctypes.c_int32
+    lib.fa_last_kernel.argtypes = []
+    lib.fa_last_kernel.restype = ctypes.c_int32
     lib.fa_sizeof_params.argtypes = []
     lib.fa_sizeof_params.restype = ctypes.c_int32
     for name in ("fa_bwd", "fa_varlen_bwd"):
@@ -133,10 +135,13 @@ def _check(cond, msg):
         raise RuntimeError(msg)
 
 
-def _call(fn, params, stream):
+def _call(fn, params, stream, device=None):
     rc = fn(ctypes.byref(params), ctypes.c_void_p(stream))
     if rc != 0:
-        raise RuntimeError(lib.fa_last_error().decode() or "libfa_mi355x: error %d" % rc)
+        msg = lib.fa_last_error().decode() or "libfa_mi355x: error %d" % rc
+        if device is not None:
+            _reset_counters(device)
+        raise RuntimeError(msg)
 
 
 def _ptr(t):
@@ -205,7 +210,8 @@ def _dropout_state(p, p_dropout, return_softmax, gen_, batch, heads, seqlen_q, s
     return rng_state, s_dmask
 
 
-_COUNTERS = {}     # (device index, stream) -> zeroed int32 words lent to the persistent decode kernel
+WORK_COUNTER_WORDS = 4      # FA_WORK_COUNTER_WORDS of include/fa_mi355x.h
+_COUNTERS = {}     # (device index, stream) -> int32 words lent to the ticket-scheduled kernels
 
 
 _RETIRED = []
@@ -215,23 +221,37 @@ WORK_LIST = True      # packed forward launches lend the library room for its de
 def _counters(device, words):
     """Counter words for launches on the current stream of `device`: zero when first handed out and left
     zero by every launch, so one tensor per (device, stream) serves all calls (launches on one stream do
-    not overlap)."""
+    not overlap).  The kernels tag the words with a number of the call and treat anything else they find as
+    zero, so a tensor that has to be made while the stream is capturing a HIP graph is handed out uncleared:
+    the graph then holds no fill of it."""
     index = device.index if device.index is not None else torch.cuda.current_device()
     key = (index, _stream(device))
     t = _COUNTERS.get(key)
     if t is None or t.numel() < words:
         if t is not None:
             _RETIRED.append(t)      # a captured graph may still point at it
-        t = torch.zeros((max(16, int(words)),), dtype=torch.int32, device=device)
+        make = torch.empty if torch.cuda.is_current_stream_capturing() else torch.zeros
+        t = make((max(16, int(words)),), dtype=torch.int32, device=device)
         _COUNTERS[key] = t
     return t
+
+
+def _reset_counters(device):
+    """After a call that returned an error: clear the counter words of the device's streams (a launch that did
+    not complete may have left them in use; the next launch would cope, this keeps them tidy)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if torch.cuda.is_current_stream_capturing():
+        return
+    for (dev, _), t in _COUNTERS.items():
+        if dev == index:
+            t[:WORK_COUNTER_WORDS].zero_()
 
 
 def _plan_and_alloc(params, api, batch, heads, seqlen_q, d, device):
     """Resolve the split count and allocate the fp32 partial buffers like the reference does
     (flash_api.cpp:373-389, 1241-1257).  The returned tensors must stay alive until launch."""
     n = ctypes.c_int32(0)
-    counter = _counters(device, 2)
+    counter = _counters(device, WORK_COUNTER_WORDS)
     params.work_counter = counter.data_ptr()
     params.work_counter_len = counter.numel()
     rc = lib.fa_plan_splits(ctypes.byref(params), api, ctypes.byref(n))
@@ -303,7 +323,7 @@ def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, wi
                                             seqlen_k, q_dtype, q.device)
         if seqlen_q > 0 and seqlen_k > 0:
             keep = _plan_and_alloc(p, 0, batch_size, num_heads, seqlen_q, head_size, q.device)
-            _call(lib.fa_fwd, p, _stream(q.device))
+            _call(lib.fa_fwd, p, _stream(q.device), q.device)
             del keep
         else:
             out.zero_()
@@ -386,10 +406,10 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
         if total_q > 0 and max_seqlen_q > 0:
             # room for the work list the library builds from cu_seqlens_q on the device (WORK_LIST = False: the
             # arithmetic order, for tests that compare the two)
-            words = lib.fa_work_list_words(ctypes.byref(p)) if WORK_LIST else 2
+            words = lib.fa_work_list_words(ctypes.byref(p)) if WORK_LIST else WORK_COUNTER_WORDS
             counter = _counters(q.device, words)
             p.work_counter, p.work_counter_len = counter.data_ptr(), counter.numel()
-            _call(lib.fa_varlen_fwd, p, _stream(q.device))
+            _call(lib.fa_varlen_fwd, p, _stream(q.device), q.device)
         elif s_dmask is not None:
             s_dmask.zero_()
 
@@ -650,7 +670,7 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
             _call(lib.fa_fwd_kvcache_noalloc, p, _stream(q.device))
         elif seqlen_q > 0 and seqlen_k > 0:
             keep.append(_plan_and_alloc(p, 2, batch_size, num_heads, seqlen_q, head_size, q.device))
-            _call(lib.fa_fwd_kvcache, p, _stream(q.device))
+            _call(lib.fa_fwd_kvcache, p, _stream(q.device), q.device)
         else:
             out.zero_()
             softmax_lse.fill_(float("inf"))
@@ -665,6 +685,19 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
             kcache.copy_(kcache_padded[..., :head_size_og])
             vcache.copy_(vcache_padded[..., :head_size_og])
     return [out, softmax_lse]
+
+
+# FA_KERNEL_* of include/fa_mi355x.h
+KERNEL_NAMES = {0: "none", 1: "tiled", 2: "tiled_tickets", 3: "pipelined", 4: "pingpong", 5: "wide", 6: "wide_pair",
+                7: "decode", 8: "decode_tickets"}
+
+
+def last_kernel():
+    """(name, dropout instantiation, key range split, head dims computed) of the attention kernel that the
+    calling thread's last forward call launched: fa_last_kernel() decoded.  Host-side bookkeeping, no device
+    work; tests assert with it that a case still reaches the kernel it was written for."""
+    w = lib.fa_last_kernel()
+    return KERNEL_NAMES.get(w & 0xff, "unknown"), bool(w & 0x100), bool(w & 0x200), (w >> 16) & 0xffff
 
 
 def num_splits_heuristic_reference(batch_nheads_mblocks, num_sms, num_n_blocks, max_splits):

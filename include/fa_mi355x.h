@@ -60,8 +60,13 @@ typedef struct fa_fwd_params {
                                        per-batch key lengths (cache_seqlens), or NULL */
     const int32_t *cache_batch_idx; /* (b) row of k/v used (and updated) for batch i, or NULL */
     int32_t *work_counter;          /* optional: work_counter_len (>= FA_WORK_COUNTER_WORDS) int32 words of
-                                       device memory whose first FA_WORK_COUNTER_WORDS words are ZERO before
-                                       the first call that uses them; every call leaves those zero again.
+                                       device memory, 8-byte aligned.  The first FA_WORK_COUNTER_WORDS words are
+                                       the ticket and exit counters of the ticket-scheduled kernels; every
+                                       launch that completes leaves them zero, and a launch treats whatever
+                                       else it finds there (a launch that was torn down mid-way, words the
+                                       caller never cleared) as zero too: each call tags its counters with a
+                                       number of its own, so no clearing launch is needed (allocate them zeroed
+                                       all the same).
                                        When set, split-KV decode launches run as a persistent kernel whose
                                        workgroups draw (batch, kv head, key chunk) items from a ticket and
                                        whose item that reaches the new rows appends them to the cache (no
@@ -116,8 +121,9 @@ typedef struct fa_fwd_params {
     int32_t reserved0;
 } fa_fwd_params;
 
-/* words the ticket-scheduled kernels need behind work_counter: ticket, exit count */
-#define FA_WORK_COUNTER_WORDS 2
+/* words the ticket-scheduled kernels need behind work_counter: two 64-bit counters (tickets drawn, workgroups
+ * that have left), each (call tag << 32) | count */
+#define FA_WORK_COUNTER_WORDS 4
 
 /*
  * Words behind work_counter with which every launch of fa_varlen_fwd on these params (b, h, h_k, seqlen_q =
@@ -146,8 +152,9 @@ int fa_varlen_fwd(const fa_fwd_params *p, void *hip_stream);
  * k_new/v_new at rows cache_seqlens[b] .. of cache row cache_batch_idx[b] (new keys rotated when
  * rotary tables are given, :763-852 of flash_fwd_kernel.h), q rotated on load (:854-891), then
  * attention over cache_seqlens[b] + seqlen_knew keys.  Mutates k and v in place.  With rotary tables and 96 or
- * more query rows, o may hold the rotated q rows before the results land in it: o must not overlap q partially
- * (o == q is recognised).
+ * more query rows, o holds the rotated q rows before the results land in it, but only when the address ranges
+ * of q and o do not meet; when they do (o == q, or views of one tensor) the kernel that rotates while it loads
+ * runs instead.  As in the reference, o may be q itself but must not overlap it in any other way.
  */
 int fa_fwd_kvcache(const fa_fwd_params *p, void *hip_stream);
 
@@ -193,6 +200,30 @@ int fa_num_splits_heuristic_reference(int32_t batch_nheads_mblocks, int32_t num_
  * rng_state inside the forward kernel (csrc/flash_attn/src/flash_fwd_kernel.h:1142-1148).
  */
 int fa_set_rng_state(uint64_t *rng_state, uint64_t seed, uint64_t offset, void *hip_stream);
+
+/*
+ * Which attention kernel the calling thread's last successful forward launch used (fa_fwd, fa_varlen_fwd,
+ * fa_fwd_kvcache, fa_fwd_kvcache_noalloc); 0 before any.  Host-side bookkeeping only: no device work, no
+ * synchronisation.  No counterpart in the reference, whose dispatch (run_mha_fwd, flash_api.cpp:194-204, and
+ * flash_fwd_launch_template.h:140-336) is not observable either; tests use it to assert that a case written for
+ * one kernel still reaches it when the dispatch thresholds move.
+ *   bits 0-7   FA_KERNEL_* below
+ *   bit  8     the dropout instantiation ran
+ *   bit  9     the key range was split (partial results + merge launch)
+ *   bits 16-31 head dims the products ran over (the bucket, or less: 96 on the 128 bucket, 160 / 192 / 224 on 256)
+ */
+#define FA_KERNEL_NONE 0
+#define FA_KERNEL_TILED 1               /* general tiled kernel, one workgroup per row block (and key chunk) */
+#define FA_KERNEL_TILED_TICKETS 2       /* the same under the ticket schedule */
+#define FA_KERNEL_PIPELINED 3           /* software-pipelined 128-row kernel, head dims up to 128 */
+#define FA_KERNEL_PINGPONG 4            /* 8-wave 256-row kernel, head dim 65-128 */
+#define FA_KERNEL_WIDE 5                /* head dims 129-256, whole head dim per wave */
+#define FA_KERNEL_WIDE_PAIR 6           /* head dims 129-256, wave pairs */
+#define FA_KERNEL_DECODE 7              /* up to 16 packed query rows, one workgroup per key chunk */
+#define FA_KERNEL_DECODE_TICKETS 8      /* the same under the ticket schedule */
+#define FA_KERNEL_FLAG_DROPOUT (1 << 8)
+#define FA_KERNEL_FLAG_SPLIT (1 << 9)
+int32_t fa_last_kernel(void);
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char *fa_last_error(void);

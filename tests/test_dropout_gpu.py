@@ -33,7 +33,24 @@ def _gen(shape, dtype, seed):
     return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype)
 
 
-def _check_all(out, lse, S, grads, q, k, v, dout, p, causal, window):
+def _ran(name, head_dims=None):
+    """the forward launch before this call took the dropout instantiation of kernel `name`"""
+    from flash_attn import _native as nat
+    got = nat.last_kernel()
+    _say("   kernel", got)
+    assert got[0] == name and got[1] and not got[2], got
+    if head_dims is not None:
+        assert got[3] == head_dims, got
+
+
+def _check_all(out, lse, S, grads, q, k, v, dout, p, causal, window, entries=None):
+    """entries: batch entries to check (independent problems), default all"""
+    if entries is not None:
+        for e in entries:
+            _say("   batch entry", e)
+            sl = lambda t: t[e:e + 1]
+            _check_all(sl(out), sl(lse), sl(S), [sl(g) for g in grads], sl(q), sl(k), sl(v), sl(dout), p, causal, window)
+        return
     b, sq, h, d = q.shape
     sk = k.shape[1]
     S = S[:, :, :sq, :sk].float().cpu()
@@ -90,7 +107,7 @@ def test_dropout_forward_backward(sq, sk, d, mode, dtype):
 @pytest.mark.parametrize("d", [64, 128, 256])
 @pytest.mark.parametrize("p", [0.1, 0.5])
 def test_dropout_on_the_long_sequence_kernels(d, p):
-    """From 512 query rows on the forward runs on the software-pipelined kernels (pairs of waves at
+    """From 96 query rows on the forward runs on the software-pipelined kernels (pairs of waves at
     head dim 256), which walk the score matrix in steps of their own."""
     _say("dropout long", d, p)
     dtype, b, h, s = torch.bfloat16, 1, 4, 1100
@@ -98,25 +115,34 @@ def test_dropout_on_the_long_sequence_kernels(d, p):
     dout = _gen((b, s, h, d), dtype, 4)
     qd, kd, vd = [t.to(DEV).requires_grad_() for t in (q, k, v)]
     out, lse, S = _fa().flash_attn_func(qd, kd, vd, dropout_p=p, causal=True, return_attn_probs=True)
+    _ran("wide_pair" if d == 256 else "pipelined")
     grads = torch.autograd.grad(out, (qd, kd, vd), dout.to(DEV))
     _check_all(out, lse, S, grads, q, k, v, dout, p, True, (-1, -1))
 
 
-@pytest.mark.parametrize("sq,sk,d,mode,dtype", [(640, 2300, 128, "full", torch.bfloat16), (600, 4200, 96, "causal", torch.float16),
-                                                  (1030, 4300, 128, "local", torch.bfloat16)])
-def test_dropout_on_the_long_key_kernel(sq, sk, d, mode, dtype):
-    """Key lengths past 768 (full) / 2048 (masked) at head dim 65..128 take the 8-wave kernel, which
-    applies the mask in its own register geometry (one query row per lane)."""
-    _say("dropout long keys", sq, sk, d, mode, dtype)
-    b, h, hk, p = 1, 4, 2, 0.17
+# The dropout instantiation of the 8-wave ping-pong kernel, which applies the mask in its own register geometry (one
+# query row per lane).  Dispatch sends a launch there at head dim 65..128 with keys beyond 768 (no mask) / from 2048
+# on (masked), more than 128 / 256 row blocks of 256 rows and no window spanning 768 keys or fewer: the batch makes
+# the launch that large, and three batch entries (independent problems) are checked.
+@pytest.mark.parametrize("sq,sk,d,mode,dtype,b,h,hk", [
+    (640, 2300, 128, "full", torch.bfloat16, 24, 2, 1),          # 3 x 2 x 24 = 144 row blocks, no mask
+    (600, 4200, 96, "causal", torch.float16, 44, 2, 2),          # 3 x 2 x 44 = 264; sq < sk; 96 of the 128 columns
+    (1030, 4300, 128, "local", torch.bfloat16, 26, 2, 1),        # 5 x 2 x 26 = 260; two-sided window of 1800 keys
+    (1300, 2100, 128, "causal", torch.float16, 22, 2, 2),        # 6 x 2 x 22 = 264; fp16 at all 128 columns
+    (2200, 2100, 80, "causal", torch.bfloat16, 15, 2, 1),        # 9 x 2 x 15 = 270; sq > sk: leading rows see nothing
+])
+def test_dropout_on_the_pingpong_kernel(sq, sk, d, mode, dtype, b, h, hk):
+    _say("dropout ping-pong", sq, sk, d, mode, dtype)
+    p = 0.17
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
     dout = _gen((b, sq, h, d), dtype, 4)
     window = (1500, 300) if mode == "local" else (-1, -1)
     qd, kd, vd = [t.to(DEV).requires_grad_() for t in (q, k, v)]
     out, lse, S = _fa().flash_attn_func(qd, kd, vd, dropout_p=p, causal=(mode == "causal"), window_size=window,
                                         return_attn_probs=True)
+    _ran("pingpong", 128)       # (the dropout instantiation always runs all 128 columns)
     grads = torch.autograd.grad(out, (qd, kd, vd), dout.to(DEV))
-    _check_all(out, lse, S, grads, q, k, v, dout, p, mode == "causal", window)
+    _check_all(out, lse, S, grads, q, k, v, dout, p, mode == "causal", window, entries=[0, b - 1, b // 2])
 
 
 def test_dropout_qkvpacked_and_varlen():

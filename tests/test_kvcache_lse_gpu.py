@@ -85,7 +85,7 @@ def test_lse_persistent_decode_and_merge(with_new):
     p.window_left = p.window_right = -1
     for name in ("q", "k", "v", "o", "softmax_lse", "work_counter", "cu_seqlens_k"):
         setattr(p, name, 256)          # non-null placeholders: planning reads no memory
-    p.work_counter_len = 2
+    p.work_counter_len = nat.WORK_COUNTER_WORDS
     import ctypes
     n = ctypes.c_int32(0)
     assert nat.lib.fa_plan_splits(ctypes.byref(p), 2, ctypes.byref(n)) == 0
@@ -190,7 +190,7 @@ def _planned_splits(nat, b, h, hk, sq, cap, d):
     for name in ("q", "k", "v", "o", "softmax_lse", "work_counter", "cu_seqlens_k"):
         setattr(p, name, 256)          # non-null placeholders: planning reads no memory
     p.q_head_stride = p.o_head_stride = d
-    p.work_counter_len = 2
+    p.work_counter_len = nat.WORK_COUNTER_WORDS
     n = ctypes.c_int32(0)
     assert nat.lib.fa_plan_splits(ctypes.byref(p), 2, ctypes.byref(n)) == 0
     return n.value
@@ -320,3 +320,126 @@ def test_appended_chunk_with_rotary_on_the_long_sequence_kernels(sq, h, hk, d, r
     assert orc.lse_ok(lse.cpu(), l_ref, 1e-3)[0]
     assert torch.equal(vc_d.cpu(), v_ref)
     assert torch.allclose(kc_d.cpu().float(), k_ref.float(), rtol=1e-3, atol=1e-3)
+
+
+def _kernel():
+    return _nat().last_kernel()
+
+
+@pytest.mark.parametrize("out_layout", ["own", "q_itself", "interleaved_with_q"])
+def test_rotary_chunk_when_out_shares_memory_with_q(out_layout):
+    """The long-sequence path of a chunk appended with rotary parks the rotated q rows in `out` first.  It may do
+    so only when out and q share no memory: with out == q, or out and q as views of one tensor, the kernel that
+    rotates while it loads must run instead (fa_last_kernel says which did) and the results must be the same."""
+    _say("rotary chunk, out layout", out_layout)
+    nat = _nat()
+    dtype, cap, b, sq, h, hk, d = torch.bfloat16, 1500, 4, 128, 64, 8, 128
+    torch.manual_seed(7)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, sq, h, d, dtype=dtype)
+    kn = torch.randn(b, sq, hk, d, dtype=dtype)
+    vn = torch.randn(b, sq, hk, d, dtype=dtype)
+    lens = torch.tensor([cap - sq, 0, 700, 1], dtype=torch.int32)
+    cos, sin = orc.rotary_table(cap, d, dtype=dtype)
+    if out_layout == "interleaved_with_q":
+        both = torch.zeros(b, sq, 2, h, d, dtype=dtype, device=DEV)     # q and out as the two slices of one tensor
+        both[:, :, 0] = q.to(DEV)
+        q_d, out_d = both[:, :, 0], both[:, :, 1]
+    else:
+        q_d = q.to(DEV)
+        out_d = q_d if out_layout == "q_itself" else None
+    out, lse = nat.fwd_kvcache(q_d, kc.to(DEV), vc.to(DEV), kn.to(DEV), vn.to(DEV), lens.to(DEV), cos.to(DEV), sin.to(DEV), None,
+                               out_d, d ** -0.5, True, -1, -1, False, 0)
+    name = _kernel()[0]
+    _say("   kernel", name)
+    assert name == ("pipelined" if out_layout == "own" else "tiled")
+    if out_layout == "interleaved_with_q":
+        assert torch.equal(q_d.cpu(), q)
+    kw = dict(causal=True, rotary_interleaved=False)
+    o_ref, l_ref, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, **kw)
+    o_pt, _, _, _ = orc.kvcache_forward(q, kc, vc, kn, vn, cos, sin, lens, upcast=False, reorder_ops=True, **kw)
+    ok, err, bound = orc.tolerance_ok(out.cpu(), o_ref, o_pt, 3.0, 1e-5)
+    _say("   out err %.3e bound %.3e" % (err, bound))
+    assert ok
+    assert orc.lse_ok(lse.cpu(), l_ref, 1e-3)[0]
+
+
+@pytest.mark.parametrize("sq,h,hk,d,cap,b", [(14, 64, 8, 128, 8192, 32), (1, 16, 16, 64, 32768, 8), (4, 32, 4, 128, 8192, 32)])
+def test_ticket_counters_left_in_use_are_treated_as_fresh(sq, h, hk, d, cap, b):
+    """The ticket-scheduled kernels (decode and tiled) find their counter words as a launch that never finished
+    would leave them -- or as a caller that did not clear them would pass them: non-zero counts under a foreign
+    tag.  The launch must schedule every item all the same (each call tags the counters with a number of its own
+    and takes anything else for zero), match the oracle, and leave the words zero; a second call right after
+    must too.  All kernels run to their normal end: nothing is torn down to set this up, the words are written
+    from the host."""
+    _say("poisoned ticket words", sq, h, hk, d, cap, b)
+    nat = _nat()
+    dtype = torch.bfloat16
+    torch.manual_seed(3 + sq)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, sq, h, d, dtype=dtype)
+    lens = torch.randint(sq, cap + 1, (b,), dtype=torch.int32)
+    lens[0], lens[1], lens[2] = cap, sq, 4096 + 5
+    q_d, kc_d, vc_d, lens_d = q.to(DEV), kc.to(DEV), vc.to(DEV), lens.to(DEV)
+    nat.fwd_kvcache(q_d, kc_d, vc_d, None, None, lens_d, None, None, None, None, d ** -0.5, True, -1, -1, True, 0)   # makes the words
+    name, _, split, _ = _kernel()
+    assert name == ("decode_tickets" if sq * (h // hk) <= 16 else "tiled_tickets") and split, (name, split)
+    torch.cuda.synchronize()
+    key = (torch.cuda.current_device(), nat._stream(q_d.device))
+    words = nat._COUNTERS[key]
+    assert not words[:nat.WORK_COUNTER_WORDS].any()
+    outs = []
+    for poison in ([1000, 0x7eadbeef, 3, 0x7eadbeef], [5, 0, 77, 0], [-1, -1, -1, -1], [0, 0, 0, 0]):
+        words[:4] = torch.tensor(poison, dtype=torch.int32, device=DEV)
+        out, lse = nat.fwd_kvcache(q_d, kc_d, vc_d, None, None, lens_d, None, None, None, None, d ** -0.5, True, -1, -1, True, 0)
+        torch.cuda.synchronize()
+        assert not words[:nat.WORK_COUNTER_WORDS].any(), (poison, words[:4].tolist())
+        outs.append((out.cpu(), lse.cpu()))
+    for o, l in outs[:-1]:           # same items whatever the words held
+        assert (o.float() - outs[-1][0].float()).abs().max().item() < 2e-2
+    for i in (0, 1, 2, b - 1):
+        sl = slice(i, i + 1)
+        o_ref, l_ref, _, _ = orc.kvcache_forward(q[sl], kc[sl], vc[sl], None, None, None, None, lens[sl], causal=True)
+        o_pt, _, _, _ = orc.kvcache_forward(q[sl], kc[sl], vc[sl], None, None, None, None, lens[sl], causal=True,
+                                            upcast=False, reorder_ops=True)
+        for o, l in outs:
+            ok, err, bound = orc.tolerance_ok(o[sl], o_ref, o_pt, 3.0, 1e-5)
+            assert ok, (i, err, bound)
+            assert orc.lse_ok(l[sl], l_ref, 1e-3)[0]
+
+
+@pytest.mark.parametrize("sq,h,hk,b,cap,expect", [
+    (14, 64, 8, 32, 8192, "tiled_tickets"),        # 112 (position, head) rows per kv head, 256 row blocks, long caches
+    (16, 64, 8, 64, 16384, "tiled_tickets"),       # 128 rows, 512 row blocks
+    (112, 8, 8, 32, 8192, "pipelined"),            # the same count of rows as plain query positions: left whole
+    (4, 64, 8, 32, 8192, "tiled_tickets"),
+])
+def test_split_plan_is_the_plan_that_runs(sq, h, hk, b, cap, expect):
+    """fa_plan_splits and the call itself must make the same plan: the caller sizes the partial buffers by the
+    former.  (position, grouped head) rows numbering 96-128 per kv head are the case where the two once differed:
+    the call saw its own already packed problem as plain query rows and left it whole on the general kernel.)"""
+    _say("plan == run", sq, h, hk, b, cap)
+    nat = _nat()
+    dtype, d = torch.bfloat16, 128
+    planned = _planned_splits(nat, b, h, hk, sq, cap, d)
+    torch.manual_seed(1)
+    kc = torch.randn(b, cap, hk, d, dtype=dtype)
+    vc = torch.randn(b, cap, hk, d, dtype=dtype)
+    q = torch.randn(b, sq, h, d, dtype=dtype)
+    lens = torch.randint(cap // 2, cap + 1, (b,), dtype=torch.int32)
+    out, lse = nat.fwd_kvcache(q.to(DEV), kc.to(DEV), vc.to(DEV), None, None, lens.to(DEV), None, None, None, None, d ** -0.5,
+                               True, -1, -1, True, 0)
+    name, _, split, _ = _kernel()
+    _say("   planned %d partial slots; ran %s, split %s" % (planned, name, split))
+    assert name == expect and split == (planned > 1)
+    out, lse = out.cpu(), lse.cpu()
+    for i in (0, b - 1):
+        sl = slice(i, i + 1)
+        o_ref, l_ref, _, _ = orc.kvcache_forward(q[sl], kc[sl], vc[sl], None, None, None, None, lens[sl], causal=True)
+        o_pt, _, _, _ = orc.kvcache_forward(q[sl], kc[sl], vc[sl], None, None, None, None, lens[sl], causal=True,
+                                            upcast=False, reorder_ops=True)
+        ok, err, bound = orc.tolerance_ok(out[sl], o_ref, o_pt, 3.0, 1e-5)
+        assert ok, (i, err, bound)
+        assert orc.lse_ok(lse[sl], l_ref, 1e-3)[0]

@@ -1,16 +1,18 @@
-"""GPU parity tests sized so that the two long-sequence kernels run (not the general 4-wave one and not
-the split path): at least 512 query rows and at least 256 row blocks in the launch.
+"""GPU parity tests sized for the long-sequence kernels (not the general 4-wave one and not the split path), each
+asserting through fa_last_kernel() that the launch reached the kernel the case was written for.  Dispatch as the
+library has it (csrc/fa_prefill_inst.hip), for an unsplit launch of 96+ query rows (32+ above head dim 128):
 
-  * software-pipelined kernel (fa_prefill_il.h): head dim <= 64 at any length, head dim <= 128 up to
-    4096 keys (causal / windowed) or 2048 keys (full attention);
-  * ping-pong kernel (fa_prefill_pp.h): head dim 65..128 beyond those key counts;
-  * the pair form of the software-pipelined kernel (two waves split the head dimension): head dim
-    129..256.
+  * ping-pong kernel (fa_prefill_pp.h): head dim 65..128, keys from 2048 on under a mask / beyond 768 without,
+    more than 256 (masked) / 128 (unmasked) row blocks of 256 rows in the launch, and no window whose two bounds
+    span 768 keys or fewer;
+  * software-pipelined kernel (fa_prefill_il.h): everything else up to head dim 128;
+  * head dim 129..256: one wave per SIMD with the whole head dimension ("wide"), pairs of waves with dropout.
 
-Cases follow the reference's own test dimensions (tests/test_flash_attn.py:530-657, 1295-1402): ragged
-lengths, seqlen_q != seqlen_k both ways, causal / local masks, MQA/GQA, padded head dims, fp16 and
-bf16, strided packed inputs, packed variable-length batches.  Acceptance: the reference's rule
-(max|out - ref| <= 2 max|lowprec - ref| + 1e-5) and log-sum-exp within 1e-3 relative."""
+Launches are made large enough for those thresholds with many query heads on few kv heads; the CPU oracle then checks
+a sample of (batch, head) pairs, which are independent problems.  Cases follow the reference's own test dimensions
+(tests/test_flash_attn.py:530-657, 1295-1402): ragged lengths, seqlen_q != seqlen_k both ways, causal / local masks,
+MQA/GQA, padded head dims, fp16 and bf16, strided packed inputs, packed variable-length batches.  Acceptance: the
+reference's rule (max|out - ref| <= 2 max|lowprec - ref| + 1e-5) and log-sum-exp within 1e-3 relative."""
 import sys
 
 import pytest
@@ -35,6 +37,25 @@ def _fa():
 def _gen(shape, dtype, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype)
+
+
+def _ran(name, head_dims=None, dropout=False):
+    """the last forward launch of this thread took kernel `name` (flash_attn._native.last_kernel)"""
+    from flash_attn import _native as nat
+    got = nat.last_kernel()
+    _say("   kernel", got)
+    assert got[0] == name and got[1] == dropout and not got[2], got
+    if head_dims is not None:
+        assert got[3] == head_dims, got
+
+
+def _check_pairs(out, lse, q, k, v, pairs, **kw):
+    """oracle check of sampled (batch, q head) pairs; k / v heads follow the GQA mapping"""
+    group = q.shape[2] // k.shape[2]
+    for (b, h) in pairs:
+        sl = lambda t, hh: t[b:b + 1, :, hh:hh + 1]
+        _say("   (b=%d, h=%d)" % (b, h))
+        _check(sl(out, h), lse[b:b + 1, h:h + 1], sl(q, h), sl(k, h // group), sl(v, h // group), **kw)
 
 
 def _check(out, lse, q, k, v, **kw):
@@ -66,6 +87,8 @@ def test_pipelined_kernel_square(d, s, mode):
     window = _window(mode, s, d * 1000 + s)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
+    # (without a mask, keys beyond 768 at head dim 65..128 are the ping-pong kernel's)
+    _ran("pingpong" if (mode == "full" and d > 64 and s >= 769) else "pipelined", 64 if d <= 64 else 96 if d <= 96 else 128)
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
@@ -81,50 +104,62 @@ def test_pipelined_kernel_rectangular(sq, sk, dtype, mode):
     window = _window(mode, sk, sq * 7 + sk)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
+    _ran("pipelined", 128)
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
-@pytest.mark.parametrize("case", ["full_2304", "causal_4200", "local_4500", "rect_causal", "rect_local", "d96_full",
-                                  "d96_causal", "d80_local", "d72_rect_causal"])
+# name: (dtype, d, b, h, hk, sq, sk, causal, window); every case has more than 256 row blocks of 256 rows (128 without
+# a mask), 2048+ keys under a mask, and no window narrower than 769 keys
+_PP_CASES = {
+    "full_2304": (torch.bfloat16, 128, 2, 8, 2, 2304, 2304, False, (-1, -1)),
+    "causal_4200": (torch.bfloat16, 128, 1, 16, 2, 4200, 4200, True, (-1, -1)),
+    "local_4500": (torch.bfloat16, 128, 1, 16, 2, 4500, 4500, False, (1000, 300)),
+    "left_only_4500": (torch.bfloat16, 128, 1, 16, 1, 4500, 4500, False, (900, -1)),
+    "rect_causal": (torch.bfloat16, 128, 3, 16, 2, 2000, 4500, True, (-1, -1)),        # sq < sk
+    "rect_causal_tall": (torch.bfloat16, 128, 2, 8, 1, 4300, 2100, True, (-1, -1)),    # sq > sk: leading rows see nothing
+    "rect_local": (torch.bfloat16, 128, 2, 8, 2, 4300, 2100, False, (900, 200)),       # sq > sk, two-sided window
+    "rect_local_wide": (torch.bfloat16, 128, 3, 16, 4, 2000, 4500, False, (1500, 400)),  # sq < sk, two-sided window
+    "ragged_causal": (torch.bfloat16, 128, 3, 16, 2, 1531, 3977, True, (-1, -1)),      # no length a multiple of a tile
+    "fp16_causal": (torch.float16, 128, 1, 16, 2, 4200, 4200, True, (-1, -1)),
+    "fp16_rect_local": (torch.float16, 128, 3, 16, 2, 2000, 4500, False, (1200, 100)),
+    "fp16_full": (torch.float16, 128, 2, 8, 2, 2304, 2304, False, (-1, -1)),
+    "d96_full": (torch.bfloat16, 96, 2, 8, 2, 2100, 2100, False, (-1, -1)),            # head dims 65..96: the 96-column variant
+    "d96_causal": (torch.bfloat16, 96, 1, 16, 2, 4200, 4200, True, (-1, -1)),
+    "d80_local": (torch.bfloat16, 80, 1, 16, 2, 4500, 4500, False, (1000, 300)),
+    "d72_rect_causal": (torch.bfloat16, 72, 3, 16, 2, 2000, 4500, True, (-1, -1)),
+    "d88_fp16_rect_tall_local": (torch.float16, 88, 2, 8, 1, 4300, 2100, False, (1100, 64)),
+    "d104_causal": (torch.bfloat16, 104, 1, 16, 2, 4200, 4200, True, (-1, -1)),        # 97..128: all 128 columns, 104 real
+    "d120_rect_local": (torch.bfloat16, 120, 3, 16, 2, 2000, 4500, False, (1500, 400)),
+}
+
+
+@pytest.mark.parametrize("case", sorted(_PP_CASES))
 def test_pingpong_kernel(case):
     _say("ping-pong", case)
-    dtype = torch.bfloat16
-    d, hk = 128, 2
-    if case == "full_2304":
-        b, h, sq, sk, causal, window = 2, 8, 2304, 2304, False, (-1, -1)
-    elif case == "causal_4200":
-        b, h, sq, sk, causal, window = 1, 8, 4200, 4200, True, (-1, -1)
-    elif case == "local_4500":
-        b, h, sq, sk, causal, window = 1, 8, 4500, 4500, False, (1000, 300)
-    elif case == "rect_causal":
-        b, h, sq, sk, causal, window = 3, 8, 2000, 4500, True, (-1, -1)     # 192 row blocks of 256: more than half the CUs
-    elif case == "rect_local":
-        b, h, sq, sk, causal, window = 2, 8, 4300, 2100, False, (700, 50)      # sq > sk: leading rows see nothing
-    elif case == "d96_causal":       # head dims 65..96 take the kernel's 96-column variant
-        b, h, sq, sk, causal, window, d = 1, 8, 4200, 4200, True, (-1, -1), 96
-    elif case == "d80_local":
-        b, h, sq, sk, causal, window, d = 1, 8, 4500, 4500, False, (1000, 300), 80
-    elif case == "d72_rect_causal":
-        b, h, sq, sk, causal, window, d = 3, 8, 2000, 4500, True, (-1, -1), 72
-    else:
-        b, h, sq, sk, causal, window, d = 2, 8, 2100, 2100, False, (-1, -1), 96
+    dtype, d, b, h, hk, sq, sk, causal, window = _PP_CASES[case]
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal, window_size=window,
                                         return_attn_probs=True)
-    _check(out, lse, q, k, v, causal=causal, window_size=window)
+    _ran("pingpong", 96 if d <= 96 else 128)
+    assert not torch.isnan(out).any()
+    # first and last head of the launch, and one in the middle of a kv group (two pairs in fp16, whose
+    # low-precision CPU run is slow)
+    pairs = [(0, 0), (b - 1, h - 1), (b // 2, h // 2 + 1)]
+    _check_pairs(out, lse, q, k, v, pairs[:2] if dtype == torch.float16 else pairs, causal=causal, window_size=window)
 
 
 @pytest.mark.parametrize("d", [136, 160, 192, 224, 256])
 @pytest.mark.parametrize("sq,sk,mode", [(777, 777, "causal"), (512, 512, "full"), (600, 1500, "causal"),
                                          (1500, 600, "local"), (1024, 1024, "local")])
-def test_pair_kernel_head_dims_above_128(d, sq, sk, mode):
-    _say("pair kernel", d, sq, sk, mode)
+def test_wide_kernel_head_dims_above_128(d, sq, sk, mode):
+    _say("wide kernel", d, sq, sk, mode)
     dtype = torch.float16 if d == 160 and sq <= 777 else torch.bfloat16
     b, h, hk = 4, 16, 2
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
     window = _window(mode, sk, d * 31 + sq)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
+    _ran("wide", 192 if d <= 192 else 256)
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
@@ -136,6 +171,7 @@ def test_long_kernels_take_strided_packed_input(s, d):
     b, h = 2, 16
     qkv = _gen((b, s, 3, h, d), dtype, 5)
     out, lse, _ = _fa().flash_attn_qkvpacked_func(qkv.to(DEV), causal=True, return_attn_probs=True)
+    _ran({64: "pipelined", 128: "pingpong", 256: "wide"}[d])        # (d 128: 9 row blocks x 16 heads x 2 = 288)
     _check(out, lse, qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], causal=True)
 
 
@@ -149,6 +185,7 @@ def test_varlen_long_with_empty_and_tiny_sequences(d):
     q = _gen((total, h, d), dtype, 1); k = _gen((total, h, d), dtype, 2); v = _gen((total, h, d), dtype, 3)
     out, lse, _ = _fa().flash_attn_varlen_func(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), cu.to(DEV), mx, mx,
                                                causal=True, return_attn_probs=True)
+    _ran({64: "pipelined", 128: "pingpong", 256: "wide"}[d])        # (d 128: 9 row blocks x 16 heads x 12 sequences)
     assert out.shape == q.shape and lse.shape == (len(lens), h, mx)
     assert not torch.isnan(out).any()
     for i, L in enumerate(lens):

@@ -131,8 +131,9 @@ def test_device_built_list_is_a_permutation_of_the_row_blocks(lens, h, hk, d):
     dev = q.device
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), nat._stream(dev))
     words = nat._COUNTERS[key].cpu().tolist()
-    assert words[0] == 0 and words[1] == 0                 # the ticket words stay zero
-    counts, body = words[2:10], words[10:]
+    W = nat.WORK_COUNTER_WORDS
+    assert not any(words[:W])                              # the ticket words stay zero
+    counts, body = words[W:W + 8], words[W + 8:]
     block_m = 256 if d == 128 else 128                     # ping-pong kernel / pipelined kernel
     n_mb = [(n + block_m - 1) // block_m for n in lens]
     nmb_max = (mx + block_m - 1) // block_m
