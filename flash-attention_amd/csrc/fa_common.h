@@ -154,6 +154,13 @@ template <int D> FA_DEV int swz_v(int chunk, int row) {
     else return chunk;                       // D == 32: four rows fill the 256 B bank window
 }
 
+// V tiles read by the transposing load in the 16x16x32 geometry: a 16-lane block reads 4 consecutive rows x 2
+// consecutive chunks, the wave 16 rows (8 per half-wave, which must fall into distinct 32-byte bank groups).
+template <int D> FA_DEV int swz_vd(int chunk, int row) {
+    if constexpr (D >= 128) return chunk ^ ((row & 7) << 1);
+    else return chunk ^ (((row >> 1) & 3) << 1);   // D == 64
+}
+
 // One swizzle that serves BOTH read patterns on the same tile (the backward kernels read every
 // streamed tile row-wise as one MFMA operand and transposed as another): a bijection of the rows that
 // share a bank window for the row-wise read, whose upper bits separate the 4 consecutive rows of a

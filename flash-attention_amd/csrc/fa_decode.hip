@@ -18,11 +18,6 @@
 
 namespace fa {
 
-template <int D> FA_DEV int swz_vd(int chunk, int row) {
-    if constexpr (D >= 128) return chunk ^ ((row & 7) << 1);
-    else return chunk ^ (((row >> 1) & 3) << 1);   // D == 64
-}
-
 template <typename T, int D>
 struct DecodeCfg {
     static constexpr int kThreads = 256, kWaves = 4;

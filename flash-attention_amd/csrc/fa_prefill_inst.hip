@@ -1,6 +1,6 @@
 // One translation unit per (dtype, head-dim bucket): compiled with -DFA_T_BF16=0/1 -DFA_D=64/128/256.
 #include "fa_prefill.h"
-#include "fa_prefill_pp.h"
+#include "fa_prefill_pp16.h"
 #include "fa_prefill_il.h"
 #include "fa_launch.h"
 
@@ -39,7 +39,9 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
         // kernel then does less masked-out work (span 128: +16-35 %, 256: +13-18 %, 512: +3-10 %, 1024: -2 %).
         const bool narrow = kp.has_left && kp.has_right && (int64_t)kp.p.window_left + kp.p.window_right <= 768;
         if (FA_D >= 128 && long_keys && (narrow || pp_wgs <= (masked ? 256 : 128))) return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
-        if (FA_D >= 128 && long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
+        if constexpr (FA_D >= 128) {
+            if (long_keys) return launch_prefill_pp<InstT, FA_D, 64>(kp, stream);
+        }
         return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }
 #else

@@ -422,13 +422,4 @@ int launch_prefill_pp_one(KParams kp, hipStream_t stream) {
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
     return note_kernel((int)hipGetLastError(), FA_KERNEL_PINGPONG, DROPOUT, false, DV);
 }
-template <typename T, int D, int BN>
-int launch_prefill_pp(const KParams& kp, hipStream_t stream) {
-    if (kp.p.p_dropout > 0.f) return launch_prefill_pp_one<T, D, BN, true>(kp, stream);
-    if constexpr (D == 128) {
-        if (kp.p.d <= 96) return launch_prefill_pp_one<T, D, BN, false, 96>(kp, stream);
-    }
-    return launch_prefill_pp_one<T, D, BN, false>(kp, stream);
-}
-
 }  // namespace fa

@@ -100,15 +100,16 @@ def test_work_list_words_reported_through_the_c_abi():
     nat = _nat()
     p = nat.FaFwdParams()
     p.b, p.h, p.h_k, p.seqlen_q, p.d = 64, 16, 16, 4096, 128
-    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == 2       # dense batch: no list
+    W = nat.WORK_COUNTER_WORDS
+    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == W       # dense batch: no list
     cu = torch.zeros(65, dtype=torch.int32, device=DEV)
     p.cu_seqlens_q = cu.data_ptr()
-    # 64 sequences x 16 heads x 32 row blocks of 128 rows, two words each, + 8 counts + 2 ticket words
-    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == 2 + 8 + 2 * 64 * 16 * 32
+    # 64 sequences x 16 heads x 32 row blocks of 128 rows, two words each, + 8 counts + the ticket words
+    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == W + 8 + 2 * 64 * 16 * 32
     p.h, p.h_k = 12, 2                                             # 6 q heads per kv head cannot be cut into 8 / h_k parts
-    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == 2
+    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == W
     p.h, p.h_k, p.b = 16, 16, 5000                                 # more sequences than the builder ranks
-    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == 2
+    assert nat.lib.fa_work_list_words(ctypes.byref(p)) == W
 
 
 @pytest.mark.parametrize("lens,h,hk,d", [
