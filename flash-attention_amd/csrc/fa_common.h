@@ -648,15 +648,20 @@ FA_DEV void item_key_range(const KParams& kp, int mode, int idx, int hi, int& c_
 
 // A counter that needs no set-up launch and survives a launch that never finished.  The 64-bit word (two of the
 // caller's int32 words, 8-byte aligned) holds (epoch << 32) | count; `epoch` is a non-zero number the host draws
-// anew for every launch.  A word whose upper half is not this launch's epoch -- zero as every finished launch
-// leaves it, or whatever a launch that was torn down mid-way, or a caller that did not clear the words, left
-// behind -- counts as zero: the first draw that finds it so installs (epoch, 1) with a compare-and-swap and takes
-// value 0, draws that lose that race see the epoch and count on.  Returns the value before the increment.  The
-// usual draw is one atomic add; only the first draws of a launch take the second path, and every path ends after
-// at most one failed compare-and-swap per other lane drawing at that moment (nothing waits for another workgroup).
+// anew, rising, for every call.  A word whose upper half is not this launch's epoch -- zero as every finished
+// launch leaves it, or whatever a launch that was torn down mid-way, or a caller that did not clear the words, left
+// behind -- counts as zero.  The usual draw is one atomic add.  A draw that finds a foreign upper half raises the
+// word to (epoch, 0) with one atomic maximum (idempotent: whoever comes first installs, increments made on the old
+// contents are dropped with them) and draws again; only contents ABOVE the epoch -- a word poisoned from outside,
+// or the replay of an old graph after a younger call was torn down -- need the compare-and-swap loop, which ends
+// after at most one failed attempt per other lane installing at that moment.  Nothing waits for another workgroup.
+// Returns the value before the increment.
 FA_DEV uint32_t epoch_counter_next(int32_t* words, uint32_t epoch) {
     uint64_t* w = reinterpret_cast<uint64_t*>(words);
     uint64_t old = __hip_atomic_fetch_add(w, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((uint32_t)(old >> 32) == epoch) return (uint32_t)old;
+    __hip_atomic_fetch_max(w, (uint64_t)epoch << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __hip_atomic_fetch_add(w, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if ((uint32_t)(old >> 32) == epoch) return (uint32_t)old;
     const uint64_t fresh = ((uint64_t)epoch << 32) | 1u;
     for (;;) {
