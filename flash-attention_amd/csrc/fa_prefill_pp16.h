@@ -410,10 +410,6 @@ int launch_prefill_pp16_one(KParams kp, hipStream_t stream) {
 template <typename T, int D, int BN>
 int launch_prefill_pp(const KParams& kp, hipStream_t stream) {
     if (kp.p.p_dropout > 0.f) return launch_prefill_pp_one<T, D, BN, true>(kp, stream);
-#ifdef FA_PP_32X32      // comparison builds: the 32x32x16 kernel without dropout too
-    if (kp.p.d <= 96 && D == 128) return launch_prefill_pp_one<T, D, BN, false, D == 128 ? 96 : D>(kp, stream);
-    return launch_prefill_pp_one<T, D, BN, false>(kp, stream);
-#endif
     if constexpr (D == 128) {
         if (kp.p.d <= 96) return launch_prefill_pp16_one<T, D, BN, 96>(kp, stream);
     }
