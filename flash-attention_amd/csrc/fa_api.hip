@@ -589,16 +589,11 @@ int fa_rotary(const fa_rotary_params* p, void* hip_stream) {
     if (p->dtype != FA_DTYPE_FP16 && p->dtype != FA_DTYPE_BF16) return fail("rotary only supports fp16 and bf16 data");
     if (p->cs_dtype != FA_DTYPE_FP16 && p->cs_dtype != FA_DTYPE_BF16 && p->cs_dtype != FA_DTYPE_FP32) return fail("cos/sin must be fp16, bf16 or fp32");
     if (p->b < 0 || p->seqlen < 0 || p->h < 0 || p->d <= 0) return fail("negative size");
-    if (p->d % 8 != 0) return fail("head dimension must be a multiple of 8");
     if (p->rotary_dim <= 0 || p->rotary_dim > p->d) return fail("rotary_dim must be <= headdim");
-    if (p->rotary_dim % 16 != 0) return fail("Only rotary dimensions divisible by 16 are currently supported");
+    if (p->rotary_dim % 2 != 0) return fail("rotary_dim must be even");
     if (p->seqlen_ro < 0) return fail("negative table length");
-    // every access is a 16-byte granule of a row (8 bytes for the tables of the interleaved form)
-    const int64_t strides[] = {p->x_batch_stride, p->x_row_stride, p->x_head_stride, p->o_batch_stride,
-                               p->o_row_stride, p->o_head_stride, p->cs_row_stride};
-    for (int64_t s : strides) if (s % 8 != 0) return fail("rotary needs strides that are multiples of 8 elements");
-    const void* ptrs[] = {p->x, p->out, p->cos, p->sin};
-    for (const void* q : ptrs) if ((uintptr_t)q % 16 != 0) return fail("rotary needs 16-byte aligned x, out, cos and sin");
+    // (16-byte granules when rotary_dim is a multiple of 16, the head dim and all strides multiples of 8 elements
+    // and the pointers 16-byte aligned; anything else takes the element-wise kernel)
     if (int e = launch_rotary(*p, (hipStream_t)hip_stream)) return fail_hip(e, "rotary kernel launch");
     return 0;
 }

@@ -118,6 +118,67 @@ __global__ void __launch_bounds__(256) rotary_kernel(const fa_rotary_params p) {
     }
 }
 
+// The general form, for what the granule form cannot address: any even rotary_dim, any head dim, any strides and
+// alignment (the reference's kernel masks its loads instead, flash_attn/ops/triton/rotary.py:81-104).  One work
+// item = one rotated pair, or one column past rotary_dim; 2-byte accesses, so far from the memory roofline, which
+// is why the granule form takes everything it can.  A work item reads both members of its pair before it writes
+// them: safe in place.
+template <typename T, typename CS>
+__global__ void __launch_bounds__(256) rotary_general_kernel(const fa_rotary_params p) {
+    const int rd = p.rotary_dim, half = rd / 2;
+    const bool inplace = p.out == p.x;
+    const int64_t per_row = half + (inplace ? 0 : p.d - rd);
+    const int64_t total = (int64_t)p.b * p.seqlen * p.h * per_row;
+    const float sign = p.conjugate ? -1.f : 1.f;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(idx % per_row);
+        int64_t r = idx / per_row;
+        const int head = (int)(r % p.h); r /= p.h;
+        const int t = (int)(r % p.seqlen);
+        const int b = (int)(r / p.seqlen);
+        int64_t xrow, orow;
+        if (p.cu_seqlens) {
+            const int s0 = p.cu_seqlens[b];
+            if (t >= p.cu_seqlens[b + 1] - s0) continue;
+            xrow = (int64_t)(s0 + t) * p.x_row_stride;
+            orow = (int64_t)(s0 + t) * p.o_row_stride;
+        } else {
+            xrow = (int64_t)b * p.x_batch_stride + (int64_t)t * p.x_row_stride;
+            orow = (int64_t)b * p.o_batch_stride + (int64_t)t * p.o_row_stride;
+        }
+        const T* x = reinterpret_cast<const T*>(p.x) + xrow + (int64_t)head * p.x_head_stride;
+        T* o = reinterpret_cast<T*>(p.out) + orow + (int64_t)head * p.o_head_stride;
+        if (c >= half) {                                             // columns past rotary_dim
+            o[rd + (c - half)] = x[rd + (c - half)];
+            continue;
+        }
+        const int i0 = p.interleaved ? 2 * c : c, i1 = p.interleaved ? 2 * c + 1 : c + half;
+        const int pos = t + (p.seqlen_offsets ? p.seqlen_offsets[b] : p.seqlen_offset);
+        float cs = 1.f, sn = 0.f;
+        if (pos >= 0 && pos < p.seqlen_ro) {                         // past the table: identity
+            cs = (float)reinterpret_cast<const CS*>(p.cos)[(int64_t)pos * p.cs_row_stride + c];
+            sn = sign * (float)reinterpret_cast<const CS*>(p.sin)[(int64_t)pos * p.cs_row_stride + c];
+        }
+        const float x0 = (float)x[i0], x1 = (float)x[i1];
+        o[i0] = (T)(x0 * cs - x1 * sn);
+        o[i1] = (T)(x0 * sn + x1 * cs);
+    }
+}
+
+template <typename T>
+static int launch_rotary_general(const fa_rotary_params& p, hipStream_t stream) {
+    const int64_t per_row = p.rotary_dim / 2 + (p.out == p.x ? 0 : p.d - p.rotary_dim);
+    const int64_t total = (int64_t)p.b * p.seqlen * p.h * per_row;
+    if (total <= 0) return 0;
+    const dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 256 * 32)), block(256);
+    switch (p.cs_dtype) {
+        case FA_DTYPE_FP16: hipLaunchKernelGGL((rotary_general_kernel<T, _Float16>), grid, block, 0, stream, p); break;
+        case FA_DTYPE_BF16: hipLaunchKernelGGL((rotary_general_kernel<T, __bf16>), grid, block, 0, stream, p); break;
+        default: hipLaunchKernelGGL((rotary_general_kernel<T, float>), grid, block, 0, stream, p); break;
+    }
+    return (int)hipGetLastError();
+}
+
 template <typename T, typename I, bool STREAM>
 static void launch_rotary_is(const fa_rotary_params& p, dim3 grid, hipStream_t stream) {
     const dim3 block(256);
@@ -149,7 +210,20 @@ static int launch_rotary_t(const fa_rotary_params& p, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// every access of the granule form is a 16-byte piece of a row (8 bytes for the tables of the interleaved form)
+static bool rotary_granules_apply(const fa_rotary_params& p) {
+    if (p.d % 8 != 0 || p.rotary_dim % 16 != 0) return false;
+    const int64_t strides[] = {p.x_batch_stride, p.x_row_stride, p.x_head_stride, p.o_batch_stride,
+                               p.o_row_stride, p.o_head_stride, p.cs_row_stride};
+    for (int64_t s : strides) if (s % 8 != 0) return false;
+    const void* ptrs[] = {p.x, p.out, p.cos, p.sin};
+    for (const void* q : ptrs) if ((uintptr_t)q % 16 != 0) return false;
+    return true;
+}
+
 int launch_rotary(const fa_rotary_params& p, hipStream_t stream) {
+    if (!rotary_granules_apply(p))
+        return p.dtype == FA_DTYPE_BF16 ? launch_rotary_general<__bf16>(p, stream) : launch_rotary_general<_Float16>(p, stream);
     return p.dtype == FA_DTYPE_BF16 ? launch_rotary_t<__bf16>(p, stream) : launch_rotary_t<_Float16>(p, stream);
 }
 

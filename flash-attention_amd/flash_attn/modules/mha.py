@@ -114,9 +114,8 @@ class MHA(nn.Module):
         self.head_dim = self.embed_dim // num_heads
         qkv_dim = self.head_dim * (self.num_heads + 2 * self.num_heads_kv)
         if self.rotary_emb_dim > 0:
-            # the rotary kernels (stand-alone and inside the KV-cache call) move 16-byte granules of a pair
-            if self.rotary_emb_dim % 16 != 0 or self.rotary_emb_dim > self.head_dim:
-                raise ValueError("rotary_emb_dim must be divisible by 16 and at most head_dim (got %d for head_dim %d)"
+            if self.rotary_emb_dim % 2 != 0 or self.rotary_emb_dim > self.head_dim:
+                raise ValueError("rotary_emb_dim must be even and at most head_dim (got %d for head_dim %d)"
                                  % (self.rotary_emb_dim, self.head_dim))
             self.rotary_emb = RotaryEmbedding(self.rotary_emb_dim, base=rotary_emb_base, scale_base=rotary_emb_scale_base,
                                               interleaved=rotary_emb_interleaved, device=device)
@@ -219,8 +218,11 @@ class MHA(nn.Module):
             rotary_max_seqlen = inference_params.max_seqlen
         batch, seqlen = x.shape[:2]
         qkv = self.Wqkv(x)
-        # the fused rotary + append path needs something cached
-        fused = inference_params is not None and inference_params.seqlen_offset > 0 and self.rotary_emb_dim > 0
+        # The fused rotary + append path needs something cached, and a rotary dimension the KV-cache call rotates
+        # (multiples of 16, as in the reference, csrc/flash_attn/flash_api.cpp:1212); other rotary dimensions are
+        # rotated by the stand-alone op at each sequence's length and appended by the same call without tables.
+        fused = (inference_params is not None and inference_params.seqlen_offset > 0 and self.rotary_emb_dim > 0
+                 and self.rotary_emb_dim % 16 == 0)
         if self.num_heads_kv == self.num_heads:
             qkv = qkv.view(batch, seqlen, 3, self.num_heads, self.head_dim)
             if fused:

@@ -3,7 +3,9 @@ generates, token selection, the token loop, and replay of one decoding step from
 
 Covers what the reference keeps in flash_attn/utils/generation.py on the attention path:
 `InferenceParams` (:18-35), the top-k / top-p helpers and `sample` (:40-97), `decode` (:100-201) with
-the same arguments and result type, and the graph cache behind `cg=True` (:604-739).  A "model" is
+the same arguments and result type, speculative decoding (`sample_speculative`, `decode_speculative`, :204-558),
+`GenerationMixin` (:561-582), and the graph cache behind `cg=True` (:604-739) with its public names
+(`DecodingCGCache`, `update_graph_cache`, `capture_graph`).  A "model" is
 any callable `model(input_ids, position_ids=None, inference_params=None, num_last_tokens=0)` whose
 result has a `.logits` tensor of shape (batch, tokens, vocab), as the reference's GPT models do.
 
@@ -84,6 +86,43 @@ def sample(logits, top_k=1, top_p=0.0, temperature=1.0):
     scaled = logits / temperature if temperature != 1.0 else logits.clone()
     modify_logits_for_top_p_filtering(scaled, top_p)
     return _draw(scaled)
+
+
+def _filtered_probs(logits, top_k, top_p, temperature):
+    """softmax of a copy of `logits` after temperature, the top-k cut and the top-p cut"""
+    logits = logits / temperature if temperature != 1.0 else logits.clone()
+    if top_k > 0:
+        modify_logits_for_top_k_filtering(logits, min(top_k, logits.shape[-1]))
+    modify_logits_for_top_p_filtering(logits, top_p)
+    return logits.softmax(dim=-1)
+
+
+def sample_speculative(logits, logits_draft, tokens_draft, top_k=1, top_p=0.0, temperature=1.0):
+    """Speculative sampling (Leviathan, Kalman, Matias: Fast Inference from Transformers via Speculative
+    Decoding, algorithm 1; the reference's function of the same name, flash_attn/utils/generation.py:204-262).
+    logits (batch, n + 1, vocab) are the verifying model's at the n drafted positions and one more,
+    logits_draft (batch, n, vocab) the drafting model's, tokens_draft (batch, n) what it drew.  A drafted token is
+    kept with probability min(1, p / p_draft); the first one that is not kept is drawn again from the positive part
+    of p - p_draft, and when all are kept one more token is drawn from the last position.  Returns tokens
+    (batch, n + 1) and how many of them count, (batch,) values in [1, n + 1]."""
+    batch, n1, vocab = logits.shape
+    n = n1 - 1
+    assert logits_draft.shape == (batch, n, vocab) and tokens_draft.shape == (batch, n)
+    assert tokens_draft.dtype in (torch.int64, torch.int32)
+    if top_p > 0.0:
+        assert top_p <= 1.0, "top-p should be in (0, 1]."
+    p = _filtered_probs(logits, top_k, top_p, temperature)
+    q = _filtered_probs(logits_draft, top_k, top_p, temperature)
+    drawn = tokens_draft.long().unsqueeze(-1)
+    p_tok, q_tok = p[:, :n].gather(-1, drawn).squeeze(-1), q.gather(-1, drawn).squeeze(-1)
+    kept = torch.rand(batch, n, device=p.device) * q_tok <= p_tok
+    # index of the first token that is not kept, n when all are
+    n_kept = torch.cat([kept, torch.zeros(batch, 1, dtype=torch.bool, device=p.device)], dim=1).int().argmin(dim=-1)
+    redraw_from = torch.cat([(p[:, :n] - q).clamp_(min=0.0), p[:, n:]], dim=1)          # (batch, n + 1, vocab)
+    row = redraw_from.gather(1, n_kept.view(batch, 1, 1).expand(batch, 1, vocab)).squeeze(1)
+    redrawn = torch.multinomial(row, num_samples=1)                                       # unnormalised weights are fine
+    tokens = torch.nn.functional.pad(tokens_draft, (0, 1)).scatter(1, n_kept.unsqueeze(1), redrawn.to(tokens_draft.dtype))
+    return tokens, n_kept + 1
 
 
 # ------------------------------------------------------------------------------------------------
@@ -257,3 +296,144 @@ def decode(input_ids, model, max_length, top_k=1, top_p=0.0, temperature=1.0, eo
         print(f"Prompt processing + decoding time: {clock[0].elapsed_time(clock[1]):.0f}ms")
     result = GreedySearchDecoderOnlyOutput if top_k == 1 else SampleDecoderOnlyOutput
     return result(sequences=torch.cat(pieces, dim=1), scores=tuple(scores))
+
+
+# ------------------------------------------------------------------------------------------------
+# the reference's names for the graph cache (flash_attn/utils/generation.py:605-739)
+# ------------------------------------------------------------------------------------------------
+DecodingCGCache = GraphedDecoder
+
+
+def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, decoding_seqlens=(1,), tensor_parallel=1,
+                       dtype=None, n_warmups=2):
+    """The model's decoder cache with a captured step for every count of new tokens in `decoding_seqlens`: `cache`
+    itself when it fits the request, else a new one.  `cache.run(input_ids, position_ids, seqlen)` then replays the
+    step for input_ids' shape with `seqlen` tokens already cached."""
+    if not isinstance(cache, GraphedDecoder) or not cache.fits(model, batch_size, max_seqlen, dtype):
+        cache = None                                  # let the old caches and graphs go first
+        cache = GraphedDecoder(model, batch_size, max_seqlen, dtype, tensor_parallel)
+    for n_tokens in decoding_seqlens:
+        cache.step(batch_size, n_tokens)
+    return cache
+
+
+def capture_graph(model, inference_params, batch_size, max_seqlen, decoding_seqlen=1, mempool=None, n_warmups=2):
+    """One captured step of `decoding_seqlen` new tokens per sequence against the caches in `inference_params`
+    (whose `lengths_per_sample` the replays read); returns run(input_ids, position_ids, seqlen) -> logits."""
+    with torch.inference_mode():
+        step = DecodeStepGraph(model, inference_params, batch_size, decoding_seqlen, mempool, n_warmups)
+    return lambda new_input_ids, new_position_ids, seqlen: step.run(new_input_ids, new_position_ids, seqlen)
+
+
+# ------------------------------------------------------------------------------------------------
+# speculative decoding
+# ------------------------------------------------------------------------------------------------
+class _Reader:
+    """A model reading one growing token sequence through its KV cache.  `seen` tokens of the sequence are in the
+    cache; `read(ctx, keep)` feeds it the tokens of ctx it has not seen and returns the logits of the last `keep`
+    positions fed.  Taking tokens back is setting `seen` lower: later calls overwrite the cache rows."""
+
+    def __init__(self, model, max_length, use_graph, graph_seqlens):
+        self.model = model
+        self.graphs = None
+        if use_graph:
+            model._decoding_cache = update_graph_cache(model, getattr(model, "_decoding_cache", None), 1, 0, max_length,
+                                                       decoding_seqlens=graph_seqlens)
+            self.graphs = model._decoding_cache
+            self.state = self.graphs.inference_params
+            self.state.reset(max_length, 1)
+        else:
+            self.state = InferenceParams(max_seqlen=max_length, max_batch_size=1)
+        self.seen = 0
+
+    def read(self, ctx, keep=1):
+        new = ctx[:, self.seen:]
+        n = new.shape[1]
+        assert n >= keep >= 1
+        self.state.seqlen_offset = self.seen
+        if self.seen == 0:
+            if self.state.lengths_per_sample is not None:
+                self.state.lengths_per_sample.zero_()
+            logits = self.model(new, position_ids=None, inference_params=self.state, num_last_tokens=keep).logits
+        else:
+            positions = self.seen + torch.arange(n, dtype=torch.long, device=ctx.device).unsqueeze(0)
+            if self.graphs is not None and (1, n) in self.graphs.steps:
+                logits = self.graphs.run(new, positions, self.seen)[:, -keep:]
+            else:
+                if self.state.lengths_per_sample is not None:
+                    self.state.lengths_per_sample.fill_(self.seen)
+                logits = self.model(new, position_ids=positions, inference_params=self.state, num_last_tokens=keep).logits
+        self.seen += n
+        self.state.seqlen_offset = self.seen
+        return logits
+
+
+@torch.inference_mode()
+def decode_speculative(input_ids, model, model_draft, max_length, speculative_lookahead=3, top_k=1, top_p=0.0,
+                       temperature=1.0, eos_token_id=None, vocab_size=None, tensor_parallel=1, cg=False,
+                       enable_timing=False, debug=False):
+    """Speculative decoding of one sequence (batch 1, as the reference's, flash_attn/utils/generation.py:265-558):
+    `model_draft` proposes up to `speculative_lookahead` tokens one by one, `model` reads them all in ONE call -- a
+    few query positions against its cache, the case the KV-cache attention call packs into one row block -- and
+    `sample_speculative` decides how many stand.  Greedy (top_k = 1) output is the output of `decode` with `model`
+    alone.  Returns sequences (1, <= max_length) and scores (1, generated, vocab): the verifying model's logits each
+    new token was taken from."""
+    assert input_ids.shape[0] == 1, "Speculative decoding implementation only supports batch_size=1"
+    assert eos_token_id is None, "Speculative decoding implementation doesn't support eos_token_id"
+    assert tensor_parallel == 1, "one GPU: tensor parallel decoding is not part of this build"
+    cut = (lambda x: x[..., :vocab_size]) if vocab_size is not None else (lambda x: x)
+    main = _Reader(model, max_length, cg, range(1, speculative_lookahead + 2))
+    draft = _Reader(model_draft, max_length, cg, (1, 2))
+    clock = None
+    if enable_timing:
+        clock = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        clock[0].record()
+    ctx, scores = input_ids, []
+    calls = drafted = stood = 0
+    while ctx.shape[1] < max_length:
+        n = min(speculative_lookahead, max_length - ctx.shape[1] - 1)
+        if n <= 0:                                   # room for one token: no draft
+            logits = cut(main.read(ctx, 1))
+            scores.append(logits)
+            ctx = torch.cat([ctx, sample(logits[:, -1], top_k, top_p, temperature).unsqueeze(1)], dim=1)
+            calls += 1
+            break
+        base = ctx.shape[1]
+        proposal, logits_draft = ctx, []
+        for _ in range(n):
+            logits_draft.append(cut(draft.read(proposal, 1))[:, -1])
+            proposal = torch.cat([proposal, sample(logits_draft[-1], top_k, top_p, temperature).unsqueeze(1)], dim=1)
+        logits = cut(main.read(proposal, n + 1))                          # (1, n + 1, vocab)
+        calls += 1
+        tokens, counted = sample_speculative(logits, torch.stack(logits_draft, dim=1), proposal[:, base:], top_k, top_p, temperature)
+        g = int(counted[0])
+        drafted, stood = drafted + n, stood + g - 1
+        ctx = torch.cat([ctx, tokens[:, :g]], dim=1)
+        scores.append(logits[:, :g])
+        # what each model has read of the new sequence: the drafts that stood (the redrawn or extra token is new to both)
+        main.seen = base + g - 1
+        draft.seen = min(draft.seen, base + g - 1)
+        if debug:
+            print("drafted %d, %d stood" % (n, g - 1))
+    if clock is not None:
+        clock[1].record()
+        torch.cuda.synchronize()
+        print(f"Prompt processing + decoding time: {clock[0].elapsed_time(clock[1]):.0f}ms")
+        print(f"Number of calls to main model: {calls}")
+        print(f"Acceptance rate: {100.0 * stood / max(drafted, 1):.2f}%")
+    result = GreedySearchDecoderOnlyOutput if top_k == 1 else SampleDecoderOnlyOutput
+    return result(sequences=ctx, scores=torch.cat(scores, dim=1))
+
+
+class GenerationMixin:
+    """`generate` for a model class, through `decode` (the reference's mixin, flash_attn/utils/generation.py:561-582)"""
+
+    def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None, **kwargs):
+        raise NotImplementedError
+
+    def generate(self, input_ids, max_length, top_k=1, top_p=0.0, temperature=1.0, return_dict_in_generate=False,
+                 output_scores=False, **kwargs):
+        output = decode(input_ids, self, max_length, top_k=top_k, top_p=top_p, temperature=temperature, **kwargs)
+        if not output_scores:
+            output = output._replace(scores=None)
+        return output if return_dict_in_generate else output.sequences

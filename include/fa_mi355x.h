@@ -247,7 +247,9 @@ int32_t fa_sizeof_params(void);
  *                 positions outside the table leave the row unrotated
  *   interleaved   pairs (2i, 2i+1) instead of (i, i + rotary_dim/2)
  *   conjugate     rotate by -angle (the backward of the operation)
- * d % 8 == 0, rotary_dim % 16 == 0, rotary_dim <= d.
+ * Any even rotary_dim <= d, any d, any strides, as the reference's op (flash_attn/ops/triton/rotary.py:176-208).
+ * The memory-bound form with 16-byte accesses runs when rotary_dim is a multiple of 16, d and all strides are
+ * multiples of 8 elements and x, out, cos, sin are 16-byte aligned; other shapes take an element-wise kernel.
  */
 typedef struct fa_rotary_params {
     const void *x;

@@ -56,16 +56,12 @@ def _model(heads_kv, rotary_dim, dtype=torch.float16, seed=0):
 def test_mha_layer_matches_oracle(heads_kv, rotary_dim):
     """One layer, no cache: projection in torch, rotary + causal attention through the package; the
     same computed with the oracle's rotary and attention on the CPU.  rotary_dim = 24 is not a
-    multiple of 16 (the standalone kernel's granule) and must be rejected with a clear error."""
+    multiple of 16 (the granule of the memory-bound rotary kernel): the element-wise kernel takes it."""
     from flash_attn.modules.mha import MHA
     _say("mha layer", heads_kv, rotary_dim)
     torch.manual_seed(1)
     dtype, b, s, dim, h = torch.float16, 2, 150, 256, 4
     d = dim // h
-    if rotary_dim == 24:
-        with pytest.raises(ValueError, match="divisible by 16"):
-            MHA(dim, h, num_heads_kv=heads_kv, causal=True, layer_idx=0, rotary_emb_dim=rotary_dim, device=DEV, dtype=dtype)
-        return
     layer = MHA(dim, h, num_heads_kv=heads_kv, causal=True, layer_idx=0, rotary_emb_dim=rotary_dim, device=DEV, dtype=dtype)
     x = torch.randn(b, s, dim, device=DEV, dtype=dtype)
     with torch.no_grad():
@@ -87,10 +83,11 @@ def test_mha_layer_matches_oracle(heads_kv, rotary_dim):
 
 
 @pytest.mark.parametrize("heads_kv", [4, 2])
-@pytest.mark.parametrize("rotary_dim", [0, 32])
+@pytest.mark.parametrize("rotary_dim", [0, 32, 24])
 def test_incremental_decoding_matches_full_forward(heads_kv, rotary_dim):
     """Teacher-forced decode: logits of step t from the cache paths (prompt pass, then the fused
-    rotary + append + attend call per token) against one full forward over the whole sequence."""
+    rotary + append + attend call per token; rotary dimension 24, which that call does not rotate, goes through
+    the stand-alone rotary op at each sequence's length) against one full forward over the whole sequence."""
     from flash_attn.utils.generation import decode
     _say("incremental", heads_kv, rotary_dim)
     model = _model(heads_kv, rotary_dim)
@@ -247,3 +244,71 @@ def test_mha_trains_with_dropout():
         grads.append([p.grad.clone() for p in layer.parameters()])
     for a, b in zip(*grads):
         assert torch.isfinite(a).all() and torch.equal(a, b)
+
+
+@pytest.mark.parametrize("cg", [False, True])
+@pytest.mark.parametrize("same_draft", [False, True])
+@pytest.mark.parametrize("heads_kv,rotary_dim", [(4, 32), (1, 0)])
+def test_speculative_decoding_reproduces_greedy_decoding(heads_kv, rotary_dim, same_draft, cg):
+    """Greedy speculative decoding must give the verifying model's own greedy continuation, whatever the drafting
+    model proposes (a different random model: most drafts are thrown away; the model itself: all stand and every
+    call of the verifier reads lookahead + 1 positions against its cache, the few-positions form of the KV-cache
+    attention call).  With cg the single- and multi-token steps replay captured graphs."""
+    from flash_attn.utils.generation import decode, decode_speculative
+    _say("speculative", heads_kv, rotary_dim, same_draft, cg)
+    model = _model(heads_kv, rotary_dim)
+    draft = model if same_draft else _model(heads_kv, rotary_dim, seed=5)
+    g = torch.Generator().manual_seed(4)
+    prompt, total = 19, 60
+    ids = torch.randint(0, 211, (1, prompt), generator=g).to(DEV)
+    plain = decode(ids, model, total)
+    for lookahead in (1, 3, 4):
+        spec = decode_speculative(ids, model, draft, total, speculative_lookahead=lookahead, cg=cg)
+        assert spec.sequences.shape == (1, total)
+        # positions where the plain run's top two logits are closer than the error between one-token and
+        # several-token evaluation may legitimately differ; everything up to the first such position must agree
+        gaps = torch.stack([s.float().topk(2, dim=-1).values for s in plain.scores], 1)[0]
+        close = ((gaps[:, 0] - gaps[:, 1]) < 2e-2).nonzero()
+        upto = total if close.numel() == 0 else prompt + int(close[0])
+        assert torch.equal(spec.sequences[:, :upto], plain.sequences[:, :upto]), lookahead
+        assert spec.scores.shape[:2] == (1, total - prompt)
+        if upto == total:
+            ref = torch.stack(list(plain.scores), 1).float()
+            assert (spec.scores.float() - ref).abs().max().item() < 2e-2 * max(1.0, ref.abs().max().item())
+
+
+def test_generation_mixin_and_graph_cache_names():
+    """`GenerationMixin.generate`, `update_graph_cache` / `DecodingCGCache` / `capture_graph` as the reference names
+    them (flash_attn/utils/generation.py:561-582, 605-739)."""
+    from flash_attn.utils import generation as gen
+
+    class Mixed(ToyLM, gen.GenerationMixin):
+        pass
+    torch.manual_seed(0)
+    model = Mixed(vocab=211, dim=256, heads=4, heads_kv=2, layers=2, rotary_dim=32, dtype=torch.float16).eval()
+    ids = torch.randint(0, 211, (2, 11), generator=torch.Generator().manual_seed(1)).to(DEV)
+    seqs = model.generate(ids, 30)
+    assert torch.is_tensor(seqs) and seqs.shape == (2, 30) and torch.equal(seqs[:, :11], ids)
+    out = model.generate(ids, 30, return_dict_in_generate=True, output_scores=True)
+    assert torch.equal(out.sequences, seqs) and len(out.scores) == 19
+    assert model.generate(ids, 30, return_dict_in_generate=True).scores is None
+    graphed = model.generate(ids, 30, cg=True)
+    assert torch.equal(graphed, seqs)
+    cache = gen.update_graph_cache(model, None, 2, 11, 40, decoding_seqlens=(1, 3))
+    assert isinstance(cache, gen.DecodingCGCache) and set(cache.steps) == {(2, 1), (2, 3)}
+    assert gen.update_graph_cache(model, cache, 2, 11, 40) is cache             # fits: kept
+    assert gen.update_graph_cache(model, cache, 2, 11, 80) is not cache         # longer sequences: rebuilt
+    # a captured three-token step against an eager one on the same cache contents
+    state = cache.inference_params
+    with torch.inference_mode():
+        state.reset(40, 2)
+        model(ids, inference_params=state, num_last_tokens=1)
+        state.seqlen_offset = 11
+        new = torch.randint(0, 211, (2, 3), generator=torch.Generator().manual_seed(2)).to(DEV)
+        pos = 11 + torch.arange(3, device=DEV).expand(2, 3)
+        replayed = cache.run(new, pos, 11)
+        state.lengths_per_sample.fill_(11)
+        eager = model(new, position_ids=pos, inference_params=state, num_last_tokens=3).logits
+        assert (replayed.float() - eager.float()).abs().max().item() < 2e-2
+        run = gen.capture_graph(model, state, 2, 40, decoding_seqlen=3, mempool=cache.pool)
+        assert (run(new, pos, 11).float() - eager.float()).abs().max().item() < 2e-2

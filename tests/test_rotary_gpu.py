@@ -304,3 +304,62 @@ def test_rotary_positions_past_the_table_pass_through():
     want = orc.rotary_apply(x, cos, sin, pos.clamp(max=s - 1), False)
     want[1, s - 40:] = x[1, s - 40:]
     _close(out, want, "out")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d,rd", [(64, 24), (128, 42), (80, 80), (36, 36), (100, 50), (64, 2), (256, 200), (30, 30)])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("inplace", [False, True])
+def test_rotary_any_even_dim_and_any_head_dim(d, rd, interleaved, inplace, dtype):
+    """Rotary dimensions that are even but not multiples of 16, head dims that are not multiples of 8 (so rows
+    start at odd 4-byte offsets), as the reference's op takes them (flash_attn/ops/triton/rotary.py:176-208; its
+    test grid has rotary fractions 1.0 and 0.5 of head dims 128: tests/test_rotary.py:46-50).  These take the
+    element-wise kernel; forward with per-sequence offsets, and the gradient (the inverse rotation)."""
+    from flash_attn.layers.rotary import apply_rotary_emb
+    _say("rotary general", d, rd, interleaved, inplace, dtype)
+    b, s, h = 3, 77, 5
+    g = torch.Generator().manual_seed(d + rd)
+    x = torch.randn(b, s, h, d, generator=g).to(dtype)
+    cos, sin = _table(s + 40, rd, dtype, 8)
+    offsets = torch.tensor([0, 13, 40], dtype=torch.int32)
+    xd = x.to(DEV).clone().requires_grad_(not inplace)
+    out = apply_rotary_emb(xd, cos.to(DEV), sin.to(DEV), seqlen_offsets=offsets.to(DEV), interleaved=interleaved, inplace=inplace)
+    pos = _positions(offsets, b, s)
+    want = orc.rotary_apply(x, cos, sin, pos, interleaved)
+    _close(out.detach(), want, "out")
+    if inplace:
+        assert out.data_ptr() == xd.data_ptr()
+    else:
+        assert torch.equal(xd.detach().cpu(), x)
+        go = torch.randn(b, s, h, d, generator=g).to(dtype)
+        (gx,) = torch.autograd.grad(out, xd, go.to(DEV))
+        # the gradient of a rotation is the rotation by the opposite angle
+        _close(gx, orc.rotary_apply(go, cos, -sin, pos, interleaved), "grad")
+
+
+def test_rotary_general_kernel_on_packed_and_strided_input():
+    """the element-wise kernel with packed variable-length rows and with x as a view whose strides are not
+    multiples of 8 elements (a slice of a wider tensor)"""
+    from flash_attn.layers.rotary import apply_rotary_emb
+    _say("rotary general packed / strided")
+    h, d, rd = 3, 44, 20
+    lens = [5, 0, 31, 1, 18]
+    cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(int(cu[-1]), h, d, generator=g).to(torch.float16)
+    cos, sin = _table(max(lens), rd, torch.float16, 3)
+    out = apply_rotary_emb(x.to(DEV), cos.to(DEV), sin.to(DEV), interleaved=True, cu_seqlens=cu.to(DEV), max_seqlen=max(lens))
+    for i, L in enumerate(lens):
+        if L:
+            a = int(cu[i])
+            want = orc.rotary_apply(x[a:a + L][None], cos, sin, torch.arange(L)[None], True)
+            _close(out[a:a + L][None], want, "sequence %d" % i)
+    wide = torch.randn(2, 50, 4, 67, generator=g).to(torch.bfloat16)      # row stride 4 * 67, head stride 67
+    xs = wide[..., 3:3 + 64]
+    cos, sin = _table(50, 32, torch.bfloat16, 4)
+    out = apply_rotary_emb(xs.to(DEV)[...], cos.to(DEV), sin.to(DEV))
+    wide_d = wide.to(DEV)
+    out2 = apply_rotary_emb(wide_d[..., 3:3 + 64], cos.to(DEV), sin.to(DEV))
+    want = orc.rotary_apply(xs, cos, sin, _positions(0, 2, 50), False)
+    _close(out, want, "contiguous copy")
+    _close(out2, want, "strided view")
