@@ -8,8 +8,9 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
                 (the configuration the headline metric is quoted on); value = TFLOP/s with the
                 reference's FLOP convention 4*b*s^2*h*d/2 (benchmarks/benchmark_flash_attention.py:27-30);
   * decode   -- flash_attn_with_kvcache, bf16, batch 64, 1 new token appended with rotary, caches
-                (64, 32768, 8, 128), 64 query heads, cache_seqlens uniform in [1024, 32767];
-                reported as achieved HBM GB/s over the algorithmic bytes.
+                (64, 32768, 8, 128), 64 query heads, cache_seqlens uniform in [1024, 32767] at the start of
+                every timed block and one longer after every step (a decoding loop: each step appends where
+                the last one stopped); reported as achieved HBM GB/s over the algorithmic bytes.
   * rotary   -- apply_rotary_emb in place on (8, 8192, 32, 128) bf16 (the standalone rotary kernel), GB/s
                 over 2 x the tensor's bytes;
   * backward -- gradients of the prefill workload (rowsum(dO o O), dQ pass, dK/dV pass); reported under
@@ -21,6 +22,8 @@ One "step" is one forward pass over one synthetic batch already resident in HBM:
                 (seed 0), 16 heads, head dim 128 and 256, causal; FLOPs over the visible (row, key) pairs;
   * gqa_window -- flash_attn_func, bf16, batch 2, seqlen 16384, 32 query / 8 kv heads, head dim 128, causal
                 with window (4096, 0); FLOPs over the visible pairs (sum_i min(i + 1, 4097) per head);
+  * config1  -- flash_attn_func, fp16, batch 2, seqlen 512, 8 heads, head dim 64, non-causal (the reference's own
+                CPU-runnable case): 1 GFLOP per call, so what is measured is the latency of one launch;
 Prints ONE JSON line.  The CPU baseline is the oracle (a restatement of the reference's
 attention_ref) timed on the host cores on a bounded sample of the same workload.
 """
@@ -60,15 +63,22 @@ class Timing(tuple):
         return t
 
 
-def time_steps(fn, steps, warmup):
+def time_steps(fn, steps, warmup, before_block=None):
     """`warmup` untimed calls, then BLOCKS blocks of exactly `steps` calls, each bracketed by HIP events
-    on the stream the kernels are launched on (torch's current stream) and by a device synchronisation."""
+    on the stream the kernels are launched on (torch's current stream) and by a device synchronisation.
+    `before_block` runs (untimed) ahead of the warm-up and of every block: a workload whose steps move its
+    state puts the state back there."""
     import torch
+    if before_block is not None:
+        before_block()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     blocks = []
     for _ in range(BLOCKS):
+        if before_block is not None:
+            before_block()
+            torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
@@ -99,7 +109,7 @@ def bench_prefill(steps, warmup):
         "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                     "kernel": "fa::prefill_pp_kernel<bf16,128,64>", "flops_per_launch": flops},
+                     "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>", "flops_per_launch": flops},
     }
 
 
@@ -111,7 +121,7 @@ def bench_head_dims(steps, warmup):
     import flash_attn
     b, s, h = 4, 8192, 32
     res = {}
-    for d, kern in ((96, "fa::prefill_pp_kernel<bf16,128,64,false,96>"), (192, "fa::prefill_il_kernel<bf16,ILCfg<bf16,256,32,192>>")):
+    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96>"), (192, "fa::prefill_il_kernel<bf16,ILCfg<bf16,256,32,192>>")):
         torch.manual_seed(0)
         q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
         with torch.no_grad():
@@ -124,7 +134,9 @@ def bench_head_dims(steps, warmup):
         res["d%d" % d] = {
             "ms": tm[0], "ms_min": tm.ms_min, "tflops": tf,
             "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS,
-                         "traffic": None, "kernel": kern, "flops_per_launch": flops},
+                         "traffic": _traffic("head_dim_%d_bf16_causal_8k" % d),
+                         "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
+                         "kernel": kern, "flops_per_launch": flops},
             "backward": {"ms": tb[0], "ms_min": tb.ms_min, "tflops": tfb, "frac": tfb / PEAK_BF16_TFLOPS},
         }
         del q, k, v, o, do
@@ -250,7 +262,8 @@ def bench_backward(steps, warmup):
         "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops,
         "workload": "flash_attn_func bwd bf16 batch=4 seqlen=8192 nheads=32 headdim=128 causal (dot + dQ + dK/dV kernels)",
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("backward_bf16_d128_causal_8k"),
+                     "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
                      "kernel": "fa::bwd_dkv3_kernel<bf16,128,64> + fa::bwd_dq_kernel<bf16,128,32> (7 tile products executed for 5 counted)",
                      "flops_per_launch": flops},
     }
@@ -276,7 +289,7 @@ def bench_varlen(steps, warmup):
                           "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                        "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("varlen_bf16_d%d_64seq_h16" % d),
                                        "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                                       "kernel": "fa::prefill_pp_kernel<bf16,128,64>" if d == 128 else "fa::prefill_il_kernel<bf16,ILCfg<bf16,256,32>>",
+                                       "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>" if d == 128 else "fa::prefill_il_kernel<bf16,ILCfg<bf16,256,32>>",
                                        "flops_per_launch": flops}}
         del q, k, v
     return res
@@ -299,8 +312,32 @@ def bench_gqa_window(steps, warmup):
         "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
         "workload": "flash_attn_func fwd bf16 batch=2 seqlen=16384 nheads=32 nheads_kv=8 headdim=128 causal window=(4096,0)",
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None,
-                     "kernel": "fa::prefill_pp_kernel<bf16,128,64>", "flops_per_launch": flops},
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("gqa_window_bf16_d128_2x16k_w4096"),
+                     "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
+                     "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>", "flops_per_launch": flops},
+    }
+
+
+def bench_config1(steps, warmup):
+    """The reference's CPU-runnable case: fp16, batch 2 x 512 x 8 heads x 64, non-causal.  1.07 GFLOP and 3 MB per
+    call: neither roofline is in sight, what a call costs is the launch (host side + one kernel of 64 workgroups on
+    256 CUs).  Reported as microseconds per call on the stream and calls per second of host wall time."""
+    import torch
+    import flash_attn
+    b, s, h, d = 2, 512, 8, 64
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.float16) for _ in range(3))
+    fn = lambda: flash_attn.flash_attn_func(q, k, v)
+    tm = time_steps(fn, max(steps, 200), max(warmup, 20))
+    ms, wall_ms = tm
+    flops = 4.0 * b * s * s * h * d
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {
+        "us_per_call": ms * 1e3, "us_per_call_min": tm.ms_min * 1e3, "host_us_per_call": wall_ms * 1e3, "calls_per_s": 1e3 / wall_ms, "tflops": tflops,
+        "workload": "flash_attn_func fwd fp16 batch=2 seqlen=512 nheads=8 headdim=64 non-causal",
+        "bound": "launch latency (64 workgroups of one 128-row block each; 1.07 GFLOP)",
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
+                     "traffic": None, "kernel": "fa::prefill_il_kernel<fp16,ILCfg<fp16,64,64>>", "flops_per_launch": flops},
     }
 
 
@@ -339,24 +376,34 @@ def bench_decode(steps, warmup):
     q = torch.randn(b, 1, h, d, device="cuda", dtype=torch.bfloat16)
     kn = torch.randn(b, 1, hk, d, device="cuda", dtype=torch.bfloat16)
     vn = torch.randn(b, 1, hk, d, device="cuda", dtype=torch.bfloat16)
-    cache_seqlens = torch.randint(1024, cap, (b,), dtype=torch.int32).cuda()   # [1024, 32767]
+    start = torch.randint(1024, cap, (b,), dtype=torch.int32).cuda()          # [1024, 32767]
+    # A decoding loop: every step appends one token where the last step stopped.  The lengths go back to `start`
+    # ahead of every timed block; a sequence drawn within `steps` tokens of the end of the cache starts that many
+    # tokens earlier, so that no block runs past the cache.
+    start = torch.clamp(start, max=cap - 1 - max(steps, warmup))
+    cache_seqlens = start.clone()
     # cos / sin of position x inverse frequency, base 10000, as flash_attn/layers/rotary.py builds its cache
     inv_freq = 1.0 / (10000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
     ang = torch.outer(torch.arange(cap, dtype=torch.float32), inv_freq)
     cos, sin = torch.cos(ang).to(torch.bfloat16).cuda(), torch.sin(ang).to(torch.bfloat16).cuda()
-    fn = lambda: flash_attn.flash_attn_with_kvcache(q, k_cache, v_cache, kn, vn, cos, sin, cache_seqlens,
-                                                    causal=True, rotary_interleaved=True)
-    tm = time_steps(fn, steps, warmup)
+
+    def fn():
+        flash_attn.flash_attn_with_kvcache(q, k_cache, v_cache, kn, vn, cos, sin, cache_seqlens, causal=True, rotary_interleaved=True)
+        cache_seqlens.add_(1)          # (part of the step: a decoding loop does this too)
+
+    tm = time_steps(fn, steps, warmup, before_block=lambda: cache_seqlens.copy_(start))
     ms, wall_ms = tm
-    keys = int((cache_seqlens.long() + 1).sum().item())
+    # keys read by the average step of a block: step t of a block sees start + t + 1 keys
+    t = torch.arange(steps, device="cuda", dtype=torch.int64)[:, None]
+    keys = float((start.long()[None, :] + t + 1).sum().item()) / steps
     algo_bytes = keys * hk * d * 2 * 2 + 2 * b * h * d * 2 + 2 * b * hk * d * 2 * 2
     gbs = algo_bytes / (ms * 1e-3) / 1e9
     return {
         "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "gb_per_s": gbs, "tokens_per_s": b / (ms * 1e-3),
-        "workload": "flash_attn_with_kvcache bf16 b64 cache(64,32768,8,128) hq64 append1+rotary128 causal",
+        "workload": "flash_attn_with_kvcache bf16 b64 cache(64,32768,8,128) hq64 append1+rotary128 causal, lengths advancing by one per step",
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": gbs / PEAK_HBM_GBS, "traffic": _traffic("decode_bf16_d128_b64_32k"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                     "kernel": "fa::decode_persistent_kernel<bf16,128,append,stream> (step = that kernel, which also appends the new rows, + fa::combine_kernel)", "bytes_per_launch": algo_bytes},
+                     "kernel": "fa::decode_persistent_kernel<bf16,128,append,stream> (step = that kernel, which also appends the new rows, + fa::combine_kernel + the length update)", "bytes_per_launch": algo_bytes},
     }
 
 
@@ -385,7 +432,9 @@ def bench_decode_variants(steps, warmup):
         res[name] = {"ms": ms, "ms_min": tm.ms_min, "gb_per_s": gbs,
                      "workload": "flash_attn_with_kvcache bf16 b%d cache(%d,%d,%d,%d) hq%d seqlen_q %d causal" % (b, b, cap, hk, d, h, sq),
                      "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                                  "traffic": None, "kernel": kern + " + fa::combine_kernel", "bytes_per_launch": algo_bytes}}
+                                  "traffic": _traffic("decode_variant_" + name),
+                                  "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
+                                  "kernel": kern + " + fa::combine_kernel", "bytes_per_launch": algo_bytes}}
         del k_cache, v_cache
     return res
 
@@ -423,7 +472,7 @@ def main():
     ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default=None,
-                    choices=["prefill", "mfma_peak", "hbm_peak", "lds_peak", "decode", "decode_variants", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
+                    choices=["prefill", "config1", "mfma_peak", "hbm_peak", "lds_peak", "decode", "decode_variants", "rotary", "backward", "fwd_bwd", "varlen", "gqa_window", "head_dims"],
                     help="run one leg alone and print its record (for profiler runs: the trace then holds that leg's kernels only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that hardware-counter readings of "
@@ -447,7 +496,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.only:
-        leg = {"prefill": bench_prefill, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "lds_peak": bench_lds_peak, "decode": bench_decode, "decode_variants": bench_decode_variants, "rotary": bench_rotary,
+        leg = {"prefill": bench_prefill, "config1": bench_config1, "mfma_peak": bench_mfma_peak, "hbm_peak": bench_hbm_peak, "lds_peak": bench_lds_peak, "decode": bench_decode, "decode_variants": bench_decode_variants, "rotary": bench_rotary,
                "backward": bench_backward, "fwd_bwd": bench_fwd_bwd, "varlen": bench_varlen, "gqa_window": bench_gqa_window,
                "head_dims": bench_head_dims}[a.only]
         print(json.dumps({"only": a.only, "steps": a.steps, "warmup": a.warmup, a.only: leg(a.steps, a.warmup)}))
@@ -484,6 +533,7 @@ def main():
         out["varlen"] = bench_varlen(a.steps, a.warmup)
         out["gqa_window"] = bench_gqa_window(a.steps, a.warmup)
         out["head_dims"] = bench_head_dims(a.steps, a.warmup)
+        out["config1"] = bench_config1(a.steps, a.warmup)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
