@@ -632,10 +632,15 @@ template <typename T, typename C>
 int launch_prefill_il_cfg(const KParams& kp, hipStream_t stream) {
     return kp.p.p_dropout > 0.f ? launch_prefill_il_one<T, C, true>(kp, stream) : launch_prefill_il_one<T, C, false>(kp, stream);
 }
+// The reference's head-dim buckets 32 and 96 (csrc/flash_attn/src/flash_fwd_launch_template.h:141-149, 179-205) run on
+// the tiles of the next larger bucket with the k-steps and output column blocks past the head dim left out.
 template <typename T, int D, int BN>
 int launch_prefill_il(const KParams& kp, hipStream_t stream) {
     if constexpr (D == 128) {
         if (kp.p.d <= 96 && !(kp.p.p_dropout > 0.f)) return launch_prefill_il_one<T, ILCfg<T, D, BN, 96>, false>(kp, stream);
+    }
+    if constexpr (D == 64) {
+        if (kp.p.d <= 32 && !(kp.p.p_dropout > 0.f)) return launch_prefill_il_one<T, ILCfg<T, D, BN, 32>, false>(kp, stream);
     }
     return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream);
 }
@@ -647,7 +652,10 @@ int launch_prefill_il(const KParams& kp, hipStream_t stream) {
 template <typename T>
 int launch_prefill_il_256(const KParams& kp, hipStream_t stream) {
     if (kp.p.p_dropout > 0.f) return launch_prefill_il_one<T, ILCfgPair<T>, true>(kp, stream);
+    // the reference's buckets 160, 192, 224, 256 (flash_fwd_launch_template.h:236-336)
+    if (kp.p.d <= 160) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 160>, false>(kp, stream);
     if (kp.p.d <= 192) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 192>, false>(kp, stream);
+    if (kp.p.d <= 224) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 224>, false>(kp, stream);
     return launch_prefill_il_one<T, ILCfg<T, 256, 32>, false>(kp, stream);
 }
 

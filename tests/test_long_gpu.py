@@ -76,7 +76,7 @@ def _window(mode, sk, seed):
     return tuple(torch.randint(0, sk, (2,), generator=g).tolist())
 
 
-@pytest.mark.parametrize("d", [40, 64, 96, 128])
+@pytest.mark.parametrize("d", [24, 32, 40, 64, 96, 128])
 @pytest.mark.parametrize("s", [512, 777, 1024])
 @pytest.mark.parametrize("mode", ["full", "causal", "local"])
 def test_pipelined_kernel_square(d, s, mode):
@@ -88,7 +88,7 @@ def test_pipelined_kernel_square(d, s, mode):
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
     # (without a mask, keys beyond 768 at head dim 65..128 are the ping-pong kernel's)
-    _ran("pingpong" if (mode == "full" and d > 64 and s >= 769) else "pipelined", 64 if d <= 64 else 96 if d <= 96 else 128)
+    _ran("pingpong" if (mode == "full" and d > 64 and s >= 769) else "pipelined", 32 if d <= 32 else 64 if d <= 64 else 96 if d <= 96 else 128)
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
@@ -159,7 +159,7 @@ def test_wide_kernel_head_dims_above_128(d, sq, sk, mode):
     window = _window(mode, sk, d * 31 + sq)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
-    _ran("wide", 192 if d <= 192 else 256)
+    _ran("wide", 160 if d <= 160 else 192 if d <= 192 else 224 if d <= 224 else 256)      # the reference's buckets above 128
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
