@@ -168,7 +168,29 @@ def _round_up(x, m):
 
 
 def _stream(device):
-    return torch.cuda.current_stream(device).cuda_stream
+    """raw handle of torch's current stream on `device` (what `torch.cuda.current_stream(device).cuda_stream`
+    returns, without building the Stream object: this runs twice per call)"""
+    index = device.index
+    return torch._C._cuda_getCurrentRawStream(index if index is not None else torch.cuda.current_device())
+
+
+class _on_device:
+    """`with torch.cuda.device(device)` that costs nothing when `device` is already the current one (the guard is
+    only there for callers that pass tensors of another GPU than the current)."""
+    __slots__ = ("guard",)
+
+    def __init__(self, device):
+        index = device.index
+        self.guard = None if index is None or index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
 
 
 _NO_DROPOUT_STATE = {}     # device -> the (never read, never written) rng_state returned when p_dropout = 0
@@ -303,7 +325,7 @@ def fwd(q, k, v, out_, p_dropout, softmax_scale, is_causal, window_size_left, wi
         out = torch.empty_like(q_padded)
     head_size = q_padded.shape[-1]
 
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         softmax_lse = torch.empty((batch_size, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
         p = FaFwdParams()
         p.q, p.k, p.v, p.o = q_padded.data_ptr(), k_padded.data_ptr(), v_padded.data_ptr(), out.data_ptr()
@@ -381,7 +403,7 @@ def varlen_fwd(q, k, v, out_, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
         out = torch.empty_like(q_padded)
     head_size = q_padded.shape[-1]
 
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         softmax_lse = torch.empty((batch_size, num_heads, max_seqlen_q), dtype=torch.float32, device=q.device)
         if zero_tensors:
             out.zero_()
@@ -502,7 +524,7 @@ def bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, p_dropout, softmax_scale
     _check(tuple(softmax_lse.shape) == (batch_size, num_heads, seqlen_q) and softmax_lse.dtype == torch.float32
            and softmax_lse.is_contiguous(), "softmax_lse must be a contiguous fp32 (batch, nheads, seqlen_q) tensor")
     seqlen_q_rounded = _round_up(seqlen_q, 128)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         softmax_d = torch.empty((batch_size, num_heads, seqlen_q_rounded), dtype=torch.float32, device=q.device)
         p = FaBwdParams()
         _fill_bwd(p, dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, softmax_d, softmax_scale, is_causal,
@@ -533,7 +555,7 @@ def varlen_bwd(dout, q, k, v, out, softmax_lse, dq_, dk_, dv_, cu_seqlens_q, cu_
     _check(tuple(softmax_lse.shape) == (batch_size, num_heads, max_seqlen_q) and softmax_lse.dtype == torch.float32
            and softmax_lse.is_contiguous(), "softmax_lse must be a contiguous fp32 (batch, nheads, max_seqlen_q) tensor")
     seqlen_q_rounded = _round_up(max_seqlen_q, 128)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         softmax_d = torch.empty((batch_size, num_heads, seqlen_q_rounded), dtype=torch.float32, device=q.device)
         if zero_tensors:
             dq.zero_(); dk.zero_(); dv.zero_(); softmax_d.zero_()
@@ -593,7 +615,7 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
         out = torch.empty_like(q_padded)
     head_size = q_padded.shape[-1]
 
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if lse_ is not None:
             _check(lse_.dtype == torch.float32 and lse_.is_contiguous() and tuple(lse_.shape) == (batch_size, num_heads, seqlen_q),
                    "lse_ must be a contiguous fp32 tensor of shape (batch_size, num_heads, seqlen_q)")

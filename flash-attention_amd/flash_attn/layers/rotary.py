@@ -89,7 +89,7 @@ def apply_rotary(x, cos, sin, seqlen_offsets: Union[int, torch.Tensor] = 0, cu_s
     p.interleaved, p.conjugate = int(bool(interleaved)), int(bool(conjugate))
     p.dtype = nat._dtype_code(x.dtype)
     p.cs_dtype = {torch.float16: nat.FA_DTYPE_FP16, torch.bfloat16: nat.FA_DTYPE_BF16, torch.float32: nat.FA_DTYPE_FP32}[cos.dtype]
-    with torch.cuda.device(x.device):
+    with nat._on_device(x.device):
         rc = nat.lib.fa_rotary(ctypes.byref(p), ctypes.c_void_p(nat._stream(x.device)))
     if rc != 0:
         raise RuntimeError(nat.lib.fa_last_error().decode() or "libfa_mi355x: error %d" % rc)
