@@ -1,7 +1,7 @@
 """Model of how an MI355X hands the workgroups of a grid to the CUs of one XCD, used to choose the work order
 of the forward and backward kernels (xcd_stream_unit in csrc/fa_common.h).
 
-Observed with per-workgroup time stamps and HW_ID (benchmarks/pp_stage_timing.py): the workgroups that fall
+Observed with per-workgroup time stamps and HW_ID taken by an instrumented build of the ping-pong kernel: the workgroups that fall
 to an XCD go to its 4 shader engines in strict rotation and in order.  Workgroup j waits until engine j mod 4
 has a free CU (8 CUs per engine; one 8-wave workgroup of these kernels fills a CU), and workgroup j + 1 is
 not started before workgroup j, even if its own engine has idle CUs.  `in_order` replays that rule,

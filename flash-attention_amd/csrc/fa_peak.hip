@@ -1,12 +1,13 @@
-// Matrix-pipe microbenchmark: what one MI355X sustains on v_mfma_f32_32x32x16_bf16 alone.
+// Matrix-pipe microbenchmark: what one MI355X sustains on v_mfma_f32_32x32x16_bf16 (or 16x16x32) alone.
 //
 // The published dense bf16 peak (2.5 PFLOP/s) is 256 CUs x 4 SIMDs x one 32x32x16 MFMA per 32 cycles at
 // 2.4 GHz.  With every CU busy the part does not hold 2.4 GHz: the clock follows the switching activity
 // of the operands, so the sustained rate depends on the DATA.  This kernel runs nothing but independent
-// MFMAs (one wave per SIMD, four accumulators in rotation, operands resident in registers) on operands
+// MFMAs (four waves per SIMD, four or eight accumulators in rotation, operands resident in registers) on operands
 // that are either random bf16 values (sign, three exponents around 1, random mantissa) or zeros, and the
-// benchmark reports both next to the attention kernels' rates.  Beside it: the same for HBM reads and for
-// LDS reads.
+// benchmark reports both next to the attention kernels' rates.  The two instruction shapes differ: 16x16x32
+// moves 4 accumulator registers per 16K flops where 32x32x16 moves 16 per 32K, and on random operands the part
+// holds a higher clock with the small shape (2.12 against 1.85 PFLOP/s).  Beside it: the same for HBM reads and for LDS reads.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "fa_mi355x.h"
@@ -17,6 +18,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 peak_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float peak_f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t peak_u32x4;
 
+typedef __attribute__((ext_vector_type(4))) float peak_f32x4;
+
+template <int SHAPE>        // 0: 32x32x16, 1: 16x16x32 (twice as many instructions for the same flops)
 __global__ void __launch_bounds__(256) mfma_peak_kernel(float* sink, int iters, int random_operands) {
     peak_u32x4 a[4], b[4];
     uint32_t st = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
@@ -38,20 +42,36 @@ __global__ void __launch_bounds__(256) mfma_peak_kernel(float* sink, int iters, 
             a[i][e] = va;
             b[i][e] = vb;
         }
-    peak_f32x16 acc[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
-    for (int it = 0; it < iters; it++) {
-#pragma unroll
-        for (int j = 0; j < 16; j++)
-            acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(peak_bf16x8, a[j & 3]),
-                                                                 __builtin_bit_cast(peak_bf16x8, b[(j >> 2) & 3]), acc[j & 3], 0, 0, 0);
-    }
     float res = 0.f;
+    if constexpr (SHAPE == 0) {
+        peak_f32x16 acc[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) res += acc[i][0] + acc[i][9];
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int j = 0; j < 16; j++)
+                acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(peak_bf16x8, a[j & 3]),
+                                                                     __builtin_bit_cast(peak_bf16x8, b[(j >> 2) & 3]), acc[j & 3], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) res += acc[i][0] + acc[i][9];
+    } else {
+        peak_f32x4 acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = (peak_f32x4){0.f, 0.f, 0.f, 0.f};
+        // Written as assembly with the accumulators as in/out operands: left to the register allocator, the
+        // builtin form of this loop rotates the eight accumulators through copies on every iteration, which costs
+        // a third of the issue slots.  Eight instructions lie between two uses of one accumulator.
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int j = 0; j < 32; j++)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[j & 7]) : "v"(a[j & 3]), "v"(b[(j >> 3) & 3]));
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) res += acc[i][0] + acc[i][3];
+    }
     if (res == 1.2345e-30f) *sink = res;        // keeps the accumulators alive; never true in practice
 }
 
@@ -130,10 +150,14 @@ extern "C" int fa_hbm_read_peak(const void* src, int64_t bytes, int32_t nontempo
     return (int)hipGetLastError();
 }
 
-extern "C" int fa_mfma_peak(float* sink, int32_t iters, int32_t random_operands, int64_t* flops, void* hip_stream) {
-    if (!sink || iters <= 0 || !flops) return 1;
+extern "C" int fa_mfma_peak_shape(float* sink, int32_t iters, int32_t random_operands, int32_t shape, int64_t* flops, void* hip_stream) {
+    if (!sink || iters <= 0 || !flops || (shape != 0 && shape != 1)) return 1;
     const int grid = 1024;                      // four workgroups of 4 waves per CU: every SIMD holds 4 waves
-    hipLaunchKernelGGL(fa::mfma_peak_kernel, dim3(grid), dim3(256), 0, (hipStream_t)hip_stream, sink, iters, random_operands);
-    *flops = (int64_t)grid * 4 * iters * 16 * 32768LL;
+    if (shape == 0) hipLaunchKernelGGL(fa::mfma_peak_kernel<0>, dim3(grid), dim3(256), 0, (hipStream_t)hip_stream, sink, iters, random_operands);
+    else hipLaunchKernelGGL(fa::mfma_peak_kernel<1>, dim3(grid), dim3(256), 0, (hipStream_t)hip_stream, sink, iters, random_operands);
+    *flops = (int64_t)grid * 4 * iters * 16 * 32768LL;      // 16 x 32x32x16 or 32 x 16x16x32 per iteration
     return (int)hipGetLastError();
+}
+extern "C" int fa_mfma_peak(float* sink, int32_t iters, int32_t random_operands, int64_t* flops, void* hip_stream) {
+    return fa_mfma_peak_shape(sink, iters, random_operands, 0, flops, hip_stream);
 }

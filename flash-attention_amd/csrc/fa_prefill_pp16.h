@@ -1,8 +1,8 @@
 // The 8-wave ping-pong forward kernel of fa_prefill_pp.h on v_mfma_f32_16x16x32 instead of v_mfma_f32_32x32x16.
 //
 // Why the other instruction: on Gaussian operands this part is power-bound, not issue-bound.  A kernel that only
-// issues matrix instructions on random bf16 data sustains 1.85 PFLOP/s with 32x32x16 and 2.05 with 16x16x32 (the
-// clock settles at 1.81 against 2.03 GHz): per flop the small shape moves half the accumulator registers (4
+// issues matrix instructions on random bf16 data sustains 1.85 PFLOP/s with 32x32x16 and 2.12 with 16x16x32 (the
+// clock settles near 1.8 against 2.05 GHz): per flop the small shape moves half the accumulator registers (4
 // registers in and out per 16K flops against 16 per 32K).  With the operands fed from LDS at this kernel's rate
 // and a softmax wave on the same SIMD the gap is 6-8 % at equal matrix-pipe duty.
 //

@@ -330,6 +330,9 @@ int32_t fa_sizeof_bwd_params(void);
  * `sink` is 4 bytes of device memory (never written in practice).
  */
 int fa_mfma_peak(float *sink, int32_t iters, int32_t random_operands, int64_t *flops, void *hip_stream);
+/* The same with the instruction shape chosen: 0 = v_mfma_f32_32x32x16_bf16 (fa_mfma_peak), 1 = v_mfma_f32_16x16x32_bf16,
+ * twice as many instructions for the same flops.  On random operands the part is power-bound and the two differ. */
+int fa_mfma_peak_shape(float *sink, int32_t iters, int32_t random_operands, int32_t shape, int64_t *flops, void *hip_stream);
 
 /*
  * Memory microbenchmark (measurement aid; no counterpart in the reference): launches a kernel that reads

@@ -50,6 +50,14 @@ def test_mfma_peak_counts_its_operations(random_operands):
     torch.cuda.synchronize()
     assert flops.value == 1024 * 4 * 10 * 16 * 2 * 32 * 32 * 16 and float(sink.item()) == 0.0
     assert lib.fa_mfma_peak(sink.data_ptr(), 0, random_operands, ctypes.byref(flops), None) != 0
+    # the other instruction shape: twice the instructions, the same count of operations
+    lib.fa_mfma_peak_shape.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p]
+    lib.fa_mfma_peak_shape.restype = ctypes.c_int
+    flops2 = ctypes.c_int64(0)
+    assert lib.fa_mfma_peak_shape(sink.data_ptr(), 10, random_operands, 1, ctypes.byref(flops2), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert flops2.value == flops.value and float(sink.item()) == 0.0
+    assert lib.fa_mfma_peak_shape(sink.data_ptr(), 10, random_operands, 2, ctypes.byref(flops2), None) != 0
 
 
 @pytest.mark.parametrize("waves", [1, 4, 8, 16])
