@@ -431,9 +431,11 @@ FA_DEV void async_fill16(const void* base_uniform, uint32_t lane_offset, uint32_
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_base_uniform), "v"(lane_offset), "s"(sbase) : "memory", "m0");
 }
-// wait until at most N of this wave's vector-memory operations are outstanding (N < 16)
+// wait until at most N of this wave's vector-memory operations are outstanding (N < 64: the counter's low four
+// bits sit in bits 3:0 of the operand, its upper two in bits 15:14)
 template <int N> FA_DEV void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8));
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
 // A wave's 32 resident rows (each lane keeps one row in registers as MFMA operand) fetched through a
