@@ -341,7 +341,8 @@ def bench_config1(steps, warmup):
         "workload": "flash_attn_func fwd fp16 batch=2 seqlen=512 nheads=8 headdim=64 non-causal",
         "bound": "launch latency (64 workgroups of one 128-row block each; 1.07 GFLOP)",
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": tflops / PEAK_BF16_TFLOPS,
-                     "traffic": None, "kernel": "fa::prefill_il_kernel<fp16,ILCfg<fp16,64,64>>", "flops_per_launch": flops},
+                     "traffic": _traffic("config1_fp16_d64_2x512x8"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
+                     "kernel": "fa::prefill_il_kernel<fp16,ILCfg<fp16,64,64>>", "flops_per_launch": flops},
     }
 
 

@@ -163,8 +163,8 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     const bool dec = use_decode_kernel(p);
     // The tiled kernel under the persistent schedule of the decode kernel (prefill_persistent_kernel): one row
     // block per (batch, kv head) with every q head of the kv head in it, over a cache whose lengths are on the
-    // device.  Chunks of FA_TILE_MINLEN keys or more (about FA_TILE_SLOTS per launch), their remainders in halves,
-    // quarters or eighths of a chunk (1024 keys or more; see sb below).
+    // device.  Chunks of FA_TILE_MINLEN keys or more (about FA_TILE_SLOTS per launch; down to 512 keys in launches too
+    // small to fill the CUs otherwise), their remainders in halves, quarters or eighths of a chunk (see sb below).
     const int64_t wgs = (int64_t)((p.seqlen_q + prefill_block_m(db) - 1) / prefill_block_m(db)) * p.h * p.b;
     int64_t tile_chunk = 0;
     if (!dec && allow_split && p.num_splits == 0 && p.p_dropout == 0.f && counters_ok(p) && !p.cu_seqlens_q && p.cu_seqlens_k &&
@@ -249,7 +249,8 @@ static SplitPlan plan(const fa_fwd_params& p_in, bool allow_split) {
     // 2048-key one, eighths from 4096 on): shorter pieces are mostly start-up and merge (measured
     // +6 % at batch 256 x 4k and at batch 64 x 8k with 16 grouped heads, nothing lost at config 5).
     // (The tiled kernel pays more per item -- its Q rows, a first tile nothing overlaps, up to 128 partial rows to
-    // write: about what 160 keys take -- and its pieces stay at 1024 keys or more.)
+    // write: about what 160 keys take -- so its chunks below 4096 keys are only halved: pieces of 1024 keys or more for
+    // chunks of FA_TILE_MINLEN, 256 at the least for the 512-key chunks of a launch that would not fill the CUs.)
     // Halves, quarters or eighths of a multiple of 512: whole tiles.
     const int sb = tile_chunk ? (len < 4096 ? 2 : len < 8192 ? 4 : FA_DEC_SB) : len < 2048 ? 2 : len < 4096 ? 4 : FA_DEC_SB;
     if ((dec || tile_chunk) && automatic && splits > 1 && counters_ok(p) && len >= (dec ? 1024 : 512) && splits + sb <= FA_MAX_SPLITS) {
