@@ -19,6 +19,7 @@
 //   * a row's keys are spread over the 4 lanes m, m + 16, m + 32, m + 48: row sums stay per lane until the epilogue,
 //     the (rare) exact maximum is reduced over those lanes.
 #pragma once
+#include <type_traits>
 #include "fa_prefill_pp.h"
 
 namespace fa {
@@ -178,8 +179,10 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
 #pragma unroll
     for (int c = 0; c < KC; c++) kofs[c] = m16 * C::ROWB + swz_k<D>(c * 4 + g4, m16) * 16;
     f32x4 s_acc[2][KB];
-    auto qk = [&](int i) {
-        const int slot = (i & (C::NS - 1)) * C::TILE;
+    auto qk = [&](int i, auto slot_c) __attribute__((always_inline)) {
+        // the ring slot of visit i is a compile-time constant (the key loop is unrolled by the ring depth), so slot and
+        // fragment offsets go into the offset field of the LDS reads instead of a vector add per fragment pointer
+        constexpr int slot = decltype(slot_c)::value * C::TILE;
         const char* kb[KC];
 #pragma unroll
         for (int c = 0; c < KC; c++) kb[c] = smem + (slot + kofs[c]);
@@ -211,10 +214,11 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     int vofs[DB];
 #pragma unroll
     for (int db = 0; db < DB; db++)
-        vofs[db] = (4 * g4 + tj) * C::ROWB + swz_vd<D>(db * 2 + (tq >> 1), 4 * g4 + tj) * 16 + (tq & 1) * 8;
+        vofs[db] = C::NS * C::TILE + (4 * g4 + tj) * C::ROWB + swz_vd<D>(db * 2 + (tq >> 1), 4 * g4 + tj) * 16 + (tq & 1) * 8;
     v8 pf[2][T32];
-    auto pv = [&](int i) {
-        const int slot = (C::NS + (i & (C::NS - 1))) * C::TILE;
+    auto pv = [&](int i, auto slot_c) __attribute__((always_inline)) {
+        // (vofs already points into the V ring, so that slot and fragment offsets fit the 16-bit offset field)
+        constexpr int slot = decltype(slot_c)::value * C::TILE;
         const char* vb[DB];
 #pragma unroll
         for (int db = 0; db < DB; db++) vb[db] = smem + (slot + vofs[db]);
@@ -245,7 +249,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         }
     };
 
-    auto softmax = [&](int i) {
+    auto softmax = [&](int i) __attribute__((always_inline)) {
         const int tt = tile_of(i);
         if (tt < tf_lo || tt > tf_hi) {
             const int n0 = tt * BN;
@@ -325,10 +329,12 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         // ---- prologue: K(0), V(0), K(1), V(1), K(2) were requested above; S = K(0) Q
         wait_vmcnt<0>();
         __syncthreads();
-        if (active(0)) qk(0);
+        if (active(0)) qk(0, std::integral_constant<int, 0>());
         if (group == 1) __syncthreads();   // group 1 runs one phase behind group 0
 
-        for (int i = 0; i < nt; i++) {
+        // visit i of the key loop with its ring slots as compile-time constants: i % NS == SL (measured +0.5-1 %)
+        auto visit = [&](int i, auto sl) __attribute__((always_inline)) {
+            constexpr int SL = decltype(sl)::value;
             // ---- Y(i): VALU phase (and requests for the tiles needed 3 iterations ahead)
             if (i + C::PF < nt) fill_k(i + C::PF);
             if (i + C::PF - 1 < nt) fill_v(i + C::PF - 1);
@@ -337,14 +343,25 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
             __syncthreads();
             // ---- X(i): MFMA phase
             __builtin_amdgcn_s_setprio(1);
-            if (act) pv(i);
-            if (i + 1 < nt && active(i + 1)) qk(i + 1);
+            if (act) pv(i, std::integral_constant<int, SL>());
+            if (i + 1 < nt && active(i + 1)) qk(i + 1, std::integral_constant<int, (SL + 1) % C::NS>());
             __builtin_amdgcn_s_setprio(0);
             // this wave's fills of K(i+2), V(i+1) must have landed before the barrier publishes them;
             // the 2 * LOADS requests of Y(i) may stay in flight
             if (i + C::PF < nt) wait_vmcnt<2 * C::LOADS>(); else wait_vmcnt<0>();
             __syncthreads();
+        };
+        static_assert(C::NS == 4, "the loop is unrolled by the ring depth");
+        int i = 0;
+        for (; i + 4 <= nt; i += 4) {
+            visit(i, std::integral_constant<int, 0>());
+            visit(i + 1, std::integral_constant<int, 1>());
+            visit(i + 2, std::integral_constant<int, 2>());
+            visit(i + 3, std::integral_constant<int, 3>());
         }
+        if (i < nt) { visit(i, std::integral_constant<int, 0>()); i++; }
+        if (i < nt) { visit(i, std::integral_constant<int, 1>()); i++; }
+        if (i < nt) { visit(i, std::integral_constant<int, 2>()); i++; }
         if (group == 0) __syncthreads();
     }
 
