@@ -121,7 +121,7 @@ def bench_head_dims(steps, warmup):
     import flash_attn
     b, s, h = 4, 8192, 32
     res = {}
-    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96>"), (192, "fa::prefill_il_kernel<bf16,ILCfg<bf16,256,32,192>>")):
+    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96>"), (192, "fa::prefill_pp16_kernel<bf16,256,32,192,1>")):
         torch.manual_seed(0)
         q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
         with torch.no_grad():
@@ -293,7 +293,7 @@ def bench_varlen(steps, warmup):
                           "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                        "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("varlen_bf16_d%d_64seq_h16" % d),
                                        "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                                       "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>" if d == 128 else "fa::prefill_il_kernel<bf16,ILCfg<bf16,256,32>>",
+                                       "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>" if d == 128 else "fa::prefill_pp16_kernel<bf16,256,32,256,1>",
                                        "flops_per_launch": flops}}
         del q, k, v
     return res

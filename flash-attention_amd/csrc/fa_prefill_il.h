@@ -644,19 +644,12 @@ int launch_prefill_il(const KParams& kp, hipStream_t stream) {
     }
     return launch_prefill_il_cfg<T, ILCfg<T, D, BN>>(kp, stream);
 }
-// Head dims 129..256.  Without dropout: the whole head dimension in one wave, 32-key tiles, one wave per SIMD
-// (ILCfg<T, 256, 32>; head dims up to 192 run 12 of 16 k-steps and 6 of 8 output column blocks).  Measured
-// against the pair form on the same shapes: +9 % causal 8k, +15 % full, +10 % at head dim 192, +7 % on packed
-// batches.  64-key tiles do not work there: the step then holds 64 matrix instructions and the compiler no
-// longer unrolls it (the S tiles end up in scratch memory, 14 x slower).  With dropout: the pair form.
+// Head dims 129..256 with dropout: the pair form (without dropout those head dims run on the 8-wave kernel of
+// fa_prefill_pp16.h with 16 query rows per wave, measured 7-18 % ahead of the whole-head-dim form ILCfg<T, 256, 32, DV>
+// of this kernel, one wave per SIMD with all 512 registers, which is no longer instantiated).
 template <typename T>
 int launch_prefill_il_256(const KParams& kp, hipStream_t stream) {
-    if (kp.p.p_dropout > 0.f) return launch_prefill_il_one<T, ILCfgPair<T>, true>(kp, stream);
-    // the reference's buckets 160, 192, 224, 256 (flash_fwd_launch_template.h:236-336)
-    if (kp.p.d <= 160) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 160>, false>(kp, stream);
-    if (kp.p.d <= 192) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 192>, false>(kp, stream);
-    if (kp.p.d <= 224) return launch_prefill_il_one<T, ILCfg<T, 256, 32, 224>, false>(kp, stream);
-    return launch_prefill_il_one<T, ILCfg<T, 256, 32>, false>(kp, stream);
+    return launch_prefill_il_one<T, ILCfgPair<T>, true>(kp, stream);
 }
 
 }  // namespace fa

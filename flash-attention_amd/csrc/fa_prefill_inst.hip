@@ -45,9 +45,12 @@ int FA_INST_NAME(FA_D)(const KParams& kp, hipStream_t stream) {
         return launch_prefill_il<InstT, FA_D, 64>(kp, stream);
     }
 #else
-    // head dim 129..256: one wave per SIMD with the whole head dimension, or pairs of waves that split it
-    // (with dropout); fa_prefill_il.h
-    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= prefill_long_rows(FA_D) && kp.pack_g <= 1) return launch_prefill_il_256<InstT>(kp, stream);
+    // head dim 129..256: the 8-wave ping-pong kernel with 16 query rows per wave (fa_prefill_pp16.h), or, with dropout,
+    // pairs of waves that split the head dim (fa_prefill_il.h)
+    if (kp.num_splits <= 1 && !kp.rotary_q && kp.p.seqlen_q >= prefill_long_rows(FA_D) && kp.pack_g <= 1) {
+        if (kp.p.p_dropout > 0.f) return launch_prefill_il_256<InstT>(kp, stream);
+        return launch_prefill_pp_wide<InstT>(kp, stream);
+    }
 #endif
     return launch_prefill<InstT, FA_D, Tile::RB, Tile::BN, Tile::MINW>(kp, stream);
 }

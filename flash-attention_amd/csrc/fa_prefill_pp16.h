@@ -33,10 +33,16 @@ FA_DEV void mask_acc4(f32x4& s, int pos0, int lo, int hi) {
     for (int r = 0; r < 4; r++) s[r] = (uint32_t)(z + r) > span ? -INFINITY : s[r];
 }
 
-template <typename T, int D, int BN, int DV = D>
+// RB: 16-row blocks per wave (2: 256 rows per workgroup; 1: 128, the form for head dims 129-256, where 32 rows of output
+// and Q per wave leave no room for two waves per SIMD: there each fragment read from LDS feeds one matrix instruction
+// instead of two, and the kernel is bound by its fragment reads).
+template <typename T, int D, int BN, int DV = D, int RB = 2>
 __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) {
     typedef PPCfg<T, D, BN> C;
     static_assert(DV % 32 == 0 && DV <= D, "computed head dims");
+    static_assert(RB == 1 || RB == 2, "row blocks per wave");
+    constexpr int WR = 16 * RB;          // query rows of a wave
+    constexpr int BM = C::kWaves * WR;   // query rows of a workgroup
     constexpr int KC = DV / 32;          // k-steps of S (32 head dims each)
     constexpr int DB = DV / 16;          // 16-column blocks of O
     constexpr int KB = BN / 16;          // 16-key blocks of a tile
@@ -48,7 +54,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int m16 = lane & 15, g4 = lane >> 4;
-    const int group = wave >> 2;
+    const int group = __builtin_amdgcn_readfirstlane(wave >> 2);
 
     // work item of this block (32-bit arithmetic: the launcher bounds the grid by 2^31)
     const uint32_t G = (uint32_t)(p.h / p.h_k);
@@ -57,14 +63,14 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     const int head = hk * (int)G + g;
 
     const SeqInfo si = seq_info(p, b);
-    const int m0 = mb * C::BM;
+    const int m0 = mb * BM;
     if (m0 >= si.sq) return;
 
     const int shift = si.sk - si.sq;
     const int wl = p.window_left, wr = p.window_right;
     const bool has_left = kp.has_left, has_right = kp.has_right;
     int n_hi = si.sk;
-    if (has_right) n_hi = min(n_hi, min(m0 + C::BM, si.sq) + shift + wr);
+    if (has_right) n_hi = min(n_hi, min(m0 + BM, si.sq) + shift + wr);
     int n_lo = 0;
     if (has_left) n_lo = max(0, m0 + shift - wl);
     const int t_lo = n_lo / BN;
@@ -75,7 +81,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     const T* __restrict__ kg = reinterpret_cast<const T*>(p.k) + si.k_off + (int64_t)hk * p.k_head_stride;
     const T* __restrict__ vg = reinterpret_cast<const T*>(p.v) + si.v_off + (int64_t)hk * p.v_head_stride;
 
-    const int r0 = m0 + wave * 32;                // first query row of this wave
+    const int r0 = m0 + wave * WR;                // first query row of this wave
 
     // visit i of the key loop handles key tile tile_of(i) and uses ring slot i % NS
     // (from the last tile down: the masked tiles of a causal row block come first)
@@ -135,9 +141,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     }
 
     // ---- resident Q fragments (B operand of the first product): row 16 rb + m16, head dims 32 c + 8 g4 .. + 7
-    v8 qf[2][KC];
+    v8 qf[RB][KC];
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++) {
+    for (int rb = 0; rb < RB; rb++) {
         const int row = r0 + 16 * rb + m16;
         const bool valid = row < si.sq;
         const T* qrow = qg + (int64_t)row * p.q_row_stride;
@@ -150,26 +156,28 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         }
     }
 
-    f32x4 o_acc[2][DB];
+    f32x4 o_acc[RB][DB];
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++)
+    for (int rb = 0; rb < RB; rb++)
 #pragma unroll
         for (int db = 0; db < DB; db++) o_acc[rb][db] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};     // l_run: this lane's share of the row sum
+    float m_run[RB], l_run[RB];     // l_run: this lane's share of the row sum
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) { m_run[rb] = -INFINITY; l_run[rb] = 0.f; }
     const float sl2 = kp.scale_log2;
 
     // Per-wave tile classes, as ranges of the absolute key-tile index t: the wave has visible keys
-    // in tiles [ta_lo, ta_hi]; tiles in [tf_lo, tf_hi] are fully visible to all 32 rows (no masking).
+    // in tiles [ta_lo, ta_hi]; tiles in [tf_lo, tf_hi] are fully visible to all its rows (no masking).
     int ta_lo = t_lo, ta_hi = t_hi - 1, tf_lo = 0, tf_hi = si.sk / BN - 1;
     if (has_right) {
         const int c = r0 + shift + wr;            // last visible key of the wave's first row
-        ta_hi = min(ta_hi, (c + 31 >= 0) ? (c + 31) / BN : -1);
+        ta_hi = min(ta_hi, (c + WR - 1 >= 0) ? (c + WR - 1) / BN : -1);
         tf_hi = min(tf_hi, (c + 1 >= BN) ? (c + 1) / BN - 1 : -1);
     }
     if (has_left) {
         const int c = r0 + shift - wl;            // first visible key of the wave's first row
         ta_lo = max(ta_lo, (c > 0) ? c / BN : 0);
-        tf_lo = (c + 31 > 0) ? (c + 31 + BN - 1) / BN : 0;
+        tf_lo = (c + WR - 1 > 0) ? (c + WR - 1 + BN - 1) / BN : 0;
     }
     if (r0 >= si.sq) ta_hi = ta_lo - 1;
     auto active = [&](int i) -> bool { const int t = tile_of(i); return t >= ta_lo && t <= ta_hi; };
@@ -178,7 +186,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     int kofs[KC];
 #pragma unroll
     for (int c = 0; c < KC; c++) kofs[c] = m16 * C::ROWB + swz_k<D>(c * 4 + g4, m16) * 16;
-    f32x4 s_acc[2][KB];
+    f32x4 s_acc[RB][KB];
     auto qk = [&](int i, auto slot_c) __attribute__((always_inline)) {
         // the ring slot of visit i is a compile-time constant (the key loop is unrolled by the ring depth), so slot and
         // fragment offsets go into the offset field of the LDS reads instead of a vector add per fragment pointer
@@ -197,14 +205,14 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         for (int f = 0; f < NF; f++) {
             const int c = f / KB, kbk = f % KB;
             const v8 a = __builtin_bit_cast(v8, fr[f % LA]);
-            s_acc[0][kbk] = Elem<T>::mfma16(a, qf[0][c], c == 0 ? zero : s_acc[0][kbk]);
-            s_acc[1][kbk] = Elem<T>::mfma16(a, qf[1][c], c == 0 ? zero : s_acc[1][kbk]);
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) s_acc[rb][kbk] = Elem<T>::mfma16(a, qf[rb][c], c == 0 ? zero : s_acc[rb][kbk]);
             if (f + LA < NF) fr[f % LA] = *reinterpret_cast<const u32x4*>(frag_ptr(f + LA));
         }
         __builtin_amdgcn_sched_group_barrier(0x100, LA, 0);      // look-ahead reads
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMAs
+            __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);  // RB MFMAs
             if (f + LA < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 DS read
         }
     };
@@ -215,7 +223,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
 #pragma unroll
     for (int db = 0; db < DB; db++)
         vofs[db] = C::NS * C::TILE + (4 * g4 + tj) * C::ROWB + swz_vd<D>(db * 2 + (tq >> 1), 4 * g4 + tj) * 16 + (tq & 1) * 8;
-    v8 pf[2][T32];
+    v8 pf[RB][T32];
     auto pv = [&](int i, auto slot_c) __attribute__((always_inline)) {
         // (vofs already points into the V ring, so that slot and fragment offsets fit the 16-bit offset field)
         constexpr int slot = decltype(slot_c)::value * C::TILE;
@@ -237,14 +245,14 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         for (int f = 0; f < NF; f++) {
             const int t32 = f / DB, db = f % DB;
             const v8 a = __builtin_bit_cast(v8, fr[f % LA]);
-            o_acc[0][db] = Elem<T>::mfma16(a, pf[0][t32], o_acc[0][db]);
-            o_acc[1][db] = Elem<T>::mfma16(a, pf[1][t32], o_acc[1][db]);
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) o_acc[rb][db] = Elem<T>::mfma16(a, pf[rb][t32], o_acc[rb][db]);
             if (f + LA < NF) fr[f % LA] = fetch(f + LA);
         }
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * LA, 0);  // look-ahead reads
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMAs
+            __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);  // RB MFMAs
             if (f + LA < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 DS reads
         }
     };
@@ -254,7 +262,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         if (tt < tf_lo || tt > tf_hi) {
             const int n0 = tt * BN;
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
+            for (int rb = 0; rb < RB; rb++) {
                 const int row = r0 + 16 * rb + m16;
                 int lim_hi = si.sk - 1;
                 if (has_right) lim_hi = min(lim_hi, row + shift + wr);
@@ -288,12 +296,17 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
             }
             return suma + sumb;
         };
-        float tsum0 = exp_tile(0, m_run[0] * sl2), tsum1 = exp_tile(1, m_run[1] * sl2);
-        float corr0 = 1.f, corr1 = 1.f;
-        if (__builtin_amdgcn_ballot_w64(!(tsum0 <= 16384.f) || !(tsum1 <= 16384.f)) != 0) {
-            float corr[2], tsum[2];
+        float tsum[RB], corr[RB];
+        bool redo = false;
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
+        for (int rb = 0; rb < RB; rb++) {
+            tsum[rb] = exp_tile(rb, m_run[rb] * sl2);
+            corr[rb] = 1.f;
+            redo = redo || !(tsum[rb] <= 16384.f);
+        }
+        if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
                 float mx = -INFINITY;
 #pragma unroll
                 for (int kbk = 0; kbk < KB; kbk++)
@@ -309,19 +322,20 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
                 m_run[rb] = m_new;
                 tsum[rb] = exp_tile(rb, (m_new == -INFINITY) ? 0.f : m_new * sl2);
             }
-            tsum0 = tsum[0]; tsum1 = tsum[1];
-            corr0 = corr[0]; corr1 = corr[1];
         }
-        l_run[0] += tsum0;
-        l_run[1] += tsum1;
+        bool moved = false;
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            l_run[rb] += tsum[rb];
+            moved = moved || corr[rb] != 1.f;
+        }
         // (tested on the factors themselves, not on a flag set in the branch above: with a flag the compiler
         // merges this block into that branch and copies all of o_acc around it on every tile)
-        if (__builtin_amdgcn_ballot_w64(corr0 != 1.f || corr1 != 1.f) != 0) {
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
 #pragma unroll
-            for (int db = 0; db < DB; db++) {
-                o_acc[0][db] *= corr0;
-                o_acc[1][db] *= corr1;
-            }
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++) o_acc[rb][db] *= corr[rb];
         }
     };
 
@@ -366,9 +380,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     }
 
     // ---- epilogue: the row sums of the 4 lanes that share a row, normalisation, log-sum-exp
-    float inv[2];
+    float inv[RB];
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++) {
+    for (int rb = 0; rb < RB; rb++) {
         float l_tot = l_run[rb];
         l_tot += __shfl_xor(l_tot, 16);
         l_tot += __shfl_xor(l_tot, 32);
@@ -378,14 +392,14 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         const int row = r0 + 16 * rb + m16;
         if (g4 == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
     }
-    // The output tile of the wave (32 rows x D) goes through LDS so that every store instruction writes whole
+    // The output tile of the wave (its rows x D) goes through LDS so that every store instruction writes whole
     // rows (16 B per lane).  All tile reads of the ring are behind the last barrier and each wave uses its own
     // region, so no barrier is needed.
     {
         constexpr int PITCH = C::ROWB + 16;
-        char* stage = smem + wave * (32 * PITCH);
+        char* stage = smem + wave * (WR * PITCH);
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int rb = 0; rb < RB; rb++)
 #pragma unroll
             for (int db = 0; db < DB; db++) {
                 const int d0 = db * 16 + 4 * g4;
@@ -397,7 +411,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         const int srow = lane / C::CPR, sch = lane % C::CPR;
         T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + sch * 8;
 #pragma unroll
-        for (int j = 0; j < 32 / RPP; j++) {
+        for (int j = 0; j < WR / RPP; j++) {
             const int rr = j * RPP + srow;
             const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
             if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
@@ -405,21 +419,22 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     }
 }
 
-template <typename T, int D, int BN, int DV = D>
+template <typename T, int D, int BN, int DV = D, int RB = 2>
 int launch_prefill_pp16_one(KParams kp, hipStream_t stream) {
     typedef PPCfg<T, D, BN> C;
-    kp.num_m_blocks = (kp.p.seqlen_q + C::BM - 1) / C::BM;
+    constexpr int BM = C::kWaves * 16 * RB;
+    kp.num_m_blocks = (kp.p.seqlen_q + BM - 1) / BM;
     const int64_t total = (int64_t)kp.num_m_blocks * kp.p.h * kp.p.b;
     if (total <= 0) return 0;
     const int64_t nblocks = xcd_grid(kp.p, kp.num_m_blocks);
     if (nblocks == 0) return -2;
     dim3 grid((unsigned)nblocks), block(C::kThreads);
-    if (int e = prepare_work_list(kp, C::BM, nblocks, stream)) return e;
-    auto kern = prefill_pp16_kernel<T, D, BN, DV>;
+    if (int e = prepare_work_list(kp, BM, nblocks, stream)) return e;
+    auto kern = prefill_pp16_kernel<T, D, BN, DV, RB>;
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-    return note_kernel((int)hipGetLastError(), FA_KERNEL_PINGPONG, false, false, DV);
+    return note_kernel((int)hipGetLastError(), D > 128 ? FA_KERNEL_PINGPONG_WIDE : FA_KERNEL_PINGPONG, false, false, DV);
 }
 
 // Without dropout the 16x16x32 form; with dropout the 32x32x16 kernel of fa_prefill_pp.h, whose mask arithmetic
@@ -431,6 +446,18 @@ int launch_prefill_pp(const KParams& kp, hipStream_t stream) {
         if (kp.p.d <= 96) return launch_prefill_pp16_one<T, D, BN, 96>(kp, stream);
     }
     return launch_prefill_pp16_one<T, D, BN>(kp, stream);
+}
+
+// Head dims 129..256 without dropout: 16 query rows per wave (one row block: 64 accumulator registers of output and 32
+// of Q at head dim 256), 128 rows per workgroup, 32-key tiles in the same four-slot rings; the reference's buckets
+// 160, 192, 224, 256 (csrc/flash_attn/src/flash_fwd_launch_template.h:236-336) leave out the k-steps and column
+// blocks past the bucket.
+template <typename T>
+int launch_prefill_pp_wide(const KParams& kp, hipStream_t stream) {
+    if (kp.p.d <= 160) return launch_prefill_pp16_one<T, 256, 32, 160, 1>(kp, stream);
+    if (kp.p.d <= 192) return launch_prefill_pp16_one<T, 256, 32, 192, 1>(kp, stream);
+    if (kp.p.d <= 224) return launch_prefill_pp16_one<T, 256, 32, 224, 1>(kp, stream);
+    return launch_prefill_pp16_one<T, 256, 32, 256, 1>(kp, stream);
 }
 
 }  // namespace fa

@@ -6,7 +6,7 @@ library has it (csrc/fa_prefill_inst.hip), for an unsplit launch of 96+ query ro
     more than 256 (masked) / 128 (unmasked) row blocks of 256 rows in the launch, and no window whose two bounds
     span 768 keys or fewer;
   * software-pipelined kernel (fa_prefill_il.h): everything else up to head dim 128;
-  * head dim 129..256: one wave per SIMD with the whole head dimension ("wide"), pairs of waves with dropout.
+  * head dim 129..256: the 8-wave kernel with 16 query rows per wave ("pingpong_wide"), pairs of waves with dropout.
 
 Launches are made large enough for those thresholds with many query heads on few kv heads; the CPU oracle then checks
 a sample of (batch, head) pairs, which are independent problems.  Cases follow the reference's own test dimensions
@@ -152,14 +152,14 @@ def test_pingpong_kernel(case):
 @pytest.mark.parametrize("sq,sk,mode", [(777, 777, "causal"), (512, 512, "full"), (600, 1500, "causal"),
                                          (1500, 600, "local"), (1024, 1024, "local")])
 def test_wide_kernel_head_dims_above_128(d, sq, sk, mode):
-    _say("wide kernel", d, sq, sk, mode)
+    _say("head dims above 128", d, sq, sk, mode)
     dtype = torch.float16 if d == 160 and sq <= 777 else torch.bfloat16
     b, h, hk = 4, 16, 2
     q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
     window = _window(mode, sk, d * 31 + sq)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
-    _ran("wide", 160 if d <= 160 else 192 if d <= 192 else 224 if d <= 224 else 256)      # the reference's buckets above 128
+    _ran("pingpong_wide", 160 if d <= 160 else 192 if d <= 192 else 224 if d <= 224 else 256)      # the reference's buckets above 128
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
 
 
@@ -171,7 +171,7 @@ def test_long_kernels_take_strided_packed_input(s, d):
     b, h = 2, 16
     qkv = _gen((b, s, 3, h, d), dtype, 5)
     out, lse, _ = _fa().flash_attn_qkvpacked_func(qkv.to(DEV), causal=True, return_attn_probs=True)
-    _ran({64: "pipelined", 128: "pingpong", 256: "wide"}[d])        # (d 128: 9 row blocks x 16 heads x 2 = 288)
+    _ran({64: "pipelined", 128: "pingpong", 256: "pingpong_wide"}[d])        # (d 128: 9 row blocks x 16 heads x 2 = 288)
     _check(out, lse, qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], causal=True)
 
 
@@ -185,7 +185,7 @@ def test_varlen_long_with_empty_and_tiny_sequences(d):
     q = _gen((total, h, d), dtype, 1); k = _gen((total, h, d), dtype, 2); v = _gen((total, h, d), dtype, 3)
     out, lse, _ = _fa().flash_attn_varlen_func(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), cu.to(DEV), mx, mx,
                                                causal=True, return_attn_probs=True)
-    _ran({64: "pipelined", 128: "pingpong", 256: "wide"}[d])        # (d 128: 9 row blocks x 16 heads x 12 sequences)
+    _ran({64: "pipelined", 128: "pingpong", 256: "pingpong_wide"}[d])        # (d 128: 9 row blocks x 16 heads x 12 sequences)
     assert out.shape == q.shape and lse.shape == (len(lens), h, mx)
     assert not torch.isnan(out).any()
     for i, L in enumerate(lens):

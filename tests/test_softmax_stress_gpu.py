@@ -53,7 +53,7 @@ _SHAPES = {
     "wide": (256, 4, 8, 2, 512, 1024),
 }
 _KERNEL_OF = {"tiled": "tiled", "pipelined": "pipelined", "pipelined64": "pipelined", "pingpong": "pingpong",
-              "pingpong96": "pingpong", "wide": "wide"}
+              "pingpong96": "pingpong", "wide": "pingpong_wide"}
 _PATTERNS = ["rising", "falling", "spike_first", "spike_middle", "spike_last", "scale1", "x8"]
 
 
