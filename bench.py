@@ -109,7 +109,7 @@ def bench_prefill(steps, warmup):
         "ms": ms, "ms_min": tm.ms_min, "wall_ms": wall_ms, "tflops": tflops, "tokens_per_s": b * s / (ms * 1e-3),
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("prefill_bf16_d128_causal_8k"), "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                     "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>", "flops_per_launch": flops},
+                     "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128,2>", "flops_per_launch": flops},
     }
 
 
@@ -121,7 +121,7 @@ def bench_head_dims(steps, warmup):
     import flash_attn
     b, s, h = 4, 8192, 32
     res = {}
-    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96>"), (192, "fa::prefill_pp16_kernel<bf16,256,32,192,1>")):
+    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96,2>"), (192, "fa::prefill_pp16_kernel<bf16,256,32,192,1>")):
         torch.manual_seed(0)
         q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
         with torch.no_grad():
@@ -293,7 +293,7 @@ def bench_varlen(steps, warmup):
                           "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                                        "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("varlen_bf16_d%d_64seq_h16" % d),
                                        "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                                       "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>" if d == 128 else "fa::prefill_pp16_kernel<bf16,256,32,256,1>",
+                                       "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128,2>" if d == 128 else "fa::prefill_pp16_kernel<bf16,256,32,256,1>",
                                        "flops_per_launch": flops}}
         del q, k, v
     return res
@@ -318,7 +318,7 @@ def bench_gqa_window(steps, warmup):
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": _traffic("gqa_window_bf16_d128_2x16k_w4096"),
                      "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)",
-                     "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128>", "flops_per_launch": flops},
+                     "kernel": "fa::prefill_pp16_kernel<bf16,128,64,128,2>", "flops_per_launch": flops},
     }
 
 
