@@ -63,8 +63,13 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     const int head = hk * (int)G + g;
 
     const SeqInfo si = seq_info(p, b);
-    const int m0 = mb * BM;
-    if (m0 >= si.sq) return;
+    // Row blocks are aligned to the END of the sequence: the partial block of a length that is no multiple of BM is
+    // the first one, which under a causal mask sees the fewest keys (aligned to the start, the half-empty block is the
+    // one that visits the most tiles).  Measured: 64 packed sequences of 2176 tokens -2.4 %, lengths drawn from
+    // 128-4096 +-0.3 %.  m0 < 0 in that first block.
+    const int nmb_seq = (si.sq + BM - 1) / BM;
+    if (mb >= nmb_seq) return;
+    const int m0 = si.sq - (nmb_seq - mb) * BM;
 
     const int shift = si.sk - si.sq;
     const int wl = p.window_left, wr = p.window_right;
@@ -72,7 +77,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     int n_hi = si.sk;
     if (has_right) n_hi = min(n_hi, min(m0 + BM, si.sq) + shift + wr);
     int n_lo = 0;
-    if (has_left) n_lo = max(0, m0 + shift - wl);
+    if (has_left) n_lo = max(0, max(m0, 0) + shift - wl);
     const int t_lo = n_lo / BN;
     const int t_hi = n_hi > 0 ? (n_hi + BN - 1) / BN : 0;
     const int nt = max(0, t_hi - t_lo);           // tiles visited, the same for all 8 waves
@@ -145,7 +150,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         const int row = r0 + 16 * rb + m16;
-        const bool valid = row < si.sq;
+        const bool valid = row >= 0 && row < si.sq;
         const T* qrow = qg + (int64_t)row * p.q_row_stride;
 #pragma unroll
         for (int c = 0; c < KC; c++) {
@@ -179,7 +184,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         ta_lo = max(ta_lo, (c > 0) ? c / BN : 0);
         tf_lo = (c + WR - 1 > 0) ? (c + WR - 1 + BN - 1) / BN : 0;
     }
-    if (r0 >= si.sq) ta_hi = ta_lo - 1;
+    if (r0 >= si.sq || r0 + WR <= 0) ta_hi = ta_lo - 1;
     auto active = [&](int i) -> bool { const int t = tile_of(i); return t >= ta_lo && t <= ta_hi; };
 
     // ---- S^T = K Q^T.  Fragment reads run LA fragments (2 LA matrix instructions) ahead of their use.
@@ -390,7 +395,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         inv[rb] = dead ? 1.f : 1.f / l_tot;
         const float lse = dead ? INFINITY : m_run[rb] * p.softmax_scale + __logf(l_tot);
         const int row = r0 + 16 * rb + m16;
-        if (g4 == 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
+        if (g4 == 0 && row >= 0 && row < si.sq) p.softmax_lse[((int64_t)b * p.h + head) * p.seqlen_q + row] = lse;
     }
     // The output tile of the wave (its rows x D) goes through LDS so that every store instruction writes whole
     // rows (16 B per lane).  All tile reads of the ring are behind the last barrier and each wave uses its own
@@ -414,7 +419,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         for (int j = 0; j < WR / RPP; j++) {
             const int rr = j * RPP + srow;
             const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
-            if (r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
+            if (r0 + rr >= 0 && r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
         }
     }
 }
