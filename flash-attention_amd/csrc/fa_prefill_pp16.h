@@ -1,18 +1,17 @@
 // The 8-wave ping-pong forward kernel of fa_prefill_pp.h on v_mfma_f32_16x16x32 instead of v_mfma_f32_32x32x16.
 //
-// Why the other instruction: on Gaussian operands this part is power-bound, not issue-bound.  A kernel that only
-// issues matrix instructions on random bf16 data sustains 1.85 PFLOP/s with 32x32x16 and 2.12 with 16x16x32 (the
-// clock settles near 1.8 against 2.05 GHz): per flop the small shape moves half the accumulator registers (4
-// registers in and out per 16K flops against 16 per 32K).  With the operands fed from LDS at this kernel's rate
-// and a softmax wave on the same SIMD the gap is 6-8 % at equal matrix-pipe duty.
+// Why the other instruction: on Gaussian operands the part does not hold its clock.  A kernel that only issues matrix
+// instructions on random bf16 data sustains 1.85 PFLOP/s with 32x32x16 and 2.12 with 16x16x32 (the clock settles near
+// 1.8 against 2.05 GHz): per flop the small shape moves half the accumulator registers (4 registers in and out per 16K
+// flops against 16 per 32K).  This kernel runs at 2.05 GHz where its 32x32x16 form ran at 1.69.
 //
 // What stays: the work order, the tile ring (global_load_lds straight into LDS, 4 slots per tensor, 3 tiles ahead),
 // the two wave groups one phase apart, the lazy reference maximum with the max-free fast path, the staged output.
-// What changes is the register geometry.  A wave still owns 32 query rows, now as two blocks of 16 (rb):
+// What changes is the register geometry.  A wave owns 32 query rows (16 at head dims above 128) as blocks of 16 (rb):
 //   * lane (m = lane & 15, g = lane >> 4) holds, for each rb, query row 16 rb + m;
 //   * S^T = K Q^T per 16-key block kb: A = K rows (lane: key m of the block, head dims 32 c + 8 g .. + 7, one
 //     ds_read_b128), B = the resident Q fragment (row m, same head dims); the lane receives keys 4 g .. 4 g + 3 of
-//     the block for its row.  One K fragment feeds both row blocks: LDS bytes per flop as before;
+//     the block for its row.  One K fragment feeds every row block of the wave;
 //   * O^T += V^T P^T per 32 keys: the lane's probabilities of two neighbouring key blocks, packed, are the B operand
 //     (k slots 0-3 <-> keys 4 g + j of the first block, 4-7 <-> the second), the A operand is V^T read by two
 //     transposing ds_read_b64_tr_b16 of the same keys; the lane accumulates head dims 16 db + 4 g .. + 3 of its row;
