@@ -95,6 +95,7 @@ struct BwdDqCfg {
     static constexpr int TILE_BYTES = BN * ROWB;
     static constexpr int LOADS = BN * CPR / kThreads;
     static constexpr int STAGE_BYTES = stage_tile_bytes<DB>();   // a wave's dQ rows on their way out
+    static constexpr int GRP = 4;      // tile operands are read this many matrix instructions ahead
     static constexpr int SMEM = 4 * TILE_BYTES > kWaves * STAGE_BYTES ? 4 * TILE_BYTES : kWaves * STAGE_BYTES;   // {K, V} x 2 stages
     static_assert(BN % 32 == 0 && D % 32 == 0 && (BN * CPR) % kThreads == 0, "tile shape");
     static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");
@@ -168,15 +169,14 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
     const int d_last_chunk = p.d / 8 - 1;
     const uint32_t lds0 = (uint32_t)(size_t)((FA_LDS_PTR(char))smem);
     const uint32_t fill0 = __builtin_amdgcn_readfirstlane((int)(lds0 + (uint32_t)(wave * C::LOADS * 1024)));
-    int f_row[C::LOADS], f_col[C::LOADS];
+    // fill j of this lane: row f_row(j), chunk f_col(j) of the tile (recomputed where the last tile needs them)
+    auto f_row = [&](int j) { return ((wave * C::LOADS + j) * 1024 + lane * 16) / C::ROWB; };
+    auto f_col = [&](int j) { return min(swz_u<D>((((wave * C::LOADS + j) * 1024 + lane * 16) % C::ROWB) / 16, f_row(j)), d_last_chunk); };
     uint32_t f_koff[C::LOADS], f_voff[C::LOADS];
 #pragma unroll
     for (int j = 0; j < C::LOADS; j++) {
-        const int pos = (wave * C::LOADS + j) * 1024 + lane * 16;
-        f_row[j] = pos / C::ROWB;
-        f_col[j] = min(swz_u<D>((pos % C::ROWB) / 16, f_row[j]), d_last_chunk);
-        f_koff[j] = (uint32_t)((f_row[j] * (int)p.k_row_stride + f_col[j] * 8) * 2);
-        f_voff[j] = (uint32_t)((f_row[j] * (int)p.v_row_stride + f_col[j] * 8) * 2);
+        f_koff[j] = (uint32_t)((f_row(j) * (int)p.k_row_stride + f_col(j) * 8) * 2);
+        f_voff[j] = (uint32_t)((f_row(j) * (int)p.v_row_stride + f_col(j) * 8) * 2);
     }
     auto load_tile = [&](int buf, int t) {
         const int n0 = t * BN;
@@ -193,9 +193,9 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
         } else {
 #pragma unroll
             for (int j = 0; j < C::LOADS; j++) {
-                const int r = min(f_row[j], si.sk - 1 - n0);
-                async_fill16(kt, (uint32_t)((r * (int)p.k_row_stride + f_col[j] * 8) * 2), dk_ + j * 1024);
-                async_fill16(vt, (uint32_t)((r * (int)p.v_row_stride + f_col[j] * 8) * 2), dv_ + j * 1024);
+                const int r = min(f_row(j), si.sk - 1 - n0);
+                async_fill16(kt, (uint32_t)((r * (int)p.k_row_stride + f_col(j) * 8) * 2), dk_ + j * 1024);
+                async_fill16(vt, (uint32_t)((r * (int)p.v_row_stride + f_col(j) * 8) * 2), dv_ + j * 1024);
             }
         }
     };
@@ -227,8 +227,8 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 #pragma unroll
             for (int nb = 0; nb < C::NB; nb++) {
                 f32x16 s_acc[1], dp_acc[1];
-                product_rows<T, D, 1, C::KS, 4>(s_acc, kb + nb * 32 * C::ROWB, lo.r, qf);
-                product_rows<T, D, 1, C::KS, 4>(dp_acc, vb + nb * 32 * C::ROWB, lo.r, gf);
+                product_rows<T, D, 1, C::KS, C::GRP>(s_acc, kb + nb * 32 * C::ROWB, lo.r, qf);
+                product_rows<T, D, 1, C::KS, C::GRP>(dp_acc, vb + nb * 32 * C::ROWB, lo.r, gf);
                 if (need_mask) mask_acc16(s_acc[0], n0 + nb * 32 + 4 * hh, lim_lo, lim_hi);
                 uint32_t keep[8];
                 if constexpr (DROPOUT) drop_pairs_row(drop, row, n0 + nb * 32, hh, keep);
@@ -243,7 +243,7 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
                 dsf[2 * nb + 1] = pack_acc8<T>(s_acc[0], 8);
             }
             // dQ^T += K^T dS^T
-            product_cols<T, D, C::PT, C::DB, 4>(dq_acc, kb, lo.c, dsf);
+            product_cols<T, D, C::PT, C::DB, C::GRP>(dq_acc, kb, lo.c, dsf);
         }
         wait_vmcnt<0>();       // this wave's fills of the next tile have landed; the barrier publishes them
         __syncthreads();
@@ -268,9 +268,10 @@ __global__ void __launch_bounds__(256, MINW) bwd_dq_kernel(const BwdKParams kp) 
 // t - 1 (P of that tile was published before the barrier that ended step t - 1), so no barrier is
 // added and its exp-free vector work overlaps its own products.  The Q ring therefore has three
 // stages (tile t + 1 arriving, t read by the P wave, t - 1 read transposed by the dS wave); dO has two.
-// With DPARTS = 2 (head dim 256) two workgroups share a key block and each accumulates half of the
-// head dimension of dK / dV (both form S and dP in full): the accumulators of all 256 columns would
-// not fit next to the resident K / V row in 256 registers.
+// With DPARTS = 2 (head dims 193-256, or 129-256 with dropout) two workgroups share a key block and each
+// accumulates half of the head dimension of dK / dV (both form S and dP in full): the accumulators of all
+// 256 columns do not fit next to the resident K / V row in 256 registers (128 + 64 + operand sets, offsets
+// and the score block: 55 registers spilled, twice the time).  Up to head dim 192 they do (96 + 48).
 // ------------------------------------------------------------------------------------------------
 template <typename T, int D, int BM, int DPARTS, int DV = D>
 struct BwdDkv3Cfg {
@@ -283,10 +284,11 @@ struct BwdDkv3Cfg {
     static constexpr int AUX_OFF = 5 * TILE_BYTES;                   // 3 stages x {lse (log2 units), D} x BM floats
     static constexpr int X_OFF = AUX_OFF + 3 * 2 * BM * 4;           // P hand-over: 2 buffers x 4 key blocks
     static constexpr int XBLK = BM * 32 * 2;                         // one key block's P tile, fp16
-    static constexpr int SMEM = X_OFF + 2 * 4 * XBLK;
+    static constexpr int RING_END = X_OFF + 2 * 4 * XBLK;
+    static constexpr int OUT_BYTES = kWaves * stage_tile_bytes<DB>();   // the gradient rows, staged over the ring after the loop
+    static constexpr int SMEM = RING_END > OUT_BYTES ? RING_END : OUT_BYTES;
     // the resident K / V rows come in through LDS where the idle ring stages and the hand-over hold them
     static constexpr bool STAGED_ROWS = 4 * 32 * ROWB <= 2 * TILE_BYTES && 4 * 32 * ROWB <= 2 * 4 * XBLK;
-    static_assert(kWaves * 32 * (DB * 64 + 16) <= SMEM, "gradient rows are staged in the ring");
     static_assert(BM % 32 == 0 && DV % (32 * DPARTS) == 0 && DV <= D && (BM * CPR) % kThreads == 0 && 2 * BM <= kThreads, "tile shape");
     static_assert(SMEM <= 160 * 1024, "LDS budget");
     static_assert(TILE_BYTES % (kWaves * 1024) == 0 && TILE_BYTES / (kWaves * 1024) == LOADS, "one fill = 1 KB per wave");

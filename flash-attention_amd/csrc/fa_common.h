@@ -327,25 +327,30 @@ template <typename T> FA_DEV typename Elem<T>::v8 pack_acc8(const f32x16& a, int
 }
 
 // Per-lane LDS offsets of both read patterns, computed once: the swizzle only involves row & 15, so a
-// block of 32 rows (row-wise) or 16 rows (transposed) further down is a compile-time byte offset.
+// block of 32 rows (row-wise) or 16 rows (transposed) further down is a compile-time byte offset; and it
+// only changes the low four bits of the chunk index, so 16 chunks (8 k-steps, 4 column blocks: 256 bytes)
+// further along a row is one too -- the tables hold the first 8 k-steps and 4 column blocks only.
+constexpr int kOffsKS = 8, kOffsDB = 4, kOffsPeriodBytes = 256;
 template <int D, int KS, int DB>
 struct LdsOffs {
-    int r[KS];       // row-wise: row l32, k-step dk
-    int c[DB][2];    // transposed: column block db, rows 4hh + tj and 8 more
+    int r[KS < kOffsKS ? KS : kOffsKS];       // row-wise: row l32, k-step dk
+    int c[DB < kOffsDB ? DB : kOffsDB][2];    // transposed: column block db, rows 4hh + tj and 8 more
     FA_DEV void init(int lane, int db0 = 0) {      // db0: first 32-column block of the DB blocks this wave reads
         const int l32 = lane & 31, hh = lane >> 5;
 #pragma unroll
-        for (int dk = 0; dk < KS; dk++) r[dk] = l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16;
+        for (int dk = 0; dk < (KS < kOffsKS ? KS : kOffsKS); dk++) r[dk] = l32 * (D * 2) + swz_u<D>(dk * 2 + hh, l32) * 16;
         const int tj = (lane & 15) >> 2, tq = lane & 3, dhalf = (lane >> 4) & 1;
         const int row = 4 * hh + tj;
 #pragma unroll
-        for (int db = 0; db < DB; db++) {
+        for (int db = 0; db < (DB < kOffsDB ? DB : kOffsDB); db++) {
             const int cc = (db0 + db) * 4 + dhalf * 2 + (tq >> 1);
             c[db][0] = row * (D * 2) + swz_u<D>(cc, row) * 16 + (tq & 1) * 8;
             c[db][1] = (row + 8) * (D * 2) + swz_u<D>(cc, row + 8) * 16 + (tq & 1) * 8;
         }
     }
 };
+FA_DEV int offs_row(const int* offr, int dk) { return offr[dk % kOffsKS] + (dk / kOffsKS) * kOffsPeriodBytes; }
+FA_DEV int offs_col(const int (*offc)[2], int db, int half) { return offc[db % kOffsDB][half] + (db / kOffsDB) * kOffsPeriodBytes; }
 template <typename T, int D> FA_DEV typename Elem<T>::v8 lds_rows_at(const char* tile, int off, int blk32) {
     const u32x4 raw = *reinterpret_cast<const u32x4*>(tile + off + blk32 * 32 * (D * 2));
     return __builtin_bit_cast(typename Elem<T>::v8, raw);
@@ -374,14 +379,14 @@ FA_DEV void product_rows(f32x16* acc, const char* tile, const int* offr, const t
     // step st -> (k-step st / NBLK, row block st % NBLK): consecutive MFMAs go to different accumulators
     v8 a[2][GRP];
 #pragma unroll
-    for (int j = 0; j < GRP; j++) a[0][j] = lds_rows_at<T, D>(tile, offr[j / NBLK], j % NBLK);
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_rows_at<T, D>(tile, offs_row(offr, j / NBLK), j % NBLK);
 #pragma unroll
     for (int g = 0; g < NG; g++) {
         if (g + 1 < NG) {
 #pragma unroll
             for (int j = 0; j < GRP; j++) {
                 const int st = (g + 1) * GRP + j;
-                a[(g + 1) & 1][j] = lds_rows_at<T, D>(tile, offr[st / NBLK], st % NBLK);
+                a[(g + 1) & 1][j] = lds_rows_at<T, D>(tile, offs_row(offr, st / NBLK), st % NBLK);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -401,14 +406,14 @@ FA_DEV void product_cols(f32x16* acc, const char* tile, const int (*offc)[2], co
     static_assert(TOTAL % GRP == 0, "group shape");
     v8 a[2][GRP];
 #pragma unroll
-    for (int j = 0; j < GRP; j++) a[0][j] = lds_cols_at<T, D>(tile, offc[j % DB][0], offc[j % DB][1], j / DB);
+    for (int j = 0; j < GRP; j++) a[0][j] = lds_cols_at<T, D>(tile, offs_col(offc, j % DB, 0), offs_col(offc, j % DB, 1), j / DB);
 #pragma unroll
     for (int g = 0; g < NG; g++) {
         if (g + 1 < NG) {
 #pragma unroll
             for (int j = 0; j < GRP; j++) {
                 const int st = (g + 1) * GRP + j;
-                a[(g + 1) & 1][j] = lds_cols_at<T, D>(tile, offc[st % DB][0], offc[st % DB][1], st / DB);
+                a[(g + 1) & 1][j] = lds_cols_at<T, D>(tile, offs_col(offc, st % DB, 0), offs_col(offc, st % DB, 1), st / DB);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
