@@ -121,7 +121,7 @@ def bench_head_dims(steps, warmup):
     import flash_attn
     b, s, h = 4, 8192, 32
     res = {}
-    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96,2>"), (192, "fa::prefill_pp16_kernel<bf16,256,32,192,1>")):
+    for d, kern in ((96, "fa::prefill_pp16_kernel<bf16,128,64,96,2>"), (192, "fa::prefill_pp16_kernel<bf16,256,32,192,2>")):
         torch.manual_seed(0)
         q, k, v = (torch.randn(b, s, h, d, device="cuda", dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
         with torch.no_grad():

@@ -7,7 +7,7 @@
 //
 // What stays: the work order, the tile ring (global_load_lds straight into LDS, 4 slots per tensor, 3 tiles ahead),
 // the two wave groups one phase apart, the lazy reference maximum with the max-free fast path, the staged output.
-// What changes is the register geometry.  A wave owns 32 query rows (16 at head dims above 128) as blocks of 16 (rb):
+// What changes is the register geometry.  A wave owns 32 query rows (16 at head dims above 192) as blocks of 16 (rb):
 //   * lane (m = lane & 15, g = lane >> 4) holds, for each rb, query row 16 rb + m;
 //   * S^T = K Q^T per 16-key block kb: A = K rows (lane: key m of the block, head dims 32 c + 8 g .. + 7, one
 //     ds_read_b128), B = the resident Q fragment (row m, same head dims); the lane receives keys 4 g .. 4 g + 3 of
@@ -32,9 +32,10 @@ FA_DEV void mask_acc4(f32x4& s, int pos0, int lo, int hi) {
     for (int r = 0; r < 4; r++) s[r] = (uint32_t)(z + r) > span ? -INFINITY : s[r];
 }
 
-// RB: 16-row blocks per wave (2: 256 rows per workgroup; 1: 128, the form for head dims 129-256, where 32 rows of output
-// and Q per wave leave no room for two waves per SIMD: there each fragment read from LDS feeds one matrix instruction
-// instead of two, and the kernel is bound by its fragment reads).
+// RB: 16-row blocks per wave (2: 256 rows per workgroup; 1: 128, the form for head dims 193-256, where 32 rows of output
+// and Q per wave do not fit the 256 registers of two waves per SIMD: there each fragment read from LDS feeds one matrix
+// instruction instead of two, and the kernel is bound by its fragment reads; also for launches of few or short row
+// blocks at head dims 129-192, see launch_prefill_pp_wide).
 template <typename T, int D, int BN, int DV = D, int RB = 2>
 __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) {
     typedef PPCfg<T, D, BN> C;
@@ -187,9 +188,12 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     auto active = [&](int i) -> bool { const int t = tile_of(i); return t >= ta_lo && t <= ta_hi; };
 
     // ---- S^T = K Q^T.  Fragment reads run LA fragments (2 LA matrix instructions) ahead of their use.
-    int kofs[KC];
+    // (the swizzles leave bit 4 of the chunk index alone: 16 chunks = 256 bytes further along a row is a compile-time
+    // offset, so the per-lane tables hold the first 4 k-steps and 8 output blocks)
+    constexpr int KCT = KC < 4 ? KC : 4, DBT = DB < 8 ? DB : 8;
+    int kofs[KCT];
 #pragma unroll
-    for (int c = 0; c < KC; c++) kofs[c] = m16 * C::ROWB + swz_k<D>(c * 4 + g4, m16) * 16;
+    for (int c = 0; c < KCT; c++) kofs[c] = m16 * C::ROWB + swz_k<D>(c * 4 + g4, m16) * 16;
     f32x4 s_acc[RB][KB];
     auto qk = [&](int i, auto slot_c) __attribute__((always_inline)) {
         // the ring slot of visit i is a compile-time constant (the key loop is unrolled by the ring depth), so slot and
@@ -197,7 +201,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         constexpr int slot = decltype(slot_c)::value * C::TILE;
         const char* kb[KC];
 #pragma unroll
-        for (int c = 0; c < KC; c++) kb[c] = smem + (slot + kofs[c]);
+        for (int c = 0; c < KC; c++) kb[c] = smem + (slot + (c / KCT) * 256 + kofs[c % KCT]);
         constexpr int NF = KC * KB;              // fragments in (c, kb) order: 2 KB matrix instructions between two
         constexpr int LA = FA_PP_LA;             // on the same accumulator
         auto frag_ptr = [&](int f) { return kb[f / KB] + (f % KB) * 16 * C::ROWB; };
@@ -223,9 +227,9 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
 
     // ---- O^T += V^T P^T, same interleave with two transposing reads per fragment
     const int tj = m16 >> 2, tq = m16 & 3;
-    int vofs[DB];
+    int vofs[DBT];
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+    for (int db = 0; db < DBT; db++)
         vofs[db] = C::NS * C::TILE + (4 * g4 + tj) * C::ROWB + swz_vd<D>(db * 2 + (tq >> 1), 4 * g4 + tj) * 16 + (tq & 1) * 8;
     v8 pf[RB][T32];
     auto pv = [&](int i, auto slot_c) __attribute__((always_inline)) {
@@ -233,7 +237,7 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
         constexpr int slot = decltype(slot_c)::value * C::TILE;
         const char* vb[DB];
 #pragma unroll
-        for (int db = 0; db < DB; db++) vb[db] = smem + (slot + vofs[db]);
+        for (int db = 0; db < DB; db++) vb[db] = smem + (slot + (db / DBT) * 256 + vofs[db % DBT]);
         constexpr int NF = T32 * DB;             // fragments in (t32, db) order
         constexpr int LA = FA_PP_LA;
         auto fetch = [&](int f) {
@@ -400,25 +404,33 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     // rows (16 B per lane).  All tile reads of the ring are behind the last barrier and each wave uses its own
     // region, so no barrier is needed.
     {
-        constexpr int PITCH = C::ROWB + 16;
-        char* stage = smem + wave * (WR * PITCH);
-#pragma unroll
-        for (int rb = 0; rb < RB; rb++)
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                const int d0 = db * 16 + 4 * g4;
-                const f32x4& o = o_acc[rb][db];
-                const u32x2 v = {pack2<T>(o[0] * inv[rb], o[1] * inv[rb]), pack2<T>(o[2] * inv[rb], o[3] * inv[rb])};
-                *reinterpret_cast<u32x2*>(stage + (16 * rb + m16) * PITCH + d0 * 2) = v;
-            }
+        constexpr int PITCH = DV * 2 + 16;             // the computed head dims of a row (reads past them are not stored)
+        // all of the wave's rows at once where 8 such regions fit the ring, else one 16-row block after the other
+        constexpr int SRB = C::kWaves * WR * PITCH <= C::SMEM ? RB : 1;      // row blocks per pass
+        static_assert(C::kWaves * 16 * SRB * PITCH <= C::SMEM, "the staged output fits the ring");
+        char* stage = smem + wave * (16 * SRB * PITCH);
         constexpr int RPP = 64 / C::CPR;                // rows per store instruction
         const int srow = lane / C::CPR, sch = lane % C::CPR;
         T* obase = reinterpret_cast<T*>(p.o) + si.o_off + (int64_t)head * p.o_head_stride + sch * 8;
 #pragma unroll
-        for (int j = 0; j < WR / RPP; j++) {
-            const int rr = j * RPP + srow;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
-            if (r0 + rr >= 0 && r0 + rr < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)(r0 + rr) * p.o_row_stride, v);
+        for (int pass = 0; pass < RB / SRB; pass++) {
+#pragma unroll
+            for (int sb = 0; sb < SRB; sb++) {
+                const int rb = pass * SRB + sb;
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    const int d0 = db * 16 + 4 * g4;
+                    const f32x4& o = o_acc[rb][db];
+                    const u32x2 v = {pack2<T>(o[0] * inv[rb], o[1] * inv[rb]), pack2<T>(o[2] * inv[rb], o[3] * inv[rb])};
+                    *reinterpret_cast<u32x2*>(stage + (16 * sb + m16) * PITCH + d0 * 2) = v;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 16 * SRB / RPP; j++) {
+                const int rr = j * RPP + srow, row = r0 + pass * 16 * SRB + rr;
+                const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rr * PITCH + sch * 16);
+                if (row >= 0 && row < si.sq && sch * 8 < p.d) st_global16(obase + (int64_t)row * p.o_row_stride, v);
+            }
         }
     }
 }
@@ -438,7 +450,7 @@ int launch_prefill_pp16_one(KParams kp, hipStream_t stream) {
     hipError_t e = FA_ALLOW_DYNAMIC_LDS(kern, C::SMEM);
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(kern, grid, block, C::SMEM, stream, kp);
-    return note_kernel((int)hipGetLastError(), D > 128 ? FA_KERNEL_PINGPONG_WIDE : FA_KERNEL_PINGPONG, false, false, DV);
+    return note_kernel((int)hipGetLastError(), D > 128 ? (RB == 2 ? FA_KERNEL_PINGPONG_WIDE32 : FA_KERNEL_PINGPONG_WIDE) : FA_KERNEL_PINGPONG, false, false, DV);
 }
 
 // Without dropout the 16x16x32 form; with dropout the 32x32x16 kernel of fa_prefill_pp.h, whose mask arithmetic
@@ -452,14 +464,25 @@ int launch_prefill_pp(const KParams& kp, hipStream_t stream) {
     return launch_prefill_pp16_one<T, D, BN>(kp, stream);
 }
 
-// Head dims 129..256 without dropout: 16 query rows per wave (one row block: 64 accumulator registers of output and 32
-// of Q at head dim 256), 128 rows per workgroup, 32-key tiles in the same four-slot rings; the reference's buckets
-// 160, 192, 224, 256 (csrc/flash_attn/src/flash_fwd_launch_template.h:236-336) leave out the k-steps and column
-// blocks past the bucket.
+// Head dims 129..256 without dropout: 32-key tiles in the same four-slot rings, 16 query rows per wave (one row
+// block: 64 accumulator registers of output and 32 of Q at head dim 256; 128 rows per workgroup) or 32 (up to head
+// dim 192; 256 rows per workgroup); the reference's buckets 160, 192, 224, 256
+// (csrc/flash_attn/src/flash_fwd_launch_template.h:236-336) leave out the k-steps and column blocks past the bucket.
 template <typename T>
 int launch_prefill_pp_wide(const KParams& kp, hipStream_t stream) {
-    if (kp.p.d <= 160) return launch_prefill_pp16_one<T, 256, 32, 160, 1>(kp, stream);
-    if (kp.p.d <= 192) return launch_prefill_pp16_one<T, 256, 32, 192, 1>(kp, stream);
+    // Up to head dim 192 a wave's registers hold 32 query rows (two row blocks: 96 registers of output, 48 of Q), and
+    // every K / V fragment read from LDS then feeds two matrix instructions: bf16 causal 8k at d 192 874 -> 1162
+    // TFLOP/s, full 914 -> 1304, d 160 789 -> 1097, 64 packed sequences of 128-4096 tokens 3.32 -> 2.55 ms.  At 224
+    // and 256 the same form spills 15 and 78 registers (+2 % and half the speed): those keep 16 rows per wave.
+    // The 128-row blocks stay where 256-row blocks would leave CUs idle: sequences of up to 128 queries (-4 %
+    // otherwise), launches of up to 128 blocks (64-128 blocks: 128-row blocks 27-38 % faster), and up to 256 under a
+    // mask when a sequence has several blocks of unequal length (one heavy block per CU: 10-18 % faster; with one
+    // block per sequence, 129-256 queries against 4096 keys, the 256-row form is 23-30 % ahead at 256 blocks).
+    const bool masked = kp.has_right || kp.has_left;
+    const int64_t wgs256 = (int64_t)((kp.p.seqlen_q + 255) / 256) * kp.p.h * kp.p.b;
+    const bool rows32 = kp.p.d <= 192 && kp.p.seqlen_q > 128 && wgs256 > (masked && kp.p.seqlen_q > 256 ? 256 : 128);
+    if (kp.p.d <= 160) return rows32 ? launch_prefill_pp16_one<T, 256, 32, 160, 2>(kp, stream) : launch_prefill_pp16_one<T, 256, 32, 160, 1>(kp, stream);
+    if (kp.p.d <= 192) return rows32 ? launch_prefill_pp16_one<T, 256, 32, 192, 2>(kp, stream) : launch_prefill_pp16_one<T, 256, 32, 192, 1>(kp, stream);
     if (kp.p.d <= 224) return launch_prefill_pp16_one<T, 256, 32, 224, 1>(kp, stream);
     return launch_prefill_pp16_one<T, 256, 32, 256, 1>(kp, stream);
 }

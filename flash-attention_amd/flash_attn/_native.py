@@ -711,7 +711,7 @@ def fwd_kvcache(q, kcache, vcache, k_, v_, seqlens_k_, rotary_cos_, rotary_sin_,
 
 # FA_KERNEL_* of include/fa_mi355x.h
 KERNEL_NAMES = {0: "none", 1: "tiled", 2: "tiled_tickets", 3: "pipelined", 4: "pingpong", 5: "wide", 6: "wide_pair",
-                7: "decode", 8: "decode_tickets", 9: "pingpong_wide"}
+                7: "decode", 8: "decode_tickets", 9: "pingpong_wide", 10: "pingpong_wide32"}
 
 
 def last_kernel():

@@ -222,6 +222,7 @@ int fa_set_rng_state(uint64_t *rng_state, uint64_t seed, uint64_t offset, void *
 #define FA_KERNEL_DECODE 7              /* up to 16 packed query rows, one workgroup per key chunk */
 #define FA_KERNEL_DECODE_TICKETS 8      /* the same under the ticket schedule */
 #define FA_KERNEL_PINGPONG_WIDE 9       /* 8-wave 128-row kernel, head dims 129-256 */
+#define FA_KERNEL_PINGPONG_WIDE32 10    /* the same with 32 query rows per wave (256-row blocks), head dims 129-192 */
 #define FA_KERNEL_FLAG_DROPOUT (1 << 8)
 #define FA_KERNEL_FLAG_SPLIT (1 << 9)
 int32_t fa_last_kernel(void);

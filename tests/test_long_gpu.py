@@ -6,7 +6,9 @@ library has it (csrc/fa_prefill_inst.hip), for an unsplit launch of 96+ query ro
     more than 256 (masked) / 128 (unmasked) row blocks of 256 rows in the launch, and no window whose two bounds
     span 768 keys or fewer;
   * software-pipelined kernel (fa_prefill_il.h): everything else up to head dim 128;
-  * head dim 129..256: the 8-wave kernel with 16 query rows per wave ("pingpong_wide"), pairs of waves with dropout.
+  * head dim 129..256: the 8-wave kernel with 16 query rows per wave ("pingpong_wide"), or, up to head dim 192 in a
+    launch of more than 128 blocks of 256 rows (256 under a mask when sequences span several blocks) with more
+    than 128 queries per sequence, with 32 rows per wave ("pingpong_wide32"); pairs of waves with dropout.
 
 Launches are made large enough for those thresholds with many query heads on few kv heads; the CPU oracle then checks
 a sample of (batch, head) pairs, which are independent problems.  Cases follow the reference's own test dimensions
@@ -159,8 +161,60 @@ def test_wide_kernel_head_dims_above_128(d, sq, sk, mode):
     window = _window(mode, sk, d * 31 + sq)
     out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=(mode == "causal"),
                                         window_size=window, return_attn_probs=True)
-    _ran("pingpong_wide", 160 if d <= 160 else 192 if d <= 192 else 224 if d <= 224 else 256)      # the reference's buckets above 128
+    blocks256 = (sq + 255) // 256 * h * b
+    rows32 = d <= 192 and blocks256 > (256 if mode != "full" else 128)       # (1500, 600, local) below head dim 193
+    _ran("pingpong_wide32" if rows32 else "pingpong_wide",
+         160 if d <= 160 else 192 if d <= 192 else 224 if d <= 224 else 256)      # the reference's buckets above 128
     _check(out, lse, q, k, v, causal=(mode == "causal"), window_size=window)
+
+
+# The 32-rows-per-wave form of the wide kernel (head dims 129-192): launches of more than 256 blocks of 256 rows under
+# a mask, more than 128 without.  (dtype, d, b, h, hk, sq, sk, causal, window)
+_WIDE32_CASES = {
+    "d192_causal": (torch.bfloat16, 192, 1, 32, 4, 2300, 2300, True, (-1, -1)),
+    "d192_causal_fp16": (torch.float16, 192, 2, 32, 8, 1300, 1300, True, (-1, -1)),
+    "d160_full_ragged": (torch.bfloat16, 160, 3, 16, 2, 777, 1111, False, (-1, -1)),
+    "d136_more_keys_causal": (torch.bfloat16, 136, 2, 32, 4, 1100, 2900, True, (-1, -1)),
+    "d176_fewer_keys_causal": (torch.bfloat16, 176, 2, 32, 4, 1500, 700, True, (-1, -1)),
+    "d192_two_sided_window": (torch.bfloat16, 192, 1, 48, 6, 1600, 1600, False, (1000, 300)),
+    "d160_rect_local_fp16": (torch.float16, 160, 2, 32, 2, 1200, 2600, False, (900, 0)),
+    "d192_narrow_window": (torch.bfloat16, 192, 2, 32, 4, 1400, 1400, False, (100, 60)),
+    "d144_one_block_per_sequence": (torch.bfloat16, 144, 24, 8, 2, 200, 1800, True, (-1, -1)),
+}
+
+
+@pytest.mark.parametrize("case", sorted(_WIDE32_CASES))
+def test_wide_kernel_with_32_rows_per_wave(case):
+    _say("wide, 32 rows per wave", case)
+    dtype, d, b, h, hk, sq, sk, causal, window = _WIDE32_CASES[case]
+    q = _gen((b, sq, h, d), dtype, 1); k = _gen((b, sk, hk, d), dtype, 2); v = _gen((b, sk, hk, d), dtype, 3)
+    out, lse, _ = _fa().flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal, window_size=window,
+                                        return_attn_probs=True)
+    _ran("pingpong_wide32", 160 if d <= 160 else 192)
+    assert not torch.isnan(out).any()
+    pairs = [(0, 0), (b - 1, h - 1), (b // 2, h // 2 + 1)]
+    _check_pairs(out, lse, q, k, v, pairs[:2] if dtype == torch.float16 else pairs, causal=causal, window_size=window)
+
+
+def test_wide_kernel_with_32_rows_per_wave_packed_sequences():
+    """Variable-length batch at head dim 192 with empty, one-row and ragged sequences: row blocks are aligned to the
+    end of each sequence, so the first block of most sequences starts before its first row."""
+    _say("wide, 32 rows per wave, varlen")
+    dtype, h, hk, d = torch.bfloat16, 16, 4, 192
+    lens = [0, 1, 255, 256, 257, 700, 0, 1300, 2100, 129, 513, 1999, 31, 1024]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    total, mx = int(cu[-1]), max(lens)
+    q = _gen((total, h, d), dtype, 1); k = _gen((total, hk, d), dtype, 2); v = _gen((total, hk, d), dtype, 3)
+    out, lse, _ = _fa().flash_attn_varlen_func(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), cu.to(DEV), mx, mx,
+                                               causal=True, return_attn_probs=True)
+    _ran("pingpong_wide32", 192)                # 9 blocks of 256 rows x 16 heads x 14 sequences
+    assert not torch.isnan(out).any()
+    for i, n in enumerate(lens):
+        if n == 0:
+            continue
+        a, e = int(cu[i]), int(cu[i + 1])
+        _check_pairs(out[a:e][None], lse[i:i + 1, :, :n], q[a:e][None], k[a:e][None], v[a:e][None], [(0, 0), (0, h - 1)],
+                     causal=True)
 
 
 @pytest.mark.parametrize("s,d", [(1024, 64), (2304, 128), (1024, 256)])

@@ -51,9 +51,10 @@ _SHAPES = {
     "pingpong": (128, 1, 32, 4, 4352, 4352),
     "pingpong96": (96, 1, 32, 4, 4352, 4352),
     "wide": (256, 4, 8, 2, 512, 1024),
+    "wide32": (192, 1, 32, 4, 2816, 2816),            # 11 x 32 blocks of 256 rows (9 x 32 with fewer queries than keys): the 32-rows-per-wave form
 }
 _KERNEL_OF = {"tiled": "tiled", "pipelined": "pipelined", "pipelined64": "pipelined", "pingpong": "pingpong",
-              "pingpong96": "pingpong", "wide": "pingpong_wide"}
+              "pingpong96": "pingpong", "wide": "pingpong_wide", "wide32": "pingpong_wide32"}
 _PATTERNS = ["rising", "falling", "spike_first", "spike_middle", "spike_last", "scale1", "x8"]
 
 
@@ -119,7 +120,7 @@ def _run_and_check(kernel, pattern, dtype, mode, rect=False):
 
 
 @pytest.mark.parametrize("pattern", _PATTERNS)
-@pytest.mark.parametrize("kernel", ["tiled", "pipelined", "pipelined64", "pingpong", "pingpong96", "wide"])
+@pytest.mark.parametrize("kernel", ["tiled", "pipelined", "pipelined64", "pingpong", "pingpong96", "wide", "wide32"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_adversarial_rows_causal(kernel, pattern, dtype):
     _say("softmax stress causal", kernel, pattern, dtype)
@@ -127,7 +128,7 @@ def test_adversarial_rows_causal(kernel, pattern, dtype):
 
 
 @pytest.mark.parametrize("pattern", ["rising", "falling", "spike_middle", "scale1"])
-@pytest.mark.parametrize("kernel", ["pipelined", "pingpong", "wide"])
+@pytest.mark.parametrize("kernel", ["pipelined", "pingpong", "wide", "wide32"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_adversarial_rows_dense(kernel, pattern, dtype):
     _say("softmax stress dense", kernel, pattern, dtype)
@@ -135,7 +136,7 @@ def test_adversarial_rows_dense(kernel, pattern, dtype):
 
 
 @pytest.mark.parametrize("pattern", ["rising", "falling", "spike_first", "spike_last", "x8", "dead_tiles"])
-@pytest.mark.parametrize("kernel", ["tiled", "pipelined", "pipelined64", "pingpong", "wide"])
+@pytest.mark.parametrize("kernel", ["tiled", "pipelined", "pipelined64", "pingpong", "wide", "wide32"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_adversarial_rows_under_a_window(kernel, pattern, dtype):
     """dead_tiles: seqlen_q < seqlen_k, so the window of the first rows starts far into the keys"""
