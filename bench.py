@@ -423,7 +423,7 @@ def bench_decode_variants(steps, warmup):
     res = {}
     for name, (b, cap, hk, h, d, sq, lo, kern) in (
             ("four_positions_gqa8", (64, 32768, 8, 64, 128, 4, 1024, "fa::prefill_persistent_kernel<bf16,128,stream>")),
-            ("one_position_mqa32", (16, 65536, 1, 32, 128, 1, 30000, "fa::prefill_persistent_kernel<bf16,128>"))):
+            ("one_position_mqa32", (16, 65536, 1, 32, 128, 1, 30000, "fa::prefill_persistent_kernel<bf16,128,stream>"))):
         torch.manual_seed(0)
         k_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)
         v_cache = torch.randn(b, cap, hk, d, device="cuda", dtype=torch.bfloat16)

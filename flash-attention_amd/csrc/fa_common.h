@@ -58,8 +58,10 @@ struct KParams {
     // dec_compact: the tickets cover only the slots that hold keys (the kernel counts them per batch entry
     // from the lengths); the merge then derives which slots were written from the lengths as well
     int32_t dec_persistent, dec_sa, dec_sb, dec_sub, dec_append, dec_compact;
-    // K and V together hold kStreamKvBytes or more (several times what the 256 MB memory-side cache keeps): the decode
-    // kernels, which read every row once, fetch them with non-temporal loads
+    // K and V together hold kStreamKvBytes or more (1.5 times what the 256 MB memory-side cache keeps): the decode
+    // kernels, which read every row once, fetch them with non-temporal loads.  Measured, one query position, bf16
+    // d 128, non-temporal against plain loads: 245 MB read per step -3..-6 %, 367-370 MB +10..+15 %, 414-491 MB
+    // +2..+15 %, 983 MB +1 %.
     int32_t stream_kv;
     // Few query positions with grouped q heads (pack_g > 1): the rows of the tiled kernel's problem are the
     // (position, grouped head) pairs of one kv head, row = position * pack_g + head within the group; p.h is
@@ -75,7 +77,7 @@ struct KParams {
     // batch index, (q head << 16) | row block.
     const int32_t* work_items;
 };
-constexpr int64_t kStreamKvBytes = (int64_t)1 << 30;
+constexpr int64_t kStreamKvBytes = (int64_t)3 << 27;
 constexpr int kDecCompactMaxBatch = 1024;    // batch entries whose slot counts the persistent decode kernel scans in LDS
 constexpr int kWorkListHeaderWords = 8;
 constexpr int kWorkListMaxBatch = 2048;      // sequences the list builder ranks (quadratic, in LDS)
