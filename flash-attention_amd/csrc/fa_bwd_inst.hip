@@ -23,7 +23,7 @@ typedef _Float16 InstT;
 #ifndef FA_BWD_BM
 #define FA_BWD_BM (FA_D == 64 ? 128 : 64)
 #endif
-// DV: head dims the products run over (head dims up to 96 on the 128 bucket, up to 192 on the 256 bucket)
+// DV: head dims the products run over (head dims up to 96 on the 128 bucket, up to 160 and up to 192 on the 256 bucket)
 template <bool DROPOUT, int DV = FA_D>
 static int run(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D <= 128
@@ -38,9 +38,16 @@ static int run(const BwdKParams& kp, hipStream_t stream) {
     if (key_blocks < 256 && kp.p.seqlen_q >= 1024) return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 2, DROPOUT>(kp, stream);
     return launch_bwd_dkv3<InstT, FA_D, FA_BWD_BM, 1, DROPOUT, DV>(kp, stream);
 #else
-    // one workgroup (4 waves of 512 registers) per CU; up to head dim 192 the registers also hold a 64-key step,
-    // which halves the barriers and tile requests per product (head dim 192, causal 8k: dQ pass 4.18 -> 3.2 ms)
-    if (int e = launch_bwd_dq<InstT, FA_D, (DV <= 192 ? 64 : 32), 1, DROPOUT, DV>(kp, stream)) return e;
+    // Up to head dim 160 the dQ pass fits 256 registers with 32-key steps: two workgroups per CU, as at head dim 128
+    // (d 160, bf16 causal 8k, 16 heads: backward 5.79 -> 5.07 ms against one workgroup with 64-key steps).  Beyond
+    // that one workgroup (4 waves of 512 registers) per CU -- two spill 76 registers at 192 --; up to head dim 192
+    // the registers also hold a 64-key step, which halves the barriers and tile requests per product (head dim 192,
+    // causal 8k: dQ pass 7.28 -> 5.95 ms); at 256 a 64-key step spills and gains nothing.
+    if constexpr (DV <= 160) {
+        if (int e = launch_bwd_dq<InstT, FA_D, 32, 2, DROPOUT, DV>(kp, stream)) return e;
+    } else {
+        if (int e = launch_bwd_dq<InstT, FA_D, (DV <= 192 ? 64 : 32), 1, DROPOUT, DV>(kp, stream)) return e;
+    }
     // Up to head dim 192 without dropout a wave holds its whole dK / dV accumulator (96 registers) next to its
     // resident key row; beyond that, or with the dropout mask words, two workgroups share a key block and each
     // accumulates half of the head dimension
@@ -53,6 +60,7 @@ int FA_INST_NAME(FA_D)(const BwdKParams& kp, hipStream_t stream) {
 #if FA_D == 128
     if (kp.p.d <= 96) return run<false, 96>(kp, stream);
 #elif FA_D == 256
+    if (kp.p.d <= 160) return run<false, 160>(kp, stream);
     if (kp.p.d <= 192) return run<false, 192>(kp, stream);
 #endif
     return run<false>(kp, stream);
