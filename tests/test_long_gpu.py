@@ -217,6 +217,38 @@ def test_wide_kernel_with_32_rows_per_wave_packed_sequences():
                      causal=True)
 
 
+def test_wide_kernel_with_32_rows_per_wave_chunked_prefill_on_a_cache():
+    """A 512-token chunk appended to K/V caches that hold different lengths (flash_attn_with_kvcache with new keys,
+    head dim 160, GQA): per-batch key lengths that are not prefix sums, more keys than queries, causal mask aligned
+    to the end of each cache entry."""
+    _say("wide, 32 rows per wave, kv cache")
+    from flash_attn import _native as nat
+    dtype, b, h, hk, d, sq, cap = torch.bfloat16, 8, 32, 4, 160, 512, 3000
+    q = _gen((b, sq, h, d), dtype, 1)
+    kc = _gen((b, cap, hk, d), dtype, 2); vc = _gen((b, cap, hk, d), dtype, 3)
+    kn = _gen((b, sq, hk, d), dtype, 4); vn = _gen((b, sq, hk, d), dtype, 5)
+    lens = torch.tensor([0, 1, 300, 1111, 2047, 2488, 64, 777], dtype=torch.int32)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out, lse = nat.fwd_kvcache(q.to(DEV), kd, vd, kn.to(DEV), vn.to(DEV), lens.to(DEV), None, None, None, None, d ** -0.5,
+                               True, -1, -1, True, 0)
+    _ran("pingpong_wide32", 160)                # 2 blocks of 256 rows x 32 heads x 8 entries
+    assert not torch.isnan(out).any()
+    out, lse = out.cpu(), lse.cpu()
+    for i in (0, 1, 3, 5):
+        sl = slice(i, i + 1)
+        for hh in (0, h - 1):
+            g = hh // (h // hk)
+            o_ref, l_ref, k_after, v_after = orc.kvcache_forward(q[sl, :, hh:hh + 1], kc[sl, :, g:g + 1], vc[sl, :, g:g + 1],
+                                                                 kn[sl, :, g:g + 1], vn[sl, :, g:g + 1], None, None, lens[sl], causal=True)
+            o_pt, _, _, _ = orc.kvcache_forward(q[sl, :, hh:hh + 1], kc[sl, :, g:g + 1], vc[sl, :, g:g + 1], kn[sl, :, g:g + 1],
+                                                vn[sl, :, g:g + 1], None, None, lens[sl], causal=True, upcast=False, reorder_ops=True)
+            ok, err, bound = orc.tolerance_ok(out[sl, :, hh:hh + 1], o_ref, o_pt, 2.0, 1e-5)
+            _say("   entry %d head %d: err %.3e bound %.3e" % (i, hh, err, bound))
+            assert ok
+            assert orc.lse_ok(lse[sl, hh:hh + 1], l_ref)[0]
+            assert torch.equal(kd[sl, :, g:g + 1].cpu(), k_after.to(dtype)) and torch.equal(vd[sl, :, g:g + 1].cpu(), v_after.to(dtype))
+
+
 @pytest.mark.parametrize("s,d", [(1024, 64), (2304, 128), (1024, 256)])
 def test_long_kernels_take_strided_packed_input(s, d):
     """q, k, v as strided views of one (b, s, 3, h, d) tensor: row stride 3*h*d."""
