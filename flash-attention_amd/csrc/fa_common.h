@@ -438,6 +438,14 @@ FA_DEV void async_fill16(const void* base_uniform, uint32_t lane_offset, uint32_
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_base_uniform), "v"(lane_offset), "s"(sbase) : "memory", "m0");
 }
+// A pointer that is uniform over the wave by construction, read through readfirstlane so that the compiler keeps it --
+// and whatever is stepped from it -- in scalar registers (it cannot always prove the uniformity of values derived
+// from the work item, and then spends a 64-bit vector add and two readfirstlanes on every tile request).
+template <typename P> FA_DEV const P* scalar_ptr(const P* ptr) {
+    const uint64_t a = (uint64_t)ptr;
+    return (const P*)((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a) |
+                      ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32)) << 32));
+}
 // wait until at most N of this wave's vector-memory operations are outstanding (N < 64: the counter's low four
 // bits sit in bits 3:0 of the operand, its upper two in bits 15:14)
 template <int N> FA_DEV void wait_vmcnt() {

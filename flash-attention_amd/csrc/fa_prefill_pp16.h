@@ -102,8 +102,8 @@ __global__ void __launch_bounds__(512, 2) prefill_pp16_kernel(const KParams kp) 
     const int64_t kstep = (int64_t)BN * p.k_row_stride, vstep = (int64_t)BN * p.v_row_stride;
     const int64_t kpass = (int64_t)C::ROWS_PER_PASS * p.k_row_stride, vpass = (int64_t)C::ROWS_PER_PASS * p.v_row_stride;
     const int t_first = t_hi - 1;
-    const T* ktile = kg + (int64_t)t_first * BN * p.k_row_stride;       // tile next to be requested
-    const T* vtile = vg + (int64_t)t_first * BN * p.v_row_stride;
+    const T* ktile = scalar_ptr(kg + (int64_t)t_first * BN * p.k_row_stride);       // tile next to be requested
+    const T* vtile = scalar_ptr(vg + (int64_t)t_first * BN * p.v_row_stride);
     const uint32_t koff = (uint32_t)(((int64_t)frow * p.k_row_stride + kch * 8) * 2);
     const uint32_t voff = (uint32_t)(((int64_t)frow * p.v_row_stride + vch * 8) * 2);
     // only key tile t_hi - 1 can reach past seqlen_k: its rows are clamped
