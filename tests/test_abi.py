@@ -35,6 +35,17 @@ def test_header_symbols_exported(lib):
         assert hasattr(lib, n), "library does not export %s" % n
 
 
+def test_kernel_ids_of_the_header_have_names():
+    """Every FA_KERNEL_* id that fa_last_kernel() can return is decoded by flash_attn._native.last_kernel()."""
+    import flash_attn._native as nat
+    text = open(HEADER).read()
+    ids = {name: int(val) for name, val in re.findall(r"#define\s+FA_KERNEL_((?!FLAG_)[A-Z0-9_]+)\s+(\d+)\b", text)}
+    assert ids["NONE"] == 0 and len(ids) >= 10 and len(set(ids.values())) == len(ids)
+    assert set(ids.values()) == set(nat.KERNEL_NAMES)
+    for name, val in ids.items():
+        assert nat.KERNEL_NAMES[val] == name.lower(), (name, val, nat.KERNEL_NAMES[val])
+
+
 def test_struct_mirror_size(lib):
     import flash_attn._native as nat
     lib.fa_sizeof_params.restype = ctypes.c_int32
